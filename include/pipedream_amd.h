@@ -1,0 +1,125 @@
+/*
+ * pipedream_amd.h -- C ABI of libpipedream_amd.so (gfx950 / MI355X).
+ *
+ * The reference (msr-fiddle/pipedream) has no FFI on its per-stage training
+ * step: the path is Python over torch.  Each entry point below therefore cites
+ * the reference Python routine whose device work it replaces (paths relative
+ * to the reference checkout).  The Python classes in pipedream_amd/ keep the
+ * reference's class API and call these functions through ctypes.
+ *
+ * Conventions
+ *   - every function returns 0 on success, a negative PD_E* code for an
+ *     argument/shape error detected on the host, or a positive hipError_t;
+ *     pd_last_error() returns a thread-local message for the last failure;
+ *   - all tensor pointers are DEVICE pointers owned by the caller and must stay
+ *     valid until `stream` has executed the launch; nothing here allocates
+ *     device memory unless the comment says so;
+ *   - `stream` is a hipStream_t passed as void* (NULL = the null stream);
+ *     launches are asynchronous;
+ *   - fp32 unless a name says otherwise; activations of the conv kernels are
+ *     NHWC ("channels last"), filters are KRSC (out-ch, kh, kw, in-ch).
+ */
+#ifndef PIPEDREAM_AMD_H
+#define PIPEDREAM_AMD_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define PD_OK 0
+#define PD_EINVAL (-1)   /* bad argument / null pointer / misaligned pointer   */
+#define PD_ESHAPE (-2)   /* shape not supported by the kernel                  */
+#define PD_ERANGE (-3)   /* index out of range (ring slot, queue index, ...)   */
+#define PD_ENOMEM (-4)   /* host allocation failed                             */
+
+#define PD_ABI_VERSION 1
+
+int pd_abi_version(void);
+const char* pd_last_error(void);
+
+/* ------------------------------------------------------------------------- *
+ * Weight-version ring.
+ * Replaces the deque of cloned state_dicts of OptimizerWithWeightStashing
+ * (runtime/optimizer.py:58-62 initialize_queue, :64-85 get_params, :87-116
+ * set_params/load_old_params/load_new_params, :156-159 rotation in step).
+ *
+ * The ring is host-side bookkeeping over ONE caller-allocated flat device
+ * buffer of n_versions slots, each slot_stride_bytes long (a multiple of 256).
+ * queue index 0 is the oldest entry, n_versions-1 the newest, exactly like the
+ * reference's deque(maxlen=num_versions).  All selection logic is integer-only
+ * and runs on the host, so which version a backward pass sees is bit-exact.
+ * ------------------------------------------------------------------------- */
+typedef struct pd_ring pd_ring;
+
+/* All n_versions entries start at version 0 (optimizer.py:58-62). */
+int pd_ring_create(void* base, uint64_t slot_stride_bytes, int n_versions, pd_ring** out);
+int pd_ring_destroy(pd_ring* ring);
+int pd_ring_num_versions(const pd_ring* ring);
+/* queue[queue_index] -> physical slot and the version it holds. */
+int pd_ring_entry(const pd_ring* ring, int queue_index, int* slot, int64_t* version);
+/* device address of a physical slot */
+int pd_ring_slot_ptr(const pd_ring* ring, int slot, void** dev_ptr);
+/* The physical slot the next push will overwrite (= queue[0]'s storage,
+ * optimizer.py:157 `buffered_state_dicts = self.queue[0][0]`). */
+int pd_ring_write_slot(const pd_ring* ring, int* slot);
+/* deque.append((oldest storage, version)): queue[0]'s slot becomes the newest
+ * entry holding `version` (optimizer.py:158).  Returns that slot. */
+int pd_ring_push(pd_ring* ring, int64_t version, int* slot);
+/* Copy slot `src` into every other slot: the nv clones of initialize_queue
+ * (optimizer.py:60-61).  128-bit coalesced copies. n_bytes <= slot stride. */
+int pd_ring_broadcast(const pd_ring* ring, int src_slot, uint64_t n_bytes, void* stream);
+
+/* Plain 128-bit coalesced device copy / fill (get_params' per-tensor copy_,
+ * optimizer.py:83; zero_grad, optimizer.py:118-120).  n_bytes multiple of 4. */
+int pd_copy(void* dst, const void* src, uint64_t n_bytes, void* stream);
+int pd_fill_zero(void* dst, uint64_t n_bytes, void* stream);
+
+/* ------------------------------------------------------------------------- *
+ * Fused optimizer step + stash.
+ * Replaces `p.grad.div_(update_interval)`, the loss-scale division,
+ * base_optimizer.step() and the get_params(clone=False) copy into the oldest
+ * ring slot (runtime/optimizer.py:137-159) with one pass that reads grad,
+ * param and state once and writes the new param into p_out (the ring's write
+ * slot; p_out may equal p_in) and the state in place.
+ *
+ * A launch covers a list of tensors; the flat-buffer case is one tensor.
+ * ------------------------------------------------------------------------- */
+typedef struct pd_tensor_desc {
+    const float* grad;    /* [n] gradient                                        */
+    const float* p_in;    /* [n] parameters to update (the loaded version)       */
+    float*       p_out;   /* [n] where the updated parameters go                 */
+    float*       state0;  /* [n] SGD momentum buffer / Adam exp_avg (may be NULL
+                             for SGD with momentum == 0)                         */
+    float*       state1;  /* [n] Adam exp_avg_sq (NULL for SGD)                  */
+    uint16_t*    bf16_out;/* [n] optional bf16 copy of p_out (NULL = none)       */
+    uint64_t     n;       /* elements                                            */
+} pd_tensor_desc;
+
+/* torch.optim.SGD maths (selected at runtime/sgd.py:17, run at optimizer.py:151):
+ *   g = grad / loss_scale / update_interval          (each only when != 1)
+ *   g += weight_decay * p                            (when weight_decay != 0)
+ *   buf = first_step ? g : momentum*buf + (1-dampening)*g   (when momentum != 0)
+ *   g = nesterov ? g + momentum*buf : buf
+ *   p_out = p_in - lr*g
+ * `descs` is a HOST array; it is copied into kernel arguments. */
+int pd_sgd_step(const pd_tensor_desc* descs, int n_tensors,
+                double lr, double momentum, double dampening, double weight_decay,
+                int nesterov, int first_step,
+                double loss_scale, double update_interval, void* stream);
+
+/* torch.optim.Adam maths (selected at runtime/adam.py:16):
+ * eps_mode 0 = installed-torch form  p -= (lr/bc1) * m / (sqrt(v)/sqrt(bc2) + eps)
+ * eps_mode 1 = PyTorch-1.1 form      p -= (lr*sqrt(bc2)/bc1) * m / (sqrt(v) + eps)
+ * `step` is the 1-based step count AFTER the increment. */
+int pd_adam_step(const pd_tensor_desc* descs, int n_tensors,
+                 double lr, double beta1, double beta2, double eps, double weight_decay,
+                 int64_t step, int eps_mode,
+                 double loss_scale, double update_interval, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* PIPEDREAM_AMD_H */

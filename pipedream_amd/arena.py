@@ -1,0 +1,223 @@
+"""Flat-buffer weight-version ring in HBM.
+
+One contiguous device buffer holds ``num_versions`` slots; every stashable state entry
+of the stage's modules (parameters and buffers) has a fixed byte offset inside a slot.
+The live module tensors are *views* into whichever slot is loaded, so
+``load_old_params`` / ``load_new_params`` are pointer swaps (``tensor.data = view``) and
+move no bytes.  Which slot holds which version is decided by the integer-only ring in
+the C library (``pd_ring_*``).
+
+Restates the storage side of ``OptimizerWithWeightStashing`` in the reference:
+runtime/optimizer.py:58-62 (``initialize_queue`` clones the state ``num_versions``
+times), :64-85 (``get_params``: ``running_*`` keys are never stashed, ``mask`` keys are
+not rolled back), :87-116 (``set_params`` / ``load_old_params`` / ``load_new_params``).
+"""
+import collections
+import ctypes
+
+import torch
+
+from . import _cabi
+
+ALIGN = 256  # bytes; every entry and every slot starts on a 256-byte boundary
+
+
+def _round_up(x, a):
+    return (x + a - 1) // a * a
+
+
+def _stashable(key):
+    # optimizer.py:76-78 and :93-94: running statistics accumulate normally and masks
+    # are taken from the live module, so neither is ever rolled back.
+    return "running_" not in key and "mask" not in key
+
+
+class Entry(object):
+    __slots__ = ("tensor", "keys", "offset", "nbytes", "numel", "dtype", "shape", "stride",
+                 "master_index", "views")
+
+    def __init__(self, tensor):
+        self.tensor = tensor
+        self.keys = []          # [(module index, state_dict key)]
+        self.offset = 0
+        self.numel = tensor.numel()
+        self.nbytes = tensor.numel() * tensor.element_size()
+        self.dtype = tensor.dtype
+        self.shape = tuple(tensor.shape)
+        self.stride = tuple(tensor.stride())
+        self.master_index = None
+        self.views = []         # one view per physical slot
+
+
+def _is_dense(t):
+    if t.is_contiguous():
+        return True
+    # dense, non-overlapping in some permutation (e.g. channels_last)
+    pairs = sorted((st, sz) for st, sz in zip(t.stride(), t.shape) if sz > 1)
+    expect = 1
+    for st, sz in pairs:
+        if st != expect:
+            return False
+        expect *= sz
+    return True
+
+
+class WeightArena(object):
+    """``num_versions`` flat slots + the integer ring that orders them."""
+
+    def __init__(self, modules, master_parameters, num_versions):
+        self._lib = _cabi.lib()
+        self.modules = list(modules)
+        self.num_versions = int(num_versions)
+        if self.num_versions < 1:
+            raise ValueError("num_versions must be >= 1")
+
+        masters = list(master_parameters)
+        if not masters:
+            raise ValueError("optimizer got an empty parameter list")
+        device = masters[0].device
+        _cabi.require_device(masters[0], "master parameter")
+
+        by_id = collections.OrderedDict()
+        # 1. master parameters first, in optimizer order: they form one fp32 section that
+        #    the fused step kernel walks.
+        for i, p in enumerate(masters):
+            if p.dtype != torch.float32:
+                raise TypeError("master parameters must be fp32, got %s" % p.dtype)
+            if p.device != device:
+                raise ValueError("all parameters of a stage must live on one device")
+            if id(p) in by_id:
+                raise ValueError("duplicate parameter in master_parameters")
+            e = Entry(p)
+            e.master_index = i
+            by_id[id(p)] = e
+        self.num_master = len(masters)
+
+        # 2. every other stashable state entry of the modules (buffers, frozen params).
+        for mi, module in enumerate(self.modules):
+            owners = dict(module.named_parameters(remove_duplicate=False))
+            owners.update(dict(module.named_buffers(remove_duplicate=False)))
+            for key in module.state_dict().keys():
+                t = owners.get(key)
+                if t is None or not _stashable(key):
+                    continue
+                if t.device != device:
+                    raise ValueError("state entry %r is on %s, expected %s" % (key, t.device, device))
+                e = by_id.get(id(t))
+                if e is None:
+                    e = Entry(t)
+                    by_id[id(t)] = e
+                e.keys.append((mi, key))
+        self.entries = list(by_id.values())
+
+        off = 0
+        for e in self.entries:
+            if not _is_dense(e.tensor):
+                # strided views cannot be re-homed; make the owner dense first
+                e.tensor.data = e.tensor.data.contiguous()
+                e.stride = tuple(e.tensor.stride())
+            e.offset = off
+            off = _round_up(off + e.nbytes, ALIGN)
+            if e.master_index == self.num_master - 1:
+                self.master_bytes = off
+        self.slot_bytes = max(off, ALIGN)
+        self.other_bytes = self.slot_bytes - self.master_bytes
+
+        self.buffer = torch.empty(self.num_versions * self.slot_bytes, dtype=torch.uint8, device=device)
+        if self.buffer.data_ptr() % ALIGN:
+            raise RuntimeError("allocator returned a buffer that is not %d-byte aligned" % ALIGN)
+        # padding between entries must stay finite: the fused step walks it too
+        self._lib.pd_fill_zero(ctypes.c_void_p(self.buffer.data_ptr()), self.buffer.numel(), _cabi.stream_ptr())
+
+        handle = ctypes.c_void_p()
+        self._lib.pd_ring_create(ctypes.c_void_p(self.buffer.data_ptr()), self.slot_bytes, self.num_versions,
+                                 ctypes.byref(handle))
+        self._ring = handle
+
+        for e in self.entries:
+            for s in range(self.num_versions):
+                lo = s * self.slot_bytes + e.offset
+                flat = self.buffer[lo:lo + e.nbytes].view(e.dtype)
+                if e.tensor.is_contiguous():
+                    v = flat.view(e.shape)
+                else:
+                    v = flat.as_strided(e.shape, e.stride)
+                e.views.append(v)
+
+        # initial state: newest entry (queue[-1]) holds the live values, then clone it
+        # into every other slot (optimizer.py:58-62).
+        self.live_slot = self.entry(-1)[0]
+        with torch.no_grad():
+            for e in self.entries:
+                e.views[self.live_slot].copy_(e.tensor.detach())
+        self._lib.pd_ring_broadcast(self._ring, self.live_slot, self.slot_bytes, _cabi.stream_ptr())
+        self._point_live_at(self.live_slot)
+
+    def __del__(self):
+        ring = getattr(self, "_ring", None)
+        if ring is not None and ring.value:
+            try:
+                self._lib.pd_ring_destroy(ring)
+            except Exception:
+                pass
+            self._ring = None
+
+    # -- ring bookkeeping (host integers) ------------------------------------------
+    def entry(self, queue_index):
+        """(physical slot, version) of ``queue[queue_index]``; index 0 is the oldest."""
+        slot = ctypes.c_int()
+        version = ctypes.c_int64()
+        self._lib.pd_ring_entry(self._ring, int(queue_index), ctypes.byref(slot), ctypes.byref(version))
+        return slot.value, version.value
+
+    def write_slot(self):
+        slot = ctypes.c_int()
+        self._lib.pd_ring_write_slot(self._ring, ctypes.byref(slot))
+        return slot.value
+
+    def push(self, version):
+        slot = ctypes.c_int()
+        self._lib.pd_ring_push(self._ring, int(version), ctypes.byref(slot))
+        return slot.value
+
+    def slot_ptr(self, slot):
+        return self.buffer.data_ptr() + slot * self.slot_bytes
+
+    # -- live pointers -------------------------------------------------------------
+    def _point_live_at(self, slot):
+        for e in self.entries:
+            e.tensor.data = e.views[slot]
+        self.live_slot = slot
+
+    def load_slot(self, slot):
+        """Make the module tensors views of ``slot`` (no bytes move)."""
+        if slot != self.live_slot:
+            self._point_live_at(slot)
+
+    def copy_other_section(self, src_slot, dst_slot, stream=None):
+        """Carry the non-optimised entries (buffers, frozen parameters) of ``src_slot``
+        into ``dst_slot``; the fused step only writes the master section."""
+        if self.other_bytes == 0 or src_slot == dst_slot:
+            return
+        self._lib.pd_copy(ctypes.c_void_p(self.slot_ptr(dst_slot) + self.master_bytes),
+                          ctypes.c_void_p(self.slot_ptr(src_slot) + self.master_bytes),
+                          self.other_bytes, _cabi.stream_ptr(stream))
+
+    def copy_slot(self, src_slot, dst_slot, stream=None):
+        if src_slot == dst_slot:
+            return
+        self._lib.pd_copy(ctypes.c_void_p(self.slot_ptr(dst_slot)), ctypes.c_void_p(self.slot_ptr(src_slot)),
+                          self.slot_bytes, _cabi.stream_ptr(stream))
+
+    def master_view(self, master_index, slot):
+        return self.entries[master_index].views[slot]
+
+    def state_dicts(self, slot):
+        """Per-module OrderedDicts of views into ``slot`` (the reference's stash format)."""
+        dicts = [collections.OrderedDict() for _ in self.modules]
+        for e in self.entries:
+            for (mi, key) in e.keys:
+                dicts[mi][key] = e.views[slot]
+        for d in dicts:
+            d._pd_slot = slot
+        return dicts

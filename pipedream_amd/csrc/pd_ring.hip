@@ -1,0 +1,201 @@
+// Weight-version ring bookkeeping (host integers only) and the 128-bit
+// streaming copy / fill kernels that initialise and maintain its slots.
+//
+// Reference behaviour restated: runtime/optimizer.py:58-62 (initialize_queue),
+// :110-116 (load_old/new pick queue[0] / queue[-1]), :156-159 (the oldest
+// entry's storage is overwritten and re-appended as the newest).
+#include <stdlib.h>
+#include <string.h>
+
+#include "pd_internal.h"
+
+static thread_local char g_err[512] = "";
+
+void pd_set_error(const char* fmt, ...) {
+    va_list ap;
+    va_start(ap, fmt);
+    vsnprintf(g_err, sizeof(g_err), fmt, ap);
+    va_end(ap);
+}
+
+extern "C" const char* pd_last_error(void) { return g_err; }
+extern "C" int pd_abi_version(void) { return PD_ABI_VERSION; }
+
+struct pd_ring {
+    char* base;
+    uint64_t stride;
+    int nv;
+    int head;          // physical slot of queue[0] (the oldest entry)
+    int64_t* version;  // version held by each PHYSICAL slot
+};
+
+extern "C" int pd_ring_create(void* base, uint64_t slot_stride_bytes, int n_versions, pd_ring** out) {
+    PD_REQUIRE(out != nullptr, PD_EINVAL, "pd_ring_create: out is NULL");
+    *out = nullptr;
+    PD_REQUIRE(base != nullptr, PD_EINVAL, "pd_ring_create: base is NULL");
+    PD_REQUIRE(n_versions >= 1, PD_EINVAL, "pd_ring_create: n_versions=%d < 1", n_versions);
+    PD_REQUIRE(pd_aligned(base, 256), PD_EINVAL, "pd_ring_create: base not 256-byte aligned");
+    PD_REQUIRE(slot_stride_bytes > 0 && slot_stride_bytes % 256 == 0, PD_EINVAL,
+               "pd_ring_create: slot stride %llu is not a positive multiple of 256",
+               (unsigned long long)slot_stride_bytes);
+    pd_ring* r = (pd_ring*)calloc(1, sizeof(pd_ring));
+    PD_REQUIRE(r != nullptr, PD_ENOMEM, "pd_ring_create: out of host memory");
+    r->version = (int64_t*)calloc((size_t)n_versions, sizeof(int64_t));
+    if (!r->version) {
+        free(r);
+        PD_FAIL(PD_ENOMEM, "pd_ring_create: out of host memory");
+    }
+    r->base = (char*)base;
+    r->stride = slot_stride_bytes;
+    r->nv = n_versions;
+    r->head = 0;
+    *out = r;
+    return PD_OK;
+}
+
+extern "C" int pd_ring_destroy(pd_ring* ring) {
+    if (ring) {
+        free(ring->version);
+        free(ring);
+    }
+    return PD_OK;
+}
+
+extern "C" int pd_ring_num_versions(const pd_ring* ring) { return ring ? ring->nv : PD_EINVAL; }
+
+extern "C" int pd_ring_entry(const pd_ring* ring, int queue_index, int* slot, int64_t* version) {
+    PD_REQUIRE(ring != nullptr, PD_EINVAL, "pd_ring_entry: ring is NULL");
+    // Python-style negative indices, as in queue[-1].
+    if (queue_index < 0) queue_index += ring->nv;
+    PD_REQUIRE(queue_index >= 0 && queue_index < ring->nv, PD_ERANGE,
+               "pd_ring_entry: queue index out of range for %d versions", ring->nv);
+    int s = (ring->head + queue_index) % ring->nv;
+    if (slot) *slot = s;
+    if (version) *version = ring->version[s];
+    return PD_OK;
+}
+
+extern "C" int pd_ring_slot_ptr(const pd_ring* ring, int slot, void** dev_ptr) {
+    PD_REQUIRE(ring != nullptr && dev_ptr != nullptr, PD_EINVAL, "pd_ring_slot_ptr: NULL argument");
+    PD_REQUIRE(slot >= 0 && slot < ring->nv, PD_ERANGE, "pd_ring_slot_ptr: slot %d out of range", slot);
+    *dev_ptr = ring->base + (uint64_t)slot * ring->stride;
+    return PD_OK;
+}
+
+extern "C" int pd_ring_write_slot(const pd_ring* ring, int* slot) {
+    PD_REQUIRE(ring != nullptr && slot != nullptr, PD_EINVAL, "pd_ring_write_slot: NULL argument");
+    *slot = ring->head;
+    return PD_OK;
+}
+
+extern "C" int pd_ring_push(pd_ring* ring, int64_t version, int* slot) {
+    PD_REQUIRE(ring != nullptr, PD_EINVAL, "pd_ring_push: ring is NULL");
+    int s = ring->head;
+    ring->version[s] = version;
+    ring->head = (ring->head + 1) % ring->nv;  // old queue[1] is now the oldest
+    if (slot) *slot = s;
+    return PD_OK;
+}
+
+// ---------------------------------------------------------------------------
+// Streaming copy / fill.  Each thread moves UNROLL 16-byte vectors that are one
+// block-width apart, so every wave issues fully coalesced 1 KiB requests.
+// ---------------------------------------------------------------------------
+typedef float float4_t __attribute__((ext_vector_type(4)));
+
+constexpr int COPY_THREADS = 256;
+constexpr int COPY_UNROLL = 8;
+
+__global__ __launch_bounds__(COPY_THREADS) void pd_copy_kernel(float4_t* __restrict__ dst,
+                                                               const float4_t* __restrict__ src,
+                                                               uint64_t n_vec) {
+    uint64_t base = (uint64_t)blockIdx.x * (COPY_THREADS * COPY_UNROLL) + threadIdx.x;
+    float4_t v[COPY_UNROLL];
+#pragma unroll
+    for (int u = 0; u < COPY_UNROLL; ++u) {
+        uint64_t i = base + (uint64_t)u * COPY_THREADS;
+        if (i < n_vec) v[u] = __builtin_nontemporal_load(src + i);
+    }
+#pragma unroll
+    for (int u = 0; u < COPY_UNROLL; ++u) {
+        uint64_t i = base + (uint64_t)u * COPY_THREADS;
+        if (i < n_vec) __builtin_nontemporal_store(v[u], dst + i);
+    }
+}
+
+__global__ void pd_copy_tail_kernel(float* dst, const float* src, uint64_t start, uint64_t n) {
+    uint64_t i = start + blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < n) dst[i] = src[i];
+}
+
+__global__ __launch_bounds__(COPY_THREADS) void pd_fill_zero_kernel(float4_t* __restrict__ dst, uint64_t n_vec) {
+    uint64_t base = (uint64_t)blockIdx.x * (COPY_THREADS * COPY_UNROLL) + threadIdx.x;
+    float4_t z = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int u = 0; u < COPY_UNROLL; ++u) {
+        uint64_t i = base + (uint64_t)u * COPY_THREADS;
+        if (i < n_vec) dst[i] = z;
+    }
+}
+
+__global__ void pd_fill_zero_tail_kernel(float* dst, uint64_t start, uint64_t n) {
+    uint64_t i = start + blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < n) dst[i] = 0.f;
+}
+
+extern "C" int pd_copy(void* dst, const void* src, uint64_t n_bytes, void* stream) {
+    if (n_bytes == 0) return PD_OK;
+    PD_REQUIRE(dst && src, PD_EINVAL, "pd_copy: NULL pointer");
+    PD_REQUIRE(n_bytes % 4 == 0, PD_EINVAL, "pd_copy: size not a multiple of 4 bytes");
+    PD_REQUIRE(pd_aligned(dst, 16) && pd_aligned(src, 16), PD_EINVAL, "pd_copy: pointers must be 16-byte aligned");
+    hipStream_t s = (hipStream_t)stream;
+    uint64_t n_vec = n_bytes / 16;
+    if (n_vec) {
+        uint64_t per_block = (uint64_t)COPY_THREADS * COPY_UNROLL;
+        uint64_t blocks = (n_vec + per_block - 1) / per_block;
+        PD_REQUIRE(blocks <= 0x7fffffffu, PD_ESHAPE, "pd_copy: buffer too large for one launch");
+        pd_copy_kernel<<<dim3((unsigned)blocks), dim3(COPY_THREADS), 0, s>>>((float4_t*)dst, (const float4_t*)src, n_vec);
+        PD_CHECK_LAUNCH("pd_copy_kernel");
+    }
+    uint64_t n = n_bytes / 4, done = n_vec * 4;
+    if (done < n) {
+        pd_copy_tail_kernel<<<dim3(1), dim3(64), 0, s>>>((float*)dst, (const float*)src, done, n);
+        PD_CHECK_LAUNCH("pd_copy_tail_kernel");
+    }
+    return PD_OK;
+}
+
+extern "C" int pd_fill_zero(void* dst, uint64_t n_bytes, void* stream) {
+    if (n_bytes == 0) return PD_OK;
+    PD_REQUIRE(dst, PD_EINVAL, "pd_fill_zero: NULL pointer");
+    PD_REQUIRE(n_bytes % 4 == 0, PD_EINVAL, "pd_fill_zero: size not a multiple of 4 bytes");
+    PD_REQUIRE(pd_aligned(dst, 16), PD_EINVAL, "pd_fill_zero: pointer must be 16-byte aligned");
+    hipStream_t s = (hipStream_t)stream;
+    uint64_t n_vec = n_bytes / 16;
+    if (n_vec) {
+        uint64_t per_block = (uint64_t)COPY_THREADS * COPY_UNROLL;
+        uint64_t blocks = (n_vec + per_block - 1) / per_block;
+        PD_REQUIRE(blocks <= 0x7fffffffu, PD_ESHAPE, "pd_fill_zero: buffer too large for one launch");
+        pd_fill_zero_kernel<<<dim3((unsigned)blocks), dim3(COPY_THREADS), 0, s>>>((float4_t*)dst, n_vec);
+        PD_CHECK_LAUNCH("pd_fill_zero_kernel");
+    }
+    uint64_t n = n_bytes / 4, done = n_vec * 4;
+    if (done < n) {
+        pd_fill_zero_tail_kernel<<<dim3(1), dim3(64), 0, s>>>((float*)dst, done, n);
+        PD_CHECK_LAUNCH("pd_fill_zero_tail_kernel");
+    }
+    return PD_OK;
+}
+
+extern "C" int pd_ring_broadcast(const pd_ring* ring, int src_slot, uint64_t n_bytes, void* stream) {
+    PD_REQUIRE(ring != nullptr, PD_EINVAL, "pd_ring_broadcast: ring is NULL");
+    PD_REQUIRE(src_slot >= 0 && src_slot < ring->nv, PD_ERANGE, "pd_ring_broadcast: slot %d out of range", src_slot);
+    PD_REQUIRE(n_bytes <= ring->stride, PD_ERANGE, "pd_ring_broadcast: n_bytes exceeds the slot stride");
+    const char* src = ring->base + (uint64_t)src_slot * ring->stride;
+    for (int s = 0; s < ring->nv; ++s) {
+        if (s == src_slot) continue;
+        int rc = pd_copy(ring->base + (uint64_t)s * ring->stride, src, n_bytes, stream);
+        if (rc != PD_OK) return rc;
+    }
+    return PD_OK;
+}

@@ -1,0 +1,58 @@
+"""The C-ABI library loads without a GPU and exports exactly what include/*.h declares."""
+import ctypes
+import os
+import re
+import subprocess
+
+import pytest
+
+from pipedream_amd import _cabi
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+HEADER = os.path.join(ROOT, "include", "pipedream_amd.h")
+
+
+def _declared():
+    text = open(HEADER).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    text = re.sub(r"//[^\n]*", "", text)
+    return sorted(set(re.findall(r"\b(pd_[a-z0-9_]+)\s*\(", text)))
+
+
+def test_header_and_binding_agree():
+    assert _declared() == sorted(_cabi.SIGNATURES)
+
+
+def test_library_exports_every_declared_symbol():
+    dll = ctypes.CDLL(_cabi.LIB_PATH)
+    for name in _declared():
+        assert hasattr(dll, name), "libpipedream_amd.so does not export %s" % name
+
+
+def test_no_undeclared_exports():
+    out = subprocess.run(["nm", "-D", "--defined-only", _cabi.LIB_PATH], capture_output=True, text=True).stdout
+    exported = set(re.findall(r"\bT (pd_[a-z0-9_]+)$", out, flags=re.M))
+    assert exported - {"pd_set_error"} <= set(_declared()), exported - set(_declared())
+
+
+def test_abi_version_and_error_string():
+    lib = _cabi.lib()
+    assert lib.pd_abi_version() == 1
+    with pytest.raises(_cabi.PipedreamAmdError) as ei:
+        lib.pd_copy(None, None, 16, None)
+    assert "NULL" in str(ei.value)
+    # argument validation happens on the host before any launch
+    with pytest.raises(_cabi.PipedreamAmdError):
+        lib.pd_copy(ctypes.c_void_p(4096), ctypes.c_void_p(8192), 6, None)
+    with pytest.raises(_cabi.PipedreamAmdError):
+        lib.pd_adam_step(None, 1, 1e-3, 0.9, 0.999, 1e-8, 0.0, 0, 0, 1.0, 1.0, None)
+
+
+def test_product_refuses_cpu_tensors():
+    import torch
+    from pipedream_amd import sgd
+    if torch.cuda.is_available():
+        pytest.skip("host-only check")
+    model = torch.nn.Linear(4, 4)
+    with pytest.raises(RuntimeError, match="no CPU fallback"):
+        sgd.SGDWithWeightStashing([model], list(model.parameters()), None, 1.0, 2, lr=0.1)

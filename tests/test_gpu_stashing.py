@@ -1,0 +1,164 @@
+"""Weight stashing through the reference's class API on the GPU.
+
+* the reference's own known-answer test (runtime/tests/backprop/sgd_with_stashing.py),
+  with its constructor call brought up to the current signature of runtime/sgd.py:12-15;
+* N-step 1F1B runs of SGD/AdamWithWeightStashing against the CPU oracle's restatement of
+  the reference classes on identical seeded inputs: version selection bit-exact,
+  parameters within rel 1e-5."""
+import copy
+
+import pytest
+import torch
+
+from oracle import stash_oracle as so
+from pipedream_amd import adam, optimizer, sgd
+
+pytestmark = pytest.mark.gpu
+
+
+def _reference_known_answer(num_versions, assertion_ground_truth):
+    N, D_in, D_H, D_out = 4, 4, 4, 4
+    x1 = torch.randn(N, D_in).cuda().requires_grad_(True)
+    y1 = torch.randn(N, D_out).cuda()
+    x2 = x1.clone().detach().requires_grad_(True)
+    x3 = x1.clone().detach().requires_grad_(True)
+    model = torch.nn.Sequential(torch.nn.Linear(D_in, D_H), torch.nn.ReLU(), torch.nn.Linear(D_H, D_out)).cuda()
+    loss_fn = torch.nn.MSELoss()
+    opt = sgd.SGDWithWeightStashing([model], model.parameters(), None, 1.0, num_versions=num_versions, lr=1e-1)
+    inputs = [x1, x2, x3]
+    preds = [model(x) for x in inputs]
+    assert torch.equal(preds[0], preds[1]) and torch.equal(preds[0], preds[2])
+    losses = [loss_fn(p, y1) for p in preds]
+    x_grads = []
+    for loss, x in zip(losses, inputs):
+        opt.zero_grad()
+        opt.load_old_params()
+        loss.backward()
+        x_grads.append(x.grad.clone().detach())
+        opt.load_new_params()
+        opt.step()
+    assert torch.equal(x_grads[0], x_grads[1]) == assertion_ground_truth[0]
+    assert torch.equal(x_grads[0], x_grads[2]) == assertion_ground_truth[1]
+    assert not torch.equal(preds[0], model(x1))
+
+
+def test_reference_known_answer():
+    torch.manual_seed(0)
+    _reference_known_answer(1, [False, False])
+    _reference_known_answer(2, [True, False])
+    _reference_known_answer(3, [True, True])
+
+
+def _mlp(seed):
+    torch.manual_seed(seed)
+    return torch.nn.Sequential(torch.nn.Linear(12, 16), torch.nn.Tanh(), torch.nn.Linear(16, 5))
+
+
+@pytest.mark.parametrize("kind,warmup", [("SGD", 0), ("SGD", 1), ("SGD", 3), ("Adam", 2)])
+def test_1f1b_matches_oracle(kind, warmup):
+    nv = warmup + 1
+    n = 12
+    cpu_model = _mlp(0)
+    gpu_model = copy.deepcopy(cpu_model).cuda()
+    if kind == "SGD":
+        kw = dict(lr=0.05, momentum=0.9, weight_decay=1e-4)
+        opt = sgd.SGDWithWeightStashing([gpu_model], gpu_model.parameters(), None, 1.0, nv, **kw)
+    else:
+        kw = dict(lr=1e-2, betas=(0.9, 0.999))
+        opt = adam.AdamWithWeightStashing([gpu_model], gpu_model.parameters(), None, 1.0, nv, **kw)
+    ora = so.StashingOptimizerOracle(kind, [cpu_model], cpu_model.parameters(), nv, **kw)
+    g = torch.Generator().manual_seed(1)
+    xs = [torch.randn(7, 12, generator=g) for _ in range(n)]
+    ys = [torch.randn(7, 5, generator=g) for _ in range(n)]
+    inflight_cpu, inflight_gpu = [], []
+    fwd_v, bwd_v = {}, {}
+    for kind_ev, k in so.one_f_one_b(n, warmup):
+        if kind_ev == "F":
+            fwd_v[k] = opt.current_version.version if nv > 1 else opt.latest_version.version
+            assert fwd_v[k] == so.forward_version(k, warmup)
+            inflight_cpu.append(torch.nn.functional.mse_loss(cpu_model(xs[k]), ys[k]))
+            inflight_gpu.append(torch.nn.functional.mse_loss(gpu_model(xs[k].cuda()), ys[k].cuda()))
+        else:
+            lc, lg = inflight_cpu.pop(0), inflight_gpu.pop(0)
+            torch.testing.assert_close(lg.cpu(), lc, rtol=1e-5, atol=1e-6)
+            for o in (ora, opt):
+                o.zero_grad()
+                o.load_old_params()
+            # bit-exact version selection
+            if nv > 1:
+                assert opt.current_version.version == ora.current_version == so.backward_version(k, warmup)
+            lc.backward()
+            lg.backward()
+            for o in (ora, opt):
+                o.load_new_params()
+                o.step()
+            assert opt.queue.versions() == ora.versions()
+            assert opt.latest_version.version == ora.latest_version
+    for pc, pg in zip(cpu_model.parameters(), gpu_model.parameters()):
+        torch.testing.assert_close(pg.cpu(), pc, rtol=1e-5, atol=1e-6)
+
+
+def test_lr_is_a_runtime_scalar_and_attribute_relay():
+    model = _mlp(0).cuda()
+    opt = sgd.SGDWithWeightStashing([model], model.parameters(), None, 1.0, 2, lr=0.1, momentum=0.9)
+    assert opt.param_groups[0]["lr"] == 0.1          # relayed to the base optimizer
+    for g in opt.param_groups:
+        g["lr"] = 0.0                                 # written every iteration by the caller
+    before = [p.detach().clone() for p in model.parameters()]
+    model(torch.randn(3, 12).cuda()).sum().backward()
+    opt.load_new_params()
+    opt.step()
+    for b, p in zip(before, model.parameters()):
+        assert torch.equal(b, p)
+    sd = opt.state_dict()
+    assert sd["param_groups"][0]["momentum"] == 0.9 and len(sd["state"]) == 4
+    assert "momentum_buffer" in sd["state"][0]
+
+
+def test_running_stats_are_not_rolled_back_and_buffers_are_stashed():
+    torch.manual_seed(0)
+    model = torch.nn.Sequential(torch.nn.Linear(4, 4), torch.nn.BatchNorm1d(4)).cuda()
+    opt = sgd.SGDWithWeightStashing([model], model.parameters(), None, 1.0, 2, lr=0.1)
+    keys = set(opt.queue[0][0][0].keys())
+    assert keys == {"0.weight", "0.bias", "1.weight", "1.bias", "1.num_batches_tracked"}
+    model(torch.randn(8, 4).cuda()).sum().backward()
+    rm = model[1].running_mean.clone()
+    opt.load_old_params()
+    assert torch.equal(model[1].running_mean, rm)
+    opt.load_new_params()
+    opt.step()
+    assert int(model[1].num_batches_tracked) == 1     # carried into the new slot
+    opt.load_old_params()
+    assert torch.equal(model[1].running_mean, rm)
+    assert int(model[1].num_batches_tracked) == 0     # stashed entry, like the reference
+
+
+def test_macrobatch_matches_oracle():
+    cpu_model = _mlp(3)
+    gpu_model = copy.deepcopy(cpu_model).cuda()
+    opt = sgd.SGDWithWeightStashing([gpu_model], gpu_model.parameters(), None, 1.0, 4, lr=0.1, momentum=0.9,
+                                    macrobatch=True)
+    ora = so.StashingOptimizerOracle("SGD", [cpu_model], cpu_model.parameters(), 4, macrobatch=True, lr=0.1,
+                                     momentum=0.9)
+    assert opt.num_versions == 2 and opt.update_interval == 2
+    g = torch.Generator().manual_seed(5)
+    for i in range(6):
+        x = torch.randn(5, 12, generator=g)
+        for o, m, xx in ((ora, cpu_model, x), (opt, gpu_model, x.cuda())):
+            o.zero_grad()
+            loss = m(xx).pow(2).mean()
+            o.load_old_params()
+            loss.backward()
+            o.load_new_params()
+            o.step()
+        assert opt.queue.versions() == ora.versions()
+    for pc, pg in zip(cpu_model.parameters(), gpu_model.parameters()):
+        torch.testing.assert_close(pg.cpu(), pc, rtol=1e-5, atol=1e-6)
+
+
+def test_unknown_optimizer_and_fp16_lists_fail_loudly():
+    model = _mlp(0).cuda()
+    with pytest.raises(NotImplementedError):
+        optimizer.OptimizerWithWeightStashing("RMSprop", [model], model.parameters(), None, 1.0, 2, lr=0.1)
+    with pytest.raises(NotImplementedError):
+        sgd.SGDWithWeightStashing([model], model.parameters(), list(model.parameters()), 1.0, 2, lr=0.1)
