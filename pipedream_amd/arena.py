@@ -134,15 +134,23 @@ class WeightArena(object):
                                  ctypes.byref(handle))
         self._ring = handle
 
+        # Entries the optimizer does not own (buffers such as num_batches_tracked, frozen
+        # parameters) keep the reference's copy semantics: the live module holds its own
+        # copy, so what a forward pass writes into it does not leak into a stashed version.
+        # They live together in one flat "live" block so a load/store is a single copy.
+        self.live_other = torch.empty(max(self.other_bytes, ALIGN), dtype=torch.uint8, device=device)
+
+        def _view(buf, lo, e):
+            flat = buf[lo:lo + e.nbytes].view(e.dtype)
+            if e.tensor.is_contiguous():
+                return flat.view(e.shape)
+            return flat.as_strided(e.shape, e.stride)
+
         for e in self.entries:
             for s in range(self.num_versions):
-                lo = s * self.slot_bytes + e.offset
-                flat = self.buffer[lo:lo + e.nbytes].view(e.dtype)
-                if e.tensor.is_contiguous():
-                    v = flat.view(e.shape)
-                else:
-                    v = flat.as_strided(e.shape, e.stride)
-                e.views.append(v)
+                e.views.append(_view(self.buffer, s * self.slot_bytes + e.offset, e))
+        self.masters = self.entries[:self.num_master]
+        self.others = self.entries[self.num_master:]
 
         # initial state: newest entry (queue[-1]) holds the live values, then clone it
         # into every other slot (optimizer.py:58-62).
@@ -150,6 +158,10 @@ class WeightArena(object):
         with torch.no_grad():
             for e in self.entries:
                 e.views[self.live_slot].copy_(e.tensor.detach())
+            for e in self.others:
+                live = _view(self.live_other, e.offset - self.master_bytes, e)
+                live.copy_(e.tensor.detach())
+                e.tensor.data = live
         self._lib.pd_ring_broadcast(self._ring, self.live_slot, self.slot_bytes, _cabi.stream_ptr())
         self._point_live_at(self.live_slot)
 
@@ -185,29 +197,33 @@ class WeightArena(object):
 
     # -- live pointers -------------------------------------------------------------
     def _point_live_at(self, slot):
-        for e in self.entries:
+        for e in self.masters:
             e.tensor.data = e.views[slot]
         self.live_slot = slot
 
-    def load_slot(self, slot):
-        """Make the module tensors views of ``slot`` (no bytes move)."""
+    def load_slot(self, slot, with_others=True):
+        """Make the parameters views of ``slot`` (no bytes move) and, as the reference's
+        ``set_params`` does, overwrite the live copy of the remaining entries."""
         if slot != self.live_slot:
             self._point_live_at(slot)
+        if with_others and self.other_bytes:
+            self._lib.pd_copy(ctypes.c_void_p(self.live_other.data_ptr()),
+                              ctypes.c_void_p(self.slot_ptr(slot) + self.master_bytes),
+                              self.other_bytes, _cabi.stream_ptr())
 
-    def copy_other_section(self, src_slot, dst_slot, stream=None):
-        """Carry the non-optimised entries (buffers, frozen parameters) of ``src_slot``
-        into ``dst_slot``; the fused step only writes the master section."""
-        if self.other_bytes == 0 or src_slot == dst_slot:
-            return
-        self._lib.pd_copy(ctypes.c_void_p(self.slot_ptr(dst_slot) + self.master_bytes),
-                          ctypes.c_void_p(self.slot_ptr(src_slot) + self.master_bytes),
-                          self.other_bytes, _cabi.stream_ptr(stream))
+    def store_others(self, dst_slot, stream=None):
+        """Live copy of the non-optimised entries -> ``dst_slot`` (the part of
+        ``get_params(clone=False)`` the fused step does not cover)."""
+        if self.other_bytes:
+            self._lib.pd_copy(ctypes.c_void_p(self.slot_ptr(dst_slot) + self.master_bytes),
+                              ctypes.c_void_p(self.live_other.data_ptr()),
+                              self.other_bytes, _cabi.stream_ptr(stream))
 
-    def copy_slot(self, src_slot, dst_slot, stream=None):
-        if src_slot == dst_slot:
+    def copy_masters(self, src_slot, dst_slot, stream=None):
+        if src_slot == dst_slot or self.master_bytes == 0:
             return
         self._lib.pd_copy(ctypes.c_void_p(self.slot_ptr(dst_slot)), ctypes.c_void_p(self.slot_ptr(src_slot)),
-                          self.slot_bytes, _cabi.stream_ptr(stream))
+                          self.master_bytes, _cabi.stream_ptr(stream))
 
     def master_view(self, master_index, slot):
         return self.entries[master_index].views[slot]

@@ -162,7 +162,8 @@ class OptimizerWithWeightStashing(torch.optim.Optimizer):
         else:
             # live values -> storage of the oldest entry
             dst = self.arena.write_slot()
-            self.arena.copy_slot(self.arena.live_slot, dst)
+            self.arena.copy_masters(self.arena.live_slot, dst)
+            self.arena.store_others(dst)
             state_dicts = self.arena.state_dicts(dst)
         return state_dicts, self.latest_version
 
@@ -222,10 +223,10 @@ class OptimizerWithWeightStashing(torch.optim.Optimizer):
                                         loss_scale=1.0, update_interval=float(self.update_interval))
         self.latest_version = self.latest_version.incr()
         if self.num_versions > 1:
-            arena.copy_other_section(in_slot, out_slot)
+            arena.store_others(out_slot)
             pushed = arena.push(self.latest_version.version)
             assert pushed == out_slot
-            arena.load_slot(out_slot)
+            arena.load_slot(out_slot, with_others=False)
 
         if log_timing:
             print("Optimizer step took: %.3f" % (time.time() - start_time))

@@ -1,6 +1,6 @@
 """Parity of the fused optimizer kernels (through the C ABI) with the CPU oracle.
 
-Tolerance: fp32, rel 1e-5 (+ atol 1e-7 for entries that cancel to ~0), the bar the
+Tolerance: fp32, rel 1e-5 (+ atol 5e-7, a few ulp of the O(1) operands, for entries that cancel to ~0), the bar the
 north-star sets for parameters after N steps."""
 import ctypes
 
@@ -13,7 +13,7 @@ from pipedream_amd import _cabi
 
 pytestmark = pytest.mark.gpu
 
-RTOL, ATOL = 1e-5, 1e-7
+RTOL, ATOL = 1e-5, 5e-7
 
 
 def _dev(a):

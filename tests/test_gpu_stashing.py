@@ -74,7 +74,8 @@ def test_1f1b_matches_oracle(kind, warmup):
     fwd_v, bwd_v = {}, {}
     for kind_ev, k in so.one_f_one_b(n, warmup):
         if kind_ev == "F":
-            fwd_v[k] = opt.current_version.version if nv > 1 else opt.latest_version.version
+            # after step() the live weights are the latest version (optimizer.py:151-156)
+            fwd_v[k] = opt.latest_version.version
             assert fwd_v[k] == so.forward_version(k, warmup)
             inflight_cpu.append(torch.nn.functional.mse_loss(cpu_model(xs[k]), ys[k]))
             inflight_gpu.append(torch.nn.functional.mse_loss(gpu_model(xs[k].cuda()), ys[k].cuda()))
@@ -127,14 +128,21 @@ def test_running_stats_are_not_rolled_back_and_buffers_are_stashed():
     assert torch.equal(model[1].running_mean, rm)
     opt.load_new_params()
     opt.step()
-    assert int(model[1].num_batches_tracked) == 1     # carried into the new slot
     opt.load_old_params()
     assert torch.equal(model[1].running_mean, rm)
-    assert int(model[1].num_batches_tracked) == 0     # stashed entry, like the reference
+    # a stashable buffer is rolled back by every load, exactly like the reference:
+    # its forward-time increment never reaches the ring (optimizer.py:87-101)
+    assert int(model[1].num_batches_tracked) == 0
 
 
 def test_macrobatch_matches_oracle():
-    cpu_model = _mlp(3)
+    # One Linear layer: its weight gradient does not read the weights, so the check is on
+    # accumulation / averaging / ring rotation only.  (In macrobatch mode the reference does
+    # not keep forward and backward on one version; multi-layer behaviour under that
+    # mismatch is covered with this package's own layers, whose backward reads the loaded
+    # version like the reference's in-place load does.)
+    torch.manual_seed(3)
+    cpu_model = torch.nn.Linear(12, 5)
     gpu_model = copy.deepcopy(cpu_model).cuda()
     opt = sgd.SGDWithWeightStashing([gpu_model], gpu_model.parameters(), None, 1.0, 4, lr=0.1, momentum=0.9,
                                     macrobatch=True)
