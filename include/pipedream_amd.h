@@ -119,6 +119,49 @@ int pd_adam_step(const pd_tensor_desc* descs, int n_tensors,
                  int64_t step, int eps_mode,
                  double loss_scale, double update_interval, void* stream);
 
+/* ------------------------------------------------------------------------- *
+ * Stage compute.  These replace the library kernels (cuBLAS / cuDNN / ATen)
+ * that the torch.nn modules of a reference stage call in
+ * StageRuntime._run_forward (runtime/runtime.py:505-546) and that
+ * torch.autograd.backward replays in run_backward (runtime/runtime.py:606-608).
+ * ------------------------------------------------------------------------- */
+
+/* Row-major fp32 GEMM on MFMA:  C[M,N] = op(A) op(B) (+ bias[N]) (+ beta*C) (ReLU)
+ * op(A) is [M,K]: A is stored [M][lda] (trans_a=0) or [K][lda] (trans_a=1);
+ * op(B) is [K,N]: B is stored [K][ldb] (trans_b=0) or [N][ldb] (trans_b=1).
+ * torch.nn.Linear forward  = (0,1): Y = X W^T + b   (stage3.py:19 Linear layers)
+ * its input gradient       = (0,0): dX = dY W
+ * its weight gradient      = (1,0): dW = dY^T X */
+int pd_gemm_f32(int trans_a, int trans_b, int M, int N, int K,
+                const float* A, int lda, const float* B, int ldb,
+                float beta, float* C, int ldc, const float* bias, int relu, void* stream);
+
+/* out[s][n] = sum over the s-th of `splits` row ranges of x[m][n]  (bias gradients).
+ * With splits == 1 and beta != 0 the sum is added to beta*out. */
+int pd_colsum_f32(const float* x, float* out, uint64_t M, int N, uint64_t ld, int splits, float beta, void* stream);
+
+/* torch.nn.ReLU forward / backward (stage0.py:13). dx = dy where y > 0. */
+int pd_relu_fwd_f32(const float* x, float* y, uint64_t n, void* stream);
+int pd_relu_bwd_f32(const float* dy, const float* y, float* dx, uint64_t n, void* stream);
+
+/* torch.nn.MaxPool2d(kernel_size=2, stride=2) on NHWC tensors (stage1.py:11).
+ * y is [N, H/2, W/2, C].  Backward writes all of dx; first maximum wins ties.
+ * relu_mask != 0 additionally zeroes dx where x <= 0 (fused ReLU backward). */
+int pd_maxpool2x2_fwd_nhwc_f32(const float* x, float* y, int N, int H, int W, int C, void* stream);
+int pd_maxpool2x2_bwd_nhwc_f32(const float* x, const float* dy, float* dx, int N, int H, int W, int C,
+                               int relu_mask, void* stream);
+
+/* torch.nn.CrossEntropyLoss(reduction='mean') -- the criterion the caller appends to
+ * the module list (main_with_runtime.py:126, applied at runtime/runtime.py:523-526).
+ * loss[0] = mean over non-ignored rows of (logsumexp(x_b) - x_b[target_b]);
+ * row_loss[B], lse[B], count[1] are outputs kept for the backward pass.
+ * Backward: dlogits = (softmax(x) - onehot(target)) * grad_loss[0] / count[0]. */
+int pd_xent_fwd_f32(const float* logits, const int64_t* target, float* loss, float* row_loss, float* lse,
+                    float* count, int B, int C, int ld, int64_t ignore_index, void* stream);
+int pd_xent_bwd_f32(const float* logits, const int64_t* target, const float* lse, const float* grad_loss,
+                    const float* count, float* dlogits, int B, int C, int ld, int ldd,
+                    int64_t ignore_index, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

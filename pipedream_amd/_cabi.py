@@ -62,6 +62,14 @@ SIGNATURES = {
     "pd_fill_zero": (_i, [_vp, _u64, _vp], True),
     "pd_sgd_step": (_i, [ctypes.POINTER(TensorDesc), _i, _d, _d, _d, _d, _i, _i, _d, _d, _vp], True),
     "pd_adam_step": (_i, [ctypes.POINTER(TensorDesc), _i, _d, _d, _d, _d, _d, _i64, _i, _d, _d, _vp], True),
+    "pd_gemm_f32": (_i, [_i, _i, _i, _i, _i, _vp, _i, _vp, _i, _f, _vp, _i, _vp, _i, _vp], True),
+    "pd_colsum_f32": (_i, [_vp, _vp, _u64, _i, _u64, _i, _f, _vp], True),
+    "pd_relu_fwd_f32": (_i, [_vp, _vp, _u64, _vp], True),
+    "pd_relu_bwd_f32": (_i, [_vp, _vp, _vp, _u64, _vp], True),
+    "pd_maxpool2x2_fwd_nhwc_f32": (_i, [_vp, _vp, _i, _i, _i, _i, _vp], True),
+    "pd_maxpool2x2_bwd_nhwc_f32": (_i, [_vp, _vp, _vp, _i, _i, _i, _i, _i, _vp], True),
+    "pd_xent_fwd_f32": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i64, _vp], True),
+    "pd_xent_bwd_f32": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i64, _vp], True),
 }
 
 

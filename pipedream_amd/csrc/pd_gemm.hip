@@ -1,0 +1,237 @@
+// fp32 GEMM on the gfx950 matrix cores (v_mfma_f32_32x32x2_f32), used by the
+// Linear / LSTM / projection layers of a stage: forward  Y = X W^T + b,
+// input gradient dX = dY W, weight gradient dW = dY^T X.
+//
+// Replaces the cuBLAS calls torch.nn.Linear / torch.nn.LSTM make inside the
+// reference's stage modules (e.g. runtime/image_classification/models/vgg16/
+// gpus=4_straight/stage3.py:19-25) and their autograd backward
+// (runtime/runtime.py:529-530 forward, :606-608 backward).
+//
+// Bound: MFMA fp32 (157.3 TFLOP/s).  2*M*N*K flop per call.
+//
+// Tiling: a 256-thread block (4 waves, 2x2) owns a BM x BN tile of C; each wave
+// owns (BM/2) x (BN/2) = TM x TN MFMA tiles of 32x32.  K is consumed in chunks of
+// 16 staged through LDS in the operand's own memory order (no transposition on
+// the way in): a k-contiguous operand is read back with one 128-bit LDS load
+// per four MFMAs, a row-contiguous one with 32-bit loads.  The k index is
+// permuted identically for A and B (lane-half h takes k = 8g + 4h + s at MFMA
+// step s), which a sum over k does not care about.
+#include "pd_internal.h"
+
+typedef float float4_t __attribute__((ext_vector_type(4)));
+typedef float float16_t __attribute__((ext_vector_type(16)));
+
+namespace {
+
+constexpr int BK = 16;
+constexpr int GEMM_THREADS = 256;
+
+struct GemmArgs {
+    const float* A;
+    const float* B;
+    float* C;
+    const float* bias;  // [N] or null
+    int M, N, K;
+    int lda, ldb, ldc;
+    float beta;         // C = acc + beta*C_old (0 -> overwrite, C_old not read)
+    int relu;
+    int a_vec, b_vec;   // 128-bit global loads allowed for A / B
+};
+
+// Operand tile in LDS.  KC (k-contiguous): [ROWS][BK+4]; otherwise [BK][ROWS+4].
+template <int ROWS, bool KC>
+struct Tile {
+    static constexpr int STRIDE = KC ? (BK + 4) : (ROWS + 4);
+    static constexpr int SIZE = KC ? ROWS * STRIDE : BK * STRIDE;
+
+    // Global -> registers.  `rows` is the extent of the row index (M or N), `k_extent` = K.
+    // Each thread moves ROWS*BK/4/256 float4s.
+    static constexpr int VEC_PER_THREAD = ROWS * BK / 4 / GEMM_THREADS;
+
+    __device__ static void load(float4_t (&r)[VEC_PER_THREAD], const float* __restrict__ g, int ld, int row0, int k0,
+                                int rows, int k_extent, bool vec, int tid) {
+#pragma unroll
+        for (int v = 0; v < VEC_PER_THREAD; ++v) {
+            int id = tid + v * GEMM_THREADS;
+            int row, k;
+            if (KC) {
+                row = id / (BK / 4);
+                k = (id % (BK / 4)) * 4;
+            } else {
+                k = id / (ROWS / 4);
+                row = (id % (ROWS / 4)) * 4;
+            }
+            int gr = row0 + row, gk = k0 + k;
+            float4_t x = {0.f, 0.f, 0.f, 0.f};
+            if (KC) {
+                if (gr < rows) {
+                    const float* p = g + (size_t)gr * ld + gk;
+                    if (vec && gk + 3 < k_extent) {
+                        x = *(const float4_t*)p;
+                    } else {
+#pragma unroll
+                        for (int j = 0; j < 4; ++j)
+                            if (gk + j < k_extent) x[j] = p[j];
+                    }
+                }
+            } else {
+                if (gk < k_extent) {
+                    const float* p = g + (size_t)gk * ld + gr;
+                    if (vec && gr + 3 < rows) {
+                        x = *(const float4_t*)p;
+                    } else {
+#pragma unroll
+                        for (int j = 0; j < 4; ++j)
+                            if (gr + j < rows) x[j] = p[j];
+                    }
+                }
+            }
+            r[v] = x;
+        }
+    }
+
+    __device__ static void store(float* lds, const float4_t (&r)[VEC_PER_THREAD], int tid) {
+#pragma unroll
+        for (int v = 0; v < VEC_PER_THREAD; ++v) {
+            int id = tid + v * GEMM_THREADS;
+            int row, k;
+            if (KC) {
+                row = id / (BK / 4);
+                k = (id % (BK / 4)) * 4;
+                *(float4_t*)(lds + row * STRIDE + k) = r[v];
+            } else {
+                k = id / (ROWS / 4);
+                row = (id % (ROWS / 4)) * 4;
+                *(float4_t*)(lds + k * STRIDE + row) = r[v];
+            }
+        }
+    }
+
+    // Fragment for MFMA steps s=0..3 of k-group g: lane (idx = lane%32, h = lane/32)
+    // supplies element [row0+idx][8g + 4h + s].
+    __device__ static float4_t frag(const float* lds, int row, int g, int h) {
+        if (KC) {
+            return *(const float4_t*)(lds + row * STRIDE + 8 * g + 4 * h);
+        } else {
+            float4_t f;
+#pragma unroll
+            for (int s = 0; s < 4; ++s) f[s] = lds[(8 * g + 4 * h + s) * STRIDE + row];
+            return f;
+        }
+    }
+};
+
+template <int BM, int BN, bool A_KC, bool B_KC>
+__global__ __launch_bounds__(GEMM_THREADS) void pd_gemm_f32_kernel(const GemmArgs a) {
+    constexpr int TM = BM / 64, TN = BN / 64;  // MFMA tiles per wave in m / n
+    using TA = Tile<BM, A_KC>;
+    using TB = Tile<BN, B_KC>;
+    __shared__ __attribute__((aligned(16))) float lds_a[2][TA::SIZE];
+    __shared__ __attribute__((aligned(16))) float lds_b[2][TB::SIZE];
+
+    const int tid = threadIdx.x;
+    const int wave = tid / 64, lane = tid % 64;
+    const int wm = wave / 2, wn = wave % 2;
+    const int idx = lane % 32, h = lane / 32;
+    const int m0 = blockIdx.y * BM, n0 = blockIdx.x * BN;
+
+    float16_t acc[TM][TN];
+#pragma unroll
+    for (int i = 0; i < TM; ++i)
+#pragma unroll
+        for (int j = 0; j < TN; ++j)
+#pragma unroll
+            for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.f;
+
+    float4_t ra[TA::VEC_PER_THREAD], rb[TB::VEC_PER_THREAD];
+    const int nk = (a.K + BK - 1) / BK;
+    TA::load(ra, a.A, a.lda, m0, 0, a.M, a.K, a.a_vec, tid);
+    TB::load(rb, a.B, a.ldb, n0, 0, a.N, a.K, a.b_vec, tid);
+    TA::store(lds_a[0], ra, tid);
+    TB::store(lds_b[0], rb, tid);
+    __syncthreads();
+
+    for (int kt = 0; kt < nk; ++kt) {
+        const int cur = kt & 1;
+        if (kt + 1 < nk) {  // prefetch the next chunk into registers while this one is multiplied
+            TA::load(ra, a.A, a.lda, m0, (kt + 1) * BK, a.M, a.K, a.a_vec, tid);
+            TB::load(rb, a.B, a.ldb, n0, (kt + 1) * BK, a.N, a.K, a.b_vec, tid);
+        }
+#pragma unroll
+        for (int g = 0; g < BK / 8; ++g) {
+            float4_t fa[TM], fb[TN];
+#pragma unroll
+            for (int i = 0; i < TM; ++i) fa[i] = TA::frag(lds_a[cur], wm * (BM / 2) + i * 32 + idx, g, h);
+#pragma unroll
+            for (int j = 0; j < TN; ++j) fb[j] = TB::frag(lds_b[cur], wn * (BN / 2) + j * 32 + idx, g, h);
+#pragma unroll
+            for (int s = 0; s < 4; ++s)
+#pragma unroll
+                for (int i = 0; i < TM; ++i)
+#pragma unroll
+                    for (int j = 0; j < TN; ++j)
+                        acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(fa[i][s], fb[j][s], acc[i][j], 0, 0, 0);
+        }
+        if (kt + 1 < nk) {
+            TA::store(lds_a[cur ^ 1], ra, tid);
+            TB::store(lds_b[cur ^ 1], rb, tid);
+        }
+        __syncthreads();
+    }
+
+    // Epilogue.  Accumulator element e of lane (idx, h): row = 8*(e/4) + 4*h + e%4, col = idx.
+#pragma unroll
+    for (int i = 0; i < TM; ++i)
+#pragma unroll
+        for (int j = 0; j < TN; ++j) {
+            const int col = n0 + wn * (BN / 2) + j * 32 + idx;
+            if (col >= a.N) continue;
+            const float bv = a.bias ? a.bias[col] : 0.f;
+#pragma unroll
+            for (int e = 0; e < 16; ++e) {
+                const int row = m0 + wm * (BM / 2) + i * 32 + 8 * (e / 4) + 4 * h + (e % 4);
+                if (row >= a.M) continue;
+                float* p = a.C + (size_t)row * a.ldc + col;
+                float v = acc[i][j][e] + bv;
+                if (a.beta != 0.f) v += a.beta * *p;
+                if (a.relu) v = v > 0.f ? v : 0.f;
+                *p = v;
+            }
+        }
+}
+
+template <int BM, int BN>
+int launch_gemm(int trans_a, int trans_b, const GemmArgs& g, hipStream_t s) {
+    dim3 grid((g.N + BN - 1) / BN, (g.M + BM - 1) / BM);
+    // A is k-contiguous when it is NOT transposed; B (stored [K][N]) is k-contiguous when it IS.
+    if (!trans_a && trans_b) pd_gemm_f32_kernel<BM, BN, true, true><<<grid, GEMM_THREADS, 0, s>>>(g);
+    else if (!trans_a && !trans_b) pd_gemm_f32_kernel<BM, BN, true, false><<<grid, GEMM_THREADS, 0, s>>>(g);
+    else if (trans_a && !trans_b) pd_gemm_f32_kernel<BM, BN, false, false><<<grid, GEMM_THREADS, 0, s>>>(g);
+    else pd_gemm_f32_kernel<BM, BN, false, true><<<grid, GEMM_THREADS, 0, s>>>(g);
+    PD_CHECK_LAUNCH("pd_gemm_f32");
+    return PD_OK;
+}
+
+}  // namespace
+
+extern "C" int pd_gemm_f32(int trans_a, int trans_b, int M, int N, int K, const float* A, int lda, const float* B,
+                           int ldb, float beta, float* C, int ldc, const float* bias, int relu, void* stream) {
+    PD_REQUIRE(M >= 0 && N >= 0 && K >= 0, PD_ESHAPE, "pd_gemm_f32: negative dimension");
+    if (M == 0 || N == 0) return PD_OK;
+    PD_REQUIRE(A && B && C, PD_EINVAL, "pd_gemm_f32: NULL operand");
+    PD_REQUIRE(lda >= (trans_a ? M : K) && ldb >= (trans_b ? K : N) && ldc >= N, PD_ESHAPE,
+               "pd_gemm_f32: leading dimension smaller than the row length");
+    GemmArgs g;
+    g.A = A; g.B = B; g.C = C; g.bias = bias;
+    g.M = M; g.N = N; g.K = K;
+    g.lda = lda; g.ldb = ldb; g.ldc = ldc;
+    g.beta = beta;
+    g.relu = relu != 0;
+    g.a_vec = pd_aligned(A, 16) && lda % 4 == 0;
+    g.b_vec = pd_aligned(B, 16) && ldb % 4 == 0;
+    hipStream_t s = (hipStream_t)stream;
+    // Small problems use 64x64 tiles so that more of the 256 CUs get a block.
+    long tiles128 = (long)((M + 127) / 128) * ((N + 127) / 128);
+    if (tiles128 >= 256) return launch_gemm<128, 128>(trans_a, trans_b, g, s);
+    return launch_gemm<64, 64>(trans_a, trans_b, g, s);
+}

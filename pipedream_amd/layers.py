@@ -1,0 +1,176 @@
+"""Stage building blocks: ``torch.nn.Module``s whose forward and backward run on the
+hand-written HIP kernels of ``libpipedream_amd.so``.
+
+They carry the parameter names, shapes and initialisation of the ``torch.nn`` layers
+used by the reference's generated stage modules (``weight`` / ``bias``; e.g.
+runtime/image_classification/models/vgg16/gpus=4_straight/stage0.py:10-33), so their
+``state_dict()`` is interchangeable with the reference's.  Every backward reads the
+parameter tensors as they are *at backward time*, i.e. the weight version that
+``load_old_params`` made current -- the semantics of the reference's in-place
+``load_state_dict`` (runtime/optimizer.py:87-112).
+"""
+import math
+
+import torch
+
+from . import ops
+
+
+# --------------------------------------------------------------------------------------
+# Linear
+# --------------------------------------------------------------------------------------
+class _LinearFn(torch.autograd.Function):
+    @staticmethod
+    def forward(ctx, x, weight, bias, relu):
+        x2 = x.reshape(-1, x.shape[-1])
+        if x2.stride(-1) != 1 or (x2.size(0) > 1 and x2.stride(0) < x2.size(1)):
+            x2 = x2.contiguous()
+        y = ops.gemm(x2, weight, trans_b=True, bias=bias, relu=relu)
+        ctx.relu = relu
+        ctx.has_bias = bias is not None
+        ctx.x_shape = x.shape
+        ctx.save_for_backward(x2, weight, y if relu else None)
+        return y.view(*x.shape[:-1], weight.shape[0])
+
+    @staticmethod
+    def backward(ctx, dy):
+        x2, weight, y = ctx.saved_tensors
+        dy2 = dy.reshape(-1, dy.shape[-1])
+        if ctx.relu:
+            dy2 = ops.relu_backward(dy2, y)
+        elif dy2.stride(-1) != 1 or (dy2.size(0) > 1 and dy2.stride(0) < dy2.size(1)):
+            dy2 = dy2.contiguous()
+        dx = dw = db = None
+        if ctx.needs_input_grad[0]:
+            dx = ops.gemm(dy2, weight).view(ctx.x_shape)
+        if ctx.needs_input_grad[1]:
+            dw = ops.gemm(dy2, x2, trans_a=True)
+        if ctx.has_bias and ctx.needs_input_grad[2]:
+            db = ops.colsum(dy2)
+        return dx, dw, db, None
+
+
+class Linear(torch.nn.Module):
+    """``torch.nn.Linear`` (optionally with the following ReLU fused into the GEMM epilogue)."""
+
+    def __init__(self, in_features, out_features, bias=True, relu=False):
+        super(Linear, self).__init__()
+        self.in_features = in_features
+        self.out_features = out_features
+        self.relu = relu
+        self.weight = torch.nn.Parameter(torch.empty(out_features, in_features))
+        self.bias = torch.nn.Parameter(torch.empty(out_features)) if bias else None
+        self.reset_parameters()
+
+    def reset_parameters(self):
+        torch.nn.init.kaiming_uniform_(self.weight, a=math.sqrt(5))
+        if self.bias is not None:
+            bound = 1 / math.sqrt(self.in_features) if self.in_features > 0 else 0
+            torch.nn.init.uniform_(self.bias, -bound, bound)
+
+    def forward(self, x):
+        return _LinearFn.apply(x, self.weight, self.bias, self.relu)
+
+    def extra_repr(self):
+        return "in_features={}, out_features={}, bias={}, relu={}".format(
+            self.in_features, self.out_features, self.bias is not None, self.relu)
+
+
+# --------------------------------------------------------------------------------------
+# ReLU / MaxPool
+# --------------------------------------------------------------------------------------
+class _ReLUFn(torch.autograd.Function):
+    @staticmethod
+    def forward(ctx, x):
+        y = ops.relu(x)
+        ctx.save_for_backward(y)
+        return y
+
+    @staticmethod
+    def backward(ctx, dy):
+        (y,) = ctx.saved_tensors
+        return ops.relu_backward(dy, y)
+
+
+class ReLU(torch.nn.Module):
+    """``torch.nn.ReLU``.  ``inplace`` is accepted for signature compatibility; the result
+    is always a new tensor (the stash keeps every in-flight activation anyway)."""
+
+    def __init__(self, inplace=False):
+        super(ReLU, self).__init__()
+        self.inplace = inplace
+
+    def forward(self, x):
+        return _ReLUFn.apply(x)
+
+
+class _MaxPool2x2Fn(torch.autograd.Function):
+    @staticmethod
+    def forward(ctx, x, after_relu):
+        x = ops.to_nhwc(x)
+        y = ops.maxpool2x2(x)
+        ctx.after_relu = after_relu
+        ctx.save_for_backward(x)
+        return y
+
+    @staticmethod
+    def backward(ctx, dy):
+        (x,) = ctx.saved_tensors
+        return ops.maxpool2x2_backward(x, dy, relu_mask=False), None
+
+
+class MaxPool2d(torch.nn.Module):
+    """``torch.nn.MaxPool2d(kernel_size=2, stride=2)`` on NHWC activations."""
+
+    def __init__(self, kernel_size=2, stride=2, padding=0, dilation=1, ceil_mode=False):
+        super(MaxPool2d, self).__init__()
+        ks = kernel_size if isinstance(kernel_size, int) else kernel_size[0]
+        st = ks if stride is None else (stride if isinstance(stride, int) else stride[0])
+        if ks != 2 or st != 2 or padding not in (0, (0, 0)) or dilation not in (1, (1, 1)) or ceil_mode:
+            raise NotImplementedError("only MaxPool2d(kernel_size=2, stride=2) has a HIP kernel")
+
+    def forward(self, x):
+        return _MaxPool2x2Fn.apply(x, False)
+
+
+class Flatten(torch.nn.Module):
+    """``out.view(out.size(0), -1)`` of the reference's stages (stage3.py:35-36): features
+    in C,H,W order whatever the memory order of the incoming activation."""
+
+    def forward(self, x):
+        return x.contiguous().view(x.size(0), -1)
+
+
+# --------------------------------------------------------------------------------------
+# Criterion
+# --------------------------------------------------------------------------------------
+class _CrossEntropyFn(torch.autograd.Function):
+    @staticmethod
+    def forward(ctx, logits, target, ignore_index):
+        x2 = logits.reshape(-1, logits.shape[-1])
+        if x2.stride(-1) != 1:
+            x2 = x2.contiguous()
+        t = target.reshape(-1).contiguous()
+        loss, (lse, count) = ops.cross_entropy_forward(x2, t, ignore_index)
+        ctx.ignore_index = ignore_index
+        ctx.shape = logits.shape
+        ctx.save_for_backward(x2, t, lse, count)
+        return loss
+
+    @staticmethod
+    def backward(ctx, grad_loss):
+        x2, t, lse, count = ctx.saved_tensors
+        d = ops.cross_entropy_backward(x2, t, lse, count, grad_loss.contiguous(), ctx.ignore_index)
+        return d.view(ctx.shape), None, None
+
+
+class CrossEntropyLoss(torch.nn.Module):
+    """``torch.nn.CrossEntropyLoss()`` with mean reduction -- the criterion
+    runtime/image_classification/main_with_runtime.py:126 creates."""
+
+    def __init__(self, ignore_index=-100):
+        super(CrossEntropyLoss, self).__init__()
+        self.ignore_index = ignore_index
+
+    def forward(self, logits, target):
+        return _CrossEntropyFn.apply(logits, target, self.ignore_index)

@@ -1,0 +1,83 @@
+"""The 1F1B training loop of one stage, and a driver that interleaves the loops of
+several co-resident stages on one GPU.
+
+``stage_train_loop`` is the body of ``train()`` in the reference's caller
+(runtime/image_classification/main_with_runtime.py:333-427): ``W`` warm-up forwards,
+then ``n - W`` times [forward, adjust lr, zero_grad, load_old_params, backward,
+load_new_params, step], then ``W`` times the backward half.  In the reference every
+stage is its own process and simply blocks in a receive queue; here the loop is a
+generator that yields whenever its next receive would find the queue empty, and
+``run_pipeline`` round-robins the generators until all are finished.
+"""
+
+
+def stage_train_loop(r, optimizer, num_minibatches, loader=None, lr_schedule=None, on_forward=None,
+                     no_input_pipelining=False):
+    """Generator running one stage's 1F1B schedule.
+
+    ``lr_schedule(step) -> lr`` is written into every param group each iteration, as
+    ``adjust_learning_rate`` does (main_with_runtime.py:562-563).  ``on_forward(i, r)`` is
+    called after each steady-state forward (where the reference reads ``r.loss``)."""
+    n = num_minibatches
+    r.train(n)
+    r.set_loader(loader if (r.stage is None or r.stage == 0) else None)
+    warmup = 0 if no_input_pipelining else min(r.num_warmup_minibatches, n)
+
+    def forward():
+        while not r.can_run_forward():
+            yield r
+        r.run_forward()
+
+    def backward_and_update():
+        optimizer.zero_grad()
+        optimizer.load_old_params()
+        while not r.can_run_backward():
+            yield r
+        r.run_backward()
+        optimizer.load_new_params()
+        optimizer.step()
+
+    for _ in range(warmup):
+        for blocked in forward():
+            yield blocked
+    for i in range(n - warmup):
+        for blocked in forward():
+            yield blocked
+        if lr_schedule is not None:
+            lr = lr_schedule(i)
+            for param_group in optimizer.param_groups:
+                param_group['lr'] = lr
+        if on_forward is not None:
+            on_forward(i, r)
+        for blocked in backward_and_update():
+            yield blocked
+    for _ in range(warmup):
+        for blocked in backward_and_update():
+            yield blocked
+    r.wait()
+
+
+def run_pipeline(loops):
+    """Drive the stage loops to completion.  ``loops`` are ``stage_train_loop``
+    generators, first stage first.  A generator yields only when its stage is blocked on
+    an empty queue; a full round in which every stage is blocked and none has advanced
+    its minibatch counters is a deadlock and raises."""
+    live = list(loops)
+    last_signature = None
+    while live:
+        signature = []
+        finished = False
+        for g in list(live):
+            try:
+                r = next(g)
+                signature.append((r.forward_minibatch_id, r.backward_minibatch_id))
+            except StopIteration:
+                live.remove(g)
+                finished = True
+        if live and not finished:
+            if signature == last_signature:
+                raise RuntimeError("pipeline schedule deadlocked: every stage waits for a tensor "
+                                   "(minibatch counters %s)" % (signature,))
+            last_signature = signature
+        else:
+            last_signature = None

@@ -1,0 +1,151 @@
+"""Stage-compute kernels (through the C ABI) against the fp32/fp64 torch CPU library --
+the third-party routines the reference's stage modules call.
+
+Tolerances: GEMM results are compared with an fp64 product; an fp32 dot product of
+length K carries a relative rounding error of about sqrt(K)*6e-8 on its magnitude
+sum |a||b|, so the bound is atol = 2e-6*sqrt(K)*max|a||b| with rtol 1e-5.  Element-wise
+kernels must be bit-exact."""
+import math
+
+import pytest
+import torch
+import torch.nn.functional as F
+
+from pipedream_amd import layers, ops
+
+pytestmark = pytest.mark.gpu
+
+
+def _gemm_case(M, N, K, ta, tb, bias=False, relu=False, beta=0.0, seed=0):
+    g = torch.Generator().manual_seed(seed)
+    a = torch.randn((K, M) if ta else (M, K), generator=g)
+    b = torch.randn((N, K) if tb else (K, N), generator=g)
+    bv = torch.randn(N, generator=g) if bias else None
+    c0 = torch.randn(M, N, generator=g) if beta else None
+    want = (a.double().t() if ta else a.double()) @ (b.double().t() if tb else b.double())
+    if bias:
+        want = want + bv.double()
+    if beta:
+        want = want + beta * c0.double()
+    if relu:
+        want = want.clamp_min(0)
+    out = c0.cuda() if beta else None
+    got = ops.gemm(a.cuda(), b.cuda(), trans_a=ta, trans_b=tb, bias=bv.cuda() if bias else None, relu=relu,
+                   out=out, beta=beta)
+    torch.cuda.synchronize()
+    atol = 2e-6 * math.sqrt(max(K, 1)) * 9.0
+    torch.testing.assert_close(got.cpu().double(), want, rtol=1e-5, atol=atol)
+
+
+@pytest.mark.parametrize("ta,tb", [(False, True), (False, False), (True, False), (True, True)])
+@pytest.mark.parametrize("M,N,K", [(64, 64, 16), (64, 1024, 784), (130, 70, 33), (1, 10, 1024), (257, 129, 100),
+                                   (5, 3, 1), (2048, 2304, 64)])
+def test_gemm_layouts_and_ragged_shapes(M, N, K, ta, tb):
+    _gemm_case(M, N, K, ta, tb)
+
+
+def test_gemm_epilogues():
+    _gemm_case(64, 1024, 784, False, True, bias=True, relu=True)
+    _gemm_case(100, 50, 37, False, True, bias=True)
+    _gemm_case(100, 50, 37, True, False, beta=1.0)
+    _gemm_case(300, 300, 300, False, False, bias=True, relu=True, beta=0.5)
+
+
+def test_gemm_strided_views_and_identity():
+    # leading dimension larger than the row; unaligned base (scalar load path)
+    big = torch.randn(70, 90).cuda()
+    a = big[:, 1:34]          # 33 cols, ld 90, 4-byte aligned only
+    b = torch.randn(20, 33).cuda()
+    got = ops.gemm(a, b, trans_b=True)
+    torch.testing.assert_close(got.cpu().double(), a.cpu().double() @ b.cpu().double().t(), rtol=1e-5, atol=1e-4)
+    # exactness: multiplying by the identity returns the operand bit-for-bit
+    x = torch.randn(96, 64).cuda()
+    assert torch.equal(ops.gemm(x, torch.eye(64).cuda()), x)
+    assert torch.equal(ops.gemm(torch.eye(96).cuda(), x), x)
+    assert torch.equal(ops.gemm(x, torch.eye(96).cuda(), trans_a=True), x.t().contiguous())
+
+
+def test_gemm_rejects_bad_operands():
+    a = torch.randn(4, 5).cuda()
+    with pytest.raises(ValueError):
+        ops.gemm(a, torch.randn(4, 6).cuda())
+    with pytest.raises(ValueError):
+        ops.gemm(a.t(), torch.randn(4, 6).cuda())     # not row-major
+    with pytest.raises(RuntimeError, match="no CPU fallback"):
+        ops.gemm(torch.randn(4, 5), torch.randn(5, 6))
+    with pytest.raises(TypeError):
+        ops.gemm(a.double(), torch.randn(5, 6).cuda().double())
+
+
+@pytest.mark.parametrize("M,N", [(1, 1), (7, 130), (5000, 64), (200000, 10)])
+def test_colsum(M, N):
+    x = torch.randn(M, N)
+    got = ops.colsum(x.cuda())
+    torch.testing.assert_close(got.cpu().double(), x.double().sum(0), rtol=1e-5, atol=2e-6 * math.sqrt(M) * 4)
+
+
+def test_relu_forward_backward_bit_exact():
+    for n in (1, 5, 1024, 100003):
+        x = torch.randn(n)
+        dy = torch.randn(n)
+        y = ops.relu(x.cuda())
+        assert torch.equal(y.cpu(), x.clamp_min(0))
+        dx = ops.relu_backward(dy.cuda(), y)
+        assert torch.equal(dx.cpu(), dy * (x > 0))
+
+
+@pytest.mark.parametrize("shape", [(2, 8, 6, 6), (3, 4, 7, 9), (1, 64, 224, 224), (2, 12, 2, 5)])
+def test_maxpool_forward_backward_bit_exact(shape):
+    g = torch.Generator().manual_seed(1)
+    # quantised values force ties; torch's rule (first maximum in scan order) must hold
+    x = (torch.randn(shape, generator=g) * 2).round() / 2
+    x.requires_grad_(True)
+    y_ref = F.max_pool2d(x, 2, 2)
+    dy = torch.randn(y_ref.shape, generator=g)
+    if y_ref.numel():
+        y_ref.backward(dy)
+    xg = x.detach().cuda().contiguous(memory_format=torch.channels_last)
+    y = ops.maxpool2x2(xg)
+    assert y.shape == y_ref.shape and torch.equal(y.cpu(), y_ref.detach())
+    dx = ops.maxpool2x2_backward(xg, dy.cuda())
+    assert torch.equal(dx.cpu(), x.grad if x.grad is not None else torch.zeros(shape))
+    # fused ReLU mask: same as masking afterwards
+    dxm = ops.maxpool2x2_backward(xg, dy.cuda(), relu_mask=True)
+    assert torch.equal(dxm.cpu(), dx.cpu() * (x.detach() > 0))
+
+
+@pytest.mark.parametrize("B,C", [(64, 10), (64, 1000), (7, 32320), (1, 3)])
+def test_cross_entropy_vs_torch(B, C):
+    g = torch.Generator().manual_seed(2)
+    x = (torch.randn(B, C, generator=g) * 3).requires_grad_(True)
+    t = torch.randint(0, C, (B,), generator=g)
+    if B > 2:
+        t[1] = -100
+    ref = F.cross_entropy(x, t)
+    ref.backward(torch.tensor(0.7))
+    loss, (lse, count) = ops.cross_entropy_forward(x.detach().cuda(), t.cuda())
+    torch.testing.assert_close(loss.cpu(), ref.detach(), rtol=1e-5, atol=1e-6)
+    d = ops.cross_entropy_backward(x.detach().cuda(), t.cuda(), lse, count, torch.tensor(0.7).cuda())
+    torch.testing.assert_close(d.cpu(), x.grad, rtol=1e-5, atol=1e-7)
+    if B > 2:
+        assert not d[1].any()
+
+
+def test_linear_layer_matches_torch_nn():
+    torch.manual_seed(3)
+    ref = torch.nn.Linear(37, 21)
+    mine = layers.Linear(37, 21, relu=True)
+    mine.load_state_dict(ref.state_dict())
+    mine = mine.cuda()
+    x = torch.randn(4, 9, 37, requires_grad=True)
+    xg = x.detach().cuda().requires_grad_(True)
+    y_ref = torch.relu(ref(x))
+    y = mine(xg)
+    torch.testing.assert_close(y.cpu(), y_ref.detach(), rtol=1e-5, atol=1e-5)
+    dy = torch.randn(y_ref.shape)
+    y_ref.backward(dy)
+    y.backward(dy.cuda())
+    torch.testing.assert_close(xg.grad.cpu(), x.grad, rtol=1e-5, atol=1e-5)
+    torch.testing.assert_close(mine.weight.grad.cpu(), ref.weight.grad, rtol=1e-5, atol=1e-5)
+    torch.testing.assert_close(mine.bias.grad.cpu(), ref.bias.grad, rtol=1e-5, atol=1e-5)
+    assert list(mine.state_dict().keys()) == list(ref.state_dict().keys())
