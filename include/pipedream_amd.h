@@ -162,6 +162,23 @@ int pd_xent_bwd_f32(const float* logits, const int64_t* target, const float* lse
                     const float* count, float* dlogits, int B, int C, int ld, int ldd,
                     int64_t ignore_index, void* stream);
 
+/* torch.nn.Conv2d(C, K, kernel_size=3, stride=1, padding=1) on NHWC activations with a
+ * KRSC filter (the memory order of a channels_last [K,C,3,3] weight); the conv layers of
+ * the VGG16 stages (vgg16/gpus=4_straight/stage0.py:12-14).  Optional bias and fused
+ * ReLU (stage0.py:13).  y is [N,H,W,K]. */
+int pd_conv3x3_fwd_nhwc_f32(const float* x, const float* w, const float* bias, float* y,
+                            int N, int H, int W, int C, int K, int relu, void* stream);
+/* out[c][r][s][k] = w[k][2-r][2-s][c]: with this filter the forward kernel computes the
+ * input gradient, dX = conv3x3_fwd(dY, rot180(w)) (no bias, no ReLU). */
+int pd_conv3x3_filter_rot180_f32(const float* w, float* out, int K, int C, void* stream);
+/* Weight and (optional, dbias may be NULL) bias gradient of the same convolution:
+ * dw[k][r][s][c] = sum_{n,y,x} dy[n,y,x,k] * x[n,y+r-1,x+s-1,c].  Deterministic two-pass
+ * reduction through a caller-provided workspace of pd_conv3x3_wgrad_workspace_bytes(). */
+int pd_conv3x3_wgrad_workspace_bytes(int N, int H, int W, int C, int K, uint64_t* bytes);
+int pd_conv3x3_wgrad_nhwc_f32(const float* x, const float* dy, float* dw, float* dbias,
+                              void* workspace, uint64_t workspace_bytes,
+                              int N, int H, int W, int C, int K, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

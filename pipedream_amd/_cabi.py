@@ -69,6 +69,10 @@ SIGNATURES = {
     "pd_maxpool2x2_fwd_nhwc_f32": (_i, [_vp, _vp, _i, _i, _i, _i, _vp], True),
     "pd_maxpool2x2_bwd_nhwc_f32": (_i, [_vp, _vp, _vp, _i, _i, _i, _i, _i, _vp], True),
     "pd_xent_fwd_f32": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i64, _vp], True),
+    "pd_conv3x3_fwd_nhwc_f32": (_i, [_vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _vp], True),
+    "pd_conv3x3_filter_rot180_f32": (_i, [_vp, _vp, _i, _i, _vp], True),
+    "pd_conv3x3_wgrad_workspace_bytes": (_i, [_i, _i, _i, _i, _i, ctypes.POINTER(ctypes.c_uint64)], True),
+    "pd_conv3x3_wgrad_nhwc_f32": (_i, [_vp, _vp, _vp, _vp, _vp, _u64, _i, _i, _i, _i, _i, _vp], True),
     "pd_xent_bwd_f32": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i64, _vp], True),
 }
 

@@ -1,0 +1,444 @@
+// 3x3 / stride 1 / pad 1 convolution, fp32, on the gfx950 matrix cores
+// (v_mfma_f32_32x32x2_f32): forward (+bias, +ReLU), input gradient, weight and bias
+// gradient.  Activations are NHWC, filters KRSC (out-ch, kh, kw, in-ch).
+//
+// These are the kernels behind the torch.nn.Conv2d(k=3, s=1, p=1) layers of the
+// reference's VGG16 stages (runtime/image_classification/models/vgg16/
+// gpus=4_straight/stage0.py:12-14 ... stage3.py:12-17), which there run in cuDNN:
+// forward in StageRuntime._run_forward (runtime/runtime.py:529-530), the two gradients
+// inside torch.autograd.backward (runtime/runtime.py:606-608).
+//
+// Bound: MFMA fp32 (157.3 TFLOP/s).  Work per call: 2*9*C*K*N*H*W flop.
+//
+// Forward / input gradient (implicit GEMM, rows = pixels, cols = out channels,
+// reduction = 9 taps x C):
+//   a 256-thread block owns a TH x TW pixel tile (256 pixels) x 64 out channels; each
+//   of its 4 waves owns 64 pixels x 64 channels = 2x2 MFMA tiles.  The reduction runs
+//   in chunks of CC input channels: the (TH+2)x(TW+2) input halo tile and the
+//   9 x 64 x CC filter slice are staged in LDS once per chunk and all nine taps read
+//   the SAME halo tile at shifted addresses (no im2col copy).  Both LDS arrays are
+//   channel-contiguous with a row pitch of CC+4 floats, so an operand fragment for
+//   four consecutive MFMAs is one conflict-free 128-bit LDS read.
+//   The input gradient is the same kernel run on dY with the filter rotated by 180
+//   degrees and its channel roles swapped (pd_conv3x3_filter_rot180).
+// Weight gradient (rows = out channels, cols = in channels, reduction = pixels):
+//   a block owns 64 out x 64 in channels x 9 taps, each wave one 32x32 (k,c) block for
+//   all 9 taps (9 MFMA tiles = 144 accumulator registers).  Blocks stride over pixel
+//   tiles, stage dY and the X halo tile in LDS, and write per-block partial sums that a
+//   second kernel reduces in a fixed order (deterministic, no atomics).  The bias
+//   gradient falls out of the same dY tile.
+#include "pd_internal.h"
+
+typedef float float4_t __attribute__((ext_vector_type(4)));
+typedef float float16_t __attribute__((ext_vector_type(16)));
+
+namespace {
+
+constexpr int CONV_THREADS = 256;
+constexpr int BN = 64;  // out channels per block (forward / dgrad)
+
+struct ConvArgs {
+    const float* x;     // [N,H,W,C]
+    const float* w;     // [K,3,3,C]
+    const float* bias;  // [K] or null
+    float* y;           // [N,H,W,K]
+    int N, H, W, C, K;
+    int relu;
+    int tiles_x, tiles_y;
+    int c_vec;          // C % 4 == 0 and x/w 16-byte aligned: 128-bit global loads
+};
+
+template <int TH, int TW, int CC>
+__global__ __launch_bounds__(CONV_THREADS, 2) void conv3x3_fwd_kernel(const ConvArgs a) {
+    static_assert(TH * TW == 256, "a block owns 256 pixels");
+    static_assert(TW == 8 || TW == 16 || TW == 32, "an MFMA row tile is 32/TW rows of TW pixels");
+    constexpr int HW_ = TW + 2;                  // halo tile width
+    constexpr int HALO = (TH + 2) * (TW + 2);    // halo pixels
+    constexpr int CP = CC + 4;                   // LDS pitch per pixel / per filter row
+    constexpr int Q = CC / 4;                    // float4 per pixel per chunk
+    __shared__ __attribute__((aligned(16))) float in_tile[HALO * CP];
+    __shared__ __attribute__((aligned(16))) float w_tile[9 * BN * CP];
+
+    const int tid = threadIdx.x;
+    const int wave = tid / 64, lane = tid % 64;
+    const int idx = lane % 32, h = lane / 32;
+
+    int b = blockIdx.x;
+    const int tx = b % a.tiles_x;
+    b /= a.tiles_x;
+    const int ty = b % a.tiles_y;
+    const int n = b / a.tiles_y;
+    const int y0 = ty * TH, x0 = tx * TW;
+    const int k0 = blockIdx.y * BN;
+
+    float16_t acc[2][2];
+#pragma unroll
+    for (int i = 0; i < 2; ++i)
+#pragma unroll
+        for (int j = 0; j < 2; ++j)
+#pragma unroll
+            for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.f;
+
+    // LDS offsets of this lane's two pixel rows (tap 0,0) and two filter rows.
+    int a_off[2], b_off[2];
+#pragma unroll
+    for (int i = 0; i < 2; ++i) {
+        const int q = (wave * 2 + i) * 32 + idx;
+        a_off[i] = ((q / TW) * HW_ + (q % TW)) * CP + 4 * h;
+        b_off[i] = (i * 32 + idx) * CP + 4 * h;
+    }
+
+    const float* xn = a.x + (size_t)n * a.H * a.W * a.C;
+
+    for (int c0 = 0; c0 < a.C; c0 += CC) {
+        __syncthreads();  // everyone is done reading the previous chunk
+        // ---- input halo tile: pixel p, channel quad q ---------------------------------
+        for (int id = tid; id < HALO * Q; id += CONV_THREADS) {
+            const int p = id / Q, q4 = (id % Q) * 4;
+            const int gy = y0 + p / HW_ - 1, gx = x0 + p % HW_ - 1;
+            const int c = c0 + q4;
+            float4_t v = {0.f, 0.f, 0.f, 0.f};
+            if (gy >= 0 && gy < a.H && gx >= 0 && gx < a.W && c < a.C) {
+                const float* src = xn + ((size_t)gy * a.W + gx) * a.C + c;
+                if (a.c_vec) {
+                    v = *(const float4_t*)src;
+                } else {
+#pragma unroll
+                    for (int j = 0; j < 4; ++j)
+                        if (c + j < a.C) v[j] = src[j];
+                }
+            }
+            *(float4_t*)(in_tile + p * CP + q4) = v;
+        }
+        // ---- filter slice: row = tap*64 + out channel ----------------------------------
+        for (int id = tid; id < 9 * BN * Q; id += CONV_THREADS) {
+            const int row = id / Q, q4 = (id % Q) * 4;
+            const int tap = row / BN, k = k0 + row % BN;
+            const int c = c0 + q4;
+            float4_t v = {0.f, 0.f, 0.f, 0.f};
+            if (k < a.K && c < a.C) {
+                const float* src = a.w + ((size_t)k * 9 + tap) * a.C + c;
+                if (a.c_vec) {
+                    v = *(const float4_t*)src;
+                } else {
+#pragma unroll
+                    for (int j = 0; j < 4; ++j)
+                        if (c + j < a.C) v[j] = src[j];
+                }
+            }
+            *(float4_t*)(w_tile + row * CP + q4) = v;
+        }
+        __syncthreads();
+        // ---- 9 taps x CC/8 k-groups x (4 LDS reads + 16 MFMAs) ---------------------------
+#pragma unroll
+        for (int tap = 0; tap < 9; ++tap) {
+            const int shift = ((tap / 3) * HW_ + (tap % 3)) * CP;
+#pragma unroll
+            for (int g = 0; g < CC / 8; ++g) {
+                float4_t fa[2], fb[2];
+#pragma unroll
+                for (int i = 0; i < 2; ++i) fa[i] = *(const float4_t*)(in_tile + a_off[i] + shift + 8 * g);
+#pragma unroll
+                for (int j = 0; j < 2; ++j) fb[j] = *(const float4_t*)(w_tile + tap * BN * CP + b_off[j] + 8 * g);
+#pragma unroll
+                for (int s = 0; s < 4; ++s)
+#pragma unroll
+                    for (int i = 0; i < 2; ++i)
+#pragma unroll
+                        for (int j = 0; j < 2; ++j)
+                            acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(fa[i][s], fb[j][s], acc[i][j], 0, 0, 0);
+            }
+        }
+    }
+
+    // ---- epilogue: bias, ReLU, NHWC store (32 consecutive channels per lane group) ------
+    float* yn = a.y + (size_t)n * a.H * a.W * a.K;
+#pragma unroll
+    for (int j = 0; j < 2; ++j) {
+        const int k = k0 + j * 32 + idx;
+        if (k >= a.K) continue;
+        const float bv = a.bias ? a.bias[k] : 0.f;
+#pragma unroll
+        for (int i = 0; i < 2; ++i)
+#pragma unroll
+            for (int e = 0; e < 16; ++e) {
+                const int q = (wave * 2 + i) * 32 + 8 * (e / 4) + 4 * h + (e % 4);
+                const int gy = y0 + q / TW, gx = x0 + q % TW;
+                if (gy < a.H && gx < a.W) {
+                    float v = acc[i][j][e] + bv;
+                    if (a.relu) v = v > 0.f ? v : 0.f;
+                    yn[((size_t)gy * a.W + gx) * a.K + k] = v;
+                }
+            }
+    }
+}
+
+// w[K][3][3][C]  ->  out[C][3][3][K] with out[c][r][s][k] = w[k][2-r][2-s][c].
+__global__ __launch_bounds__(256) void filter_rot180_kernel(const float* __restrict__ w, float* __restrict__ out,
+                                                            int K, int C) {
+    const int total = K * 9 * C;
+    const int id = blockIdx.x * 256 + threadIdx.x;
+    if (id >= total) return;
+    const int k = id % K;
+    const int tap = (id / K) % 9;
+    const int c = id / (9 * K);
+    out[id] = w[((size_t)k * 9 + (8 - tap)) * C + c];
+}
+
+// ------------------------------------------------------------------------------------------
+// Weight gradient
+// ------------------------------------------------------------------------------------------
+struct WgradArgs {
+    const float* x;    // [N,H,W,C]
+    const float* dy;   // [N,H,W,K]
+    float* part_w;     // [gridDim.x][K][9][C]   per-block partial sums
+    float* part_b;     // [gridDim.x][K]         (null: no bias gradient)
+    int N, H, W, C, K;
+    int tiles_x, tiles_y, n_tiles;
+    int c_vec, k_vec;
+};
+
+template <int TH, int TW>
+__global__ __launch_bounds__(CONV_THREADS, 2) void conv3x3_wgrad_kernel(const WgradArgs a) {
+    constexpr int PIX = TH * TW;
+    constexpr int HW_ = TW + 2;
+    constexpr int HALO = (TH + 2) * (TW + 2);
+    constexpr int CS = 64;  // channels per LDS row (both tiles)
+    __shared__ __attribute__((aligned(16))) float dy_tile[PIX * CS];
+    __shared__ __attribute__((aligned(16))) float x_tile[HALO * CS];
+
+    const int tid = threadIdx.x;
+    const int wave = tid / 64, lane = tid % 64;
+    const int idx = lane % 32, h = lane / 32;
+    const int kt = wave / 2, ct = wave % 2;
+    const int k0 = blockIdx.y * 64, c0 = blockIdx.z * 64;
+    // this wave's 32 in-channels hold nothing when C is small: skip its MFMAs
+    const bool wave_active = (c0 + ct * 32) < a.C && (k0 + kt * 32) < a.K;
+
+    float16_t acc[9];
+#pragma unroll
+    for (int t = 0; t < 9; ++t)
+#pragma unroll
+        for (int e = 0; e < 16; ++e) acc[t][e] = 0.f;
+    float bsum = 0.f;
+
+    for (int tile = blockIdx.x; tile < a.n_tiles; tile += gridDim.x) {
+        int b = tile;
+        const int tx = b % a.tiles_x;
+        b /= a.tiles_x;
+        const int ty = b % a.tiles_y;
+        const int n = b / a.tiles_y;
+        const int y0 = ty * TH, x0 = tx * TW;
+        const float* xn = a.x + (size_t)n * a.H * a.W * a.C;
+        const float* dyn = a.dy + (size_t)n * a.H * a.W * a.K;
+
+        __syncthreads();
+        for (int id = tid; id < PIX * (CS / 4); id += CONV_THREADS) {
+            const int p = id / (CS / 4), q4 = (id % (CS / 4)) * 4;
+            const int gy = y0 + p / TW, gx = x0 + p % TW;
+            const int k = k0 + q4;
+            float4_t v = {0.f, 0.f, 0.f, 0.f};
+            if (gy < a.H && gx < a.W && k < a.K) {
+                const float* src = dyn + ((size_t)gy * a.W + gx) * a.K + k;
+                if (a.k_vec) {
+                    v = *(const float4_t*)src;
+                } else {
+#pragma unroll
+                    for (int j = 0; j < 4; ++j)
+                        if (k + j < a.K) v[j] = src[j];
+                }
+            }
+            *(float4_t*)(dy_tile + p * CS + q4) = v;
+        }
+        for (int id = tid; id < HALO * (CS / 4); id += CONV_THREADS) {
+            const int p = id / (CS / 4), q4 = (id % (CS / 4)) * 4;
+            const int gy = y0 + p / HW_ - 1, gx = x0 + p % HW_ - 1;
+            const int c = c0 + q4;
+            float4_t v = {0.f, 0.f, 0.f, 0.f};
+            if (gy >= 0 && gy < a.H && gx >= 0 && gx < a.W && c < a.C) {
+                const float* src = xn + ((size_t)gy * a.W + gx) * a.C + c;
+                if (a.c_vec) {
+                    v = *(const float4_t*)src;
+                } else {
+#pragma unroll
+                    for (int j = 0; j < 4; ++j)
+                        if (c + j < a.C) v[j] = src[j];
+                }
+            }
+            *(float4_t*)(x_tile + p * CS + q4) = v;
+        }
+        __syncthreads();
+        if (wave_active) {
+            // reduction over the tile's pixels, two per MFMA: lane-half h takes pixel 2*pp + h
+#pragma unroll 2
+            for (int pp = 0; pp < PIX / 2; ++pp) {
+                const int p = 2 * pp + h;
+                const float av = dy_tile[p * CS + kt * 32 + idx];
+                bsum += av;
+                const int xb = ((p / TW) * HW_ + (p % TW)) * CS + ct * 32 + idx;
+#pragma unroll
+                for (int t = 0; t < 9; ++t) {
+                    const float bv = x_tile[xb + ((t / 3) * HW_ + (t % 3)) * CS];
+                    acc[t] = __builtin_amdgcn_mfma_f32_32x32x2f32(av, bv, acc[t], 0, 0, 0);
+                }
+            }
+        }
+    }
+
+    // partial dW[k][tap][c]: accumulator element e of lane (idx,h) is row k = 8*(e/4)+4h+e%4, col c = idx
+    float* pw = a.part_w + (size_t)blockIdx.x * a.K * 9 * a.C;
+    const int c = c0 + ct * 32 + idx;
+    if (wave_active && c < a.C) {
+#pragma unroll
+        for (int t = 0; t < 9; ++t)
+#pragma unroll
+            for (int e = 0; e < 16; ++e) {
+                const int k = k0 + kt * 32 + 8 * (e / 4) + 4 * h + (e % 4);
+                if (k < a.K) pw[((size_t)k * 9 + t) * a.C + c] = acc[t][e];
+            }
+    }
+    if (a.part_b && blockIdx.z == 0 && ct == 0) {
+        // the two lane halves summed alternate pixels of the same out channel
+        const float other = __shfl_xor(bsum, 32, 64);
+        const int k = k0 + kt * 32 + idx;
+        if (h == 0 && k < a.K) a.part_b[(size_t)blockIdx.x * a.K + k] = bsum + other;
+    }
+}
+
+// out[i] = sum_b part[b][i]  (fixed order -> deterministic)
+__global__ __launch_bounds__(256) void reduce_partials_kernel(const float* __restrict__ part, float* __restrict__ out,
+                                                              int n_part, int n) {
+    const int i = blockIdx.x * 256 + threadIdx.x;
+    if (i >= n) return;
+    float s0 = 0.f, s1 = 0.f, s2 = 0.f, s3 = 0.f;
+    int b = 0;
+    for (; b + 3 < n_part; b += 4) {
+        s0 += part[(size_t)b * n + i];
+        s1 += part[(size_t)(b + 1) * n + i];
+        s2 += part[(size_t)(b + 2) * n + i];
+        s3 += part[(size_t)(b + 3) * n + i];
+    }
+    for (; b < n_part; ++b) s0 += part[(size_t)b * n + i];
+    out[i] = (s0 + s1) + (s2 + s3);
+}
+
+struct TileShape {
+    int th, tw;
+};
+
+// Pick the pixel tile that wastes the fewest MFMA rows on this image size.
+TileShape pick_tile(int H, int W) {
+    const TileShape cand[3] = {{16, 16}, {8, 32}, {32, 8}};
+    TileShape best = cand[0];
+    double best_eff = -1.0;
+    for (const TileShape& t : cand) {
+        const double th = (double)((H + t.th - 1) / t.th) * t.th;
+        const double tw = (double)((W + t.tw - 1) / t.tw) * t.tw;
+        const double eff = ((double)H * W) / (th * tw);
+        if (eff > best_eff + 1e-9) {
+            best_eff = eff;
+            best = t;
+        }
+    }
+    return best;
+}
+
+constexpr int WGRAD_TH = 8, WGRAD_TW = 16;
+constexpr int WGRAD_MAX_BLOCKS = 512;
+
+int wgrad_blocks(int N, int H, int W) {
+    const long tiles = (long)N * ((H + WGRAD_TH - 1) / WGRAD_TH) * ((W + WGRAD_TW - 1) / WGRAD_TW);
+    return (int)(tiles < WGRAD_MAX_BLOCKS ? tiles : WGRAD_MAX_BLOCKS);
+}
+
+int check_dims(const char* who, int N, int H, int W, int C, int K) {
+    PD_REQUIRE(N > 0 && H > 0 && W > 0 && C > 0 && K > 0, PD_ESHAPE, "%s: dimensions must be positive", who);
+    PD_REQUIRE((long)N * H * W * (C > K ? C : K) < (1L << 40), PD_ESHAPE, "%s: tensor too large", who);
+    return PD_OK;
+}
+
+}  // namespace
+
+extern "C" int pd_conv3x3_fwd_nhwc_f32(const float* x, const float* w, const float* bias, float* y, int N, int H,
+                                       int W, int C, int K, int relu, void* stream) {
+    int rc = check_dims("pd_conv3x3_fwd_nhwc_f32", N, H, W, C, K);
+    if (rc != PD_OK) return rc;
+    PD_REQUIRE(x && w && y, PD_EINVAL, "pd_conv3x3_fwd_nhwc_f32: NULL pointer");
+    ConvArgs a;
+    a.x = x; a.w = w; a.bias = bias; a.y = y;
+    a.N = N; a.H = H; a.W = W; a.C = C; a.K = K;
+    a.relu = relu != 0;
+    a.c_vec = (C % 4 == 0) && pd_aligned(x, 16) && pd_aligned(w, 16);
+    const TileShape t = pick_tile(H, W);
+    a.tiles_x = (W + t.tw - 1) / t.tw;
+    a.tiles_y = (H + t.th - 1) / t.th;
+    const long nblk = (long)N * a.tiles_x * a.tiles_y;
+    PD_REQUIRE(nblk <= 0x7fffffffL, PD_ESHAPE, "pd_conv3x3_fwd_nhwc_f32: too many tiles");
+    dim3 grid((unsigned)nblk, (K + BN - 1) / BN);
+    hipStream_t s = (hipStream_t)stream;
+    const bool small_c = C <= 8;
+#define PD_LAUNCH_FWD(TH_, TW_)                                                                        \
+    do {                                                                                               \
+        if (small_c) conv3x3_fwd_kernel<TH_, TW_, 8><<<grid, CONV_THREADS, 0, s>>>(a);                 \
+        else conv3x3_fwd_kernel<TH_, TW_, 16><<<grid, CONV_THREADS, 0, s>>>(a);                        \
+    } while (0)
+    if (t.tw == 16) PD_LAUNCH_FWD(16, 16);
+    else if (t.tw == 32) PD_LAUNCH_FWD(8, 32);
+    else PD_LAUNCH_FWD(32, 8);
+#undef PD_LAUNCH_FWD
+    PD_CHECK_LAUNCH("pd_conv3x3_fwd_nhwc_f32");
+    return PD_OK;
+}
+
+extern "C" int pd_conv3x3_filter_rot180_f32(const float* w, float* out, int K, int C, void* stream) {
+    PD_REQUIRE(K > 0 && C > 0, PD_ESHAPE, "pd_conv3x3_filter_rot180_f32: dimensions must be positive");
+    PD_REQUIRE(w && out && w != out, PD_EINVAL, "pd_conv3x3_filter_rot180_f32: NULL or aliased pointer");
+    const int total = K * 9 * C;
+    filter_rot180_kernel<<<dim3((total + 255) / 256), dim3(256), 0, (hipStream_t)stream>>>(w, out, K, C);
+    PD_CHECK_LAUNCH("pd_conv3x3_filter_rot180_f32");
+    return PD_OK;
+}
+
+extern "C" int pd_conv3x3_wgrad_workspace_bytes(int N, int H, int W, int C, int K, uint64_t* bytes) {
+    int rc = check_dims("pd_conv3x3_wgrad_workspace_bytes", N, H, W, C, K);
+    if (rc != PD_OK) return rc;
+    PD_REQUIRE(bytes != nullptr, PD_EINVAL, "pd_conv3x3_wgrad_workspace_bytes: NULL pointer");
+    const uint64_t nb = (uint64_t)wgrad_blocks(N, H, W);
+    *bytes = nb * ((uint64_t)K * 9 * C + (uint64_t)K) * sizeof(float);
+    return PD_OK;
+}
+
+extern "C" int pd_conv3x3_wgrad_nhwc_f32(const float* x, const float* dy, float* dw, float* dbias, void* workspace,
+                                         uint64_t workspace_bytes, int N, int H, int W, int C, int K, void* stream) {
+    int rc = check_dims("pd_conv3x3_wgrad_nhwc_f32", N, H, W, C, K);
+    if (rc != PD_OK) return rc;
+    PD_REQUIRE(x && dy && dw && workspace, PD_EINVAL, "pd_conv3x3_wgrad_nhwc_f32: NULL pointer");
+    uint64_t need = 0;
+    pd_conv3x3_wgrad_workspace_bytes(N, H, W, C, K, &need);
+    PD_REQUIRE(workspace_bytes >= need, PD_EINVAL, "pd_conv3x3_wgrad_nhwc_f32: workspace too small (%llu < %llu)",
+               (unsigned long long)workspace_bytes, (unsigned long long)need);
+    PD_REQUIRE(pd_aligned(workspace, 16), PD_EINVAL, "pd_conv3x3_wgrad_nhwc_f32: workspace must be 16-byte aligned");
+    WgradArgs a;
+    a.x = x; a.dy = dy;
+    a.N = N; a.H = H; a.W = W; a.C = C; a.K = K;
+    a.tiles_x = (W + WGRAD_TW - 1) / WGRAD_TW;
+    a.tiles_y = (H + WGRAD_TH - 1) / WGRAD_TH;
+    a.n_tiles = N * a.tiles_x * a.tiles_y;
+    const int nb = wgrad_blocks(N, H, W);
+    a.part_w = (float*)workspace;
+    a.part_b = dbias ? a.part_w + (size_t)nb * K * 9 * C : nullptr;
+    a.c_vec = (C % 4 == 0) && pd_aligned(x, 16);
+    a.k_vec = (K % 4 == 0) && pd_aligned(dy, 16);
+    hipStream_t s = (hipStream_t)stream;
+    dim3 grid(nb, (K + 63) / 64, (C + 63) / 64);
+    conv3x3_wgrad_kernel<WGRAD_TH, WGRAD_TW><<<grid, CONV_THREADS, 0, s>>>(a);
+    PD_CHECK_LAUNCH("pd_conv3x3_wgrad_nhwc_f32");
+    const int nw = K * 9 * C;
+    reduce_partials_kernel<<<dim3((nw + 255) / 256), dim3(256), 0, s>>>(a.part_w, dw, nb, nw);
+    PD_CHECK_LAUNCH("pd_conv3x3_wgrad_nhwc_f32(reduce)");
+    if (dbias) {
+        reduce_partials_kernel<<<dim3((K + 255) / 256), dim3(256), 0, s>>>(a.part_b, dbias, nb, K);
+        PD_CHECK_LAUNCH("pd_conv3x3_wgrad_nhwc_f32(reduce bias)");
+    }
+    return PD_OK;
+}

@@ -77,6 +77,62 @@ class Linear(torch.nn.Module):
 
 
 # --------------------------------------------------------------------------------------
+# Conv2d 3x3
+# --------------------------------------------------------------------------------------
+class _Conv3x3Fn(torch.autograd.Function):
+    @staticmethod
+    def forward(ctx, x, weight, bias, relu):
+        x = ops.to_nhwc(x)
+        y = ops.conv3x3_forward(x, weight, bias, relu)
+        ctx.relu = relu
+        ctx.has_bias = bias is not None
+        ctx.save_for_backward(x, weight, y if relu else None)
+        return y
+
+    @staticmethod
+    def backward(ctx, dy):
+        x, weight, y = ctx.saved_tensors
+        dy = ops.relu_backward(dy, y) if ctx.relu else ops.to_nhwc(dy)
+        dx = dw = db = None
+        if ctx.needs_input_grad[0]:
+            dx = ops.conv3x3_input_grad(dy, weight)
+        if ctx.needs_input_grad[1] or (ctx.has_bias and ctx.needs_input_grad[2]):
+            dw, db = ops.conv3x3_weight_grad(x, dy, with_bias=ctx.has_bias)
+        return dx, dw, db, None
+
+
+class Conv2d(torch.nn.Module):
+    """``torch.nn.Conv2d(in, out, kernel_size=3, stride=1, padding=1)`` (the only
+    convolution shape in the reference's VGG16 stages), optionally with the following
+    ReLU fused into the epilogue.  The weight has torch's logical shape [out, in, 3, 3]
+    and channels_last memory order; activations are kept in NHWC order."""
+
+    def __init__(self, in_channels, out_channels, kernel_size=3, stride=1, padding=1, bias=True, relu=False):
+        super(Conv2d, self).__init__()
+        norm = lambda v: tuple(v) if isinstance(v, (tuple, list)) else (v, v)
+        if norm(kernel_size) != (3, 3) or norm(stride) != (1, 1) or norm(padding) != (1, 1):
+            raise NotImplementedError("only Conv2d(kernel_size=3, stride=1, padding=1) has a HIP kernel")
+        self.in_channels = in_channels
+        self.out_channels = out_channels
+        self.relu = relu
+        w = torch.empty(out_channels, in_channels, 3, 3)
+        torch.nn.init.kaiming_uniform_(w, a=math.sqrt(5))
+        self.weight = torch.nn.Parameter(w.contiguous(memory_format=torch.channels_last))
+        if bias:
+            bound = 1 / math.sqrt(in_channels * 9)
+            self.bias = torch.nn.Parameter(torch.empty(out_channels).uniform_(-bound, bound))
+        else:
+            self.bias = None
+
+    def forward(self, x):
+        return _Conv3x3Fn.apply(x, self.weight, self.bias, self.relu)
+
+    def extra_repr(self):
+        return "{}, {}, kernel_size=(3, 3), stride=(1, 1), padding=(1, 1), relu={}".format(
+            self.in_channels, self.out_channels, self.relu)
+
+
+# --------------------------------------------------------------------------------------
 # ReLU / MaxPool
 # --------------------------------------------------------------------------------------
 class _ReLUFn(torch.autograd.Function):

@@ -177,3 +177,67 @@ def cross_entropy_backward(logits, target, lse, count, grad_loss, ignore_index=-
     _cabi.lib().pd_xent_bwd_f32(_ptr(logits), _ptr(target), _ptr(lse), _ptr(grad_loss), _ptr(count), _ptr(d),
                                 B, C, ld, C, int(ignore_index), _cabi.stream_ptr())
     return d
+
+
+# --------------------------------------------------------------------------------------
+# 3x3 convolution (stride 1, padding 1), NHWC activations, KRSC filter
+# --------------------------------------------------------------------------------------
+def _filter_dims(w):
+    _check(w, "weight")
+    if w.dim() != 4 or w.shape[2:] != (3, 3):
+        raise ValueError("conv3x3: weight must be [K, C, 3, 3], got %s" % (tuple(w.shape),))
+    if not w.is_contiguous(memory_format=torch.channels_last):
+        raise ValueError("conv3x3: weight must be in channels_last (K,R,S,C) memory order")
+    return w.shape[0], w.shape[1]
+
+
+def conv3x3_forward(x, w, bias=None, relu=False):
+    """y = conv2d(x, w, bias, stride 1, padding 1) (+ReLU).  x: NHWC-ordered [N,C,H,W]."""
+    _check(x, "x")
+    n, h, wd, c = _nhwc_dims(x)
+    k, cw = _filter_dims(w)
+    if cw != c:
+        raise ValueError("conv3x3: input has %d channels, filter expects %d" % (c, cw))
+    if bias is not None:
+        _check(bias, "bias")
+        if bias.numel() != k or not bias.is_contiguous():
+            raise ValueError("conv3x3: bias must be a contiguous vector of K=%d" % k)
+    y = torch.empty((n, k, h, wd), dtype=torch.float32, device=x.device, memory_format=torch.channels_last)
+    _cabi.lib().pd_conv3x3_fwd_nhwc_f32(_ptr(x), _ptr(w), _ptr(bias), _ptr(y), n, h, wd, c, k, int(relu),
+                                        _cabi.stream_ptr())
+    return y
+
+
+def conv3x3_input_grad(dy, w):
+    """dx of conv3x3_forward: the forward kernel on dy with the 180-degree-rotated filter."""
+    _check(dy, "dy")
+    n, h, wd, k = _nhwc_dims(dy)
+    kw, c = _filter_dims(w)
+    if kw != k:
+        raise ValueError("conv3x3_input_grad: dy has %d channels, filter has %d outputs" % (k, kw))
+    lib = _cabi.lib()
+    # rotated filter: logical [C, K, 3, 3] in channels_last order = memory [C][3][3][K]
+    wr = torch.empty((c, k, 3, 3), dtype=torch.float32, device=w.device, memory_format=torch.channels_last)
+    lib.pd_conv3x3_filter_rot180_f32(_ptr(w), _ptr(wr), k, c, _cabi.stream_ptr())
+    dx = torch.empty((n, c, h, wd), dtype=torch.float32, device=dy.device, memory_format=torch.channels_last)
+    lib.pd_conv3x3_fwd_nhwc_f32(_ptr(dy), _ptr(wr), None, _ptr(dx), n, h, wd, k, c, 0, _cabi.stream_ptr())
+    return dx
+
+
+def conv3x3_weight_grad(x, dy, with_bias=True):
+    """(dw [K,C,3,3] channels_last, dbias [K] or None)."""
+    _check(x, "x")
+    _check(dy, "dy")
+    n, h, wd, c = _nhwc_dims(x)
+    n2, h2, w2, k = _nhwc_dims(dy)
+    if (n, h, wd) != (n2, h2, w2):
+        raise ValueError("conv3x3_weight_grad: x %s and dy %s disagree" % (tuple(x.shape), tuple(dy.shape)))
+    lib = _cabi.lib()
+    nbytes = ctypes.c_uint64()
+    lib.pd_conv3x3_wgrad_workspace_bytes(n, h, wd, c, k, ctypes.byref(nbytes))
+    ws = torch.empty(nbytes.value, dtype=torch.uint8, device=x.device)
+    dw = torch.empty((k, c, 3, 3), dtype=torch.float32, device=x.device, memory_format=torch.channels_last)
+    db = torch.empty(k, dtype=torch.float32, device=x.device) if with_bias else None
+    lib.pd_conv3x3_wgrad_nhwc_f32(_ptr(x), _ptr(dy), _ptr(dw), _ptr(db), _ptr(ws), nbytes.value, n, h, wd, c, k,
+                                  _cabi.stream_ptr())
+    return dw, db

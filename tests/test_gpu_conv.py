@@ -1,0 +1,148 @@
+"""3x3 convolution kernels (forward, input gradient, weight/bias gradient) through the C
+ABI against the torch CPU library (the third-party routine the reference's Conv2d layers
+call) in fp64, plus a brute-force direct convolution on a tiny case that pins the index
+conventions (tap order, padding, which operand is flipped).
+
+Tolerance: fp32 accumulation over R terms against an fp64 result: rtol 1e-5 plus
+atol = 4e-7 * sqrt(R) * (typical |term| sum scale) as set per test."""
+import math
+
+import numpy as np
+import pytest
+import torch
+import torch.nn.functional as F
+
+from pipedream_amd import layers, ops
+
+pytestmark = pytest.mark.gpu
+
+
+def _nhwc(t):
+    return t.cuda().contiguous(memory_format=torch.channels_last)
+
+
+def _direct_conv(x, w, b):
+    """Brute-force NCHW 3x3 / pad 1 convolution in numpy float64."""
+    N, C, H, W = x.shape
+    K = w.shape[0]
+    xp = np.zeros((N, C, H + 2, W + 2))
+    xp[:, :, 1:-1, 1:-1] = x
+    y = np.zeros((N, K, H, W))
+    for n in range(N):
+        for k in range(K):
+            for yy in range(H):
+                for xx in range(W):
+                    y[n, k, yy, xx] = (xp[n, :, yy:yy + 3, xx:xx + 3] * w[k]).sum() + b[k]
+    return y
+
+
+def test_forward_against_brute_force():
+    rng = np.random.RandomState(0)
+    x = rng.randn(2, 3, 5, 7)
+    w = rng.randn(4, 3, 3, 3)
+    b = rng.randn(4)
+    want = _direct_conv(x, w, b)
+    got = ops.conv3x3_forward(_nhwc(torch.tensor(x, dtype=torch.float32)),
+                              _nhwc(torch.tensor(w, dtype=torch.float32)),
+                              torch.tensor(b, dtype=torch.float32).cuda())
+    np.testing.assert_allclose(got.cpu().numpy(), want, rtol=1e-5, atol=1e-5)
+    # the torch library agrees with the brute force, so it can serve as the oracle below
+    lib = F.conv2d(torch.tensor(x), torch.tensor(w), torch.tensor(b), padding=1)
+    np.testing.assert_allclose(lib.numpy(), want, rtol=1e-10, atol=1e-10)
+
+
+SHAPES = [
+    # N, C, K, H, W
+    (2, 3, 64, 32, 32),      # first VGG layer: 3 input channels
+    (2, 64, 64, 32, 48),
+    (1, 64, 128, 28, 28),    # ragged tiles
+    (2, 128, 128, 14, 14),
+    (1, 16, 32, 9, 5),       # fewer channels than a block, odd sizes
+    (1, 8, 8, 1, 1),
+    (1, 20, 70, 17, 33),     # channel counts that are not multiples of the tile
+    (3, 5, 6, 8, 8),         # C not a multiple of 4: scalar load path
+]
+
+
+@pytest.mark.parametrize("N,C,K,H,W", SHAPES)
+def test_forward_backward_vs_library(N, C, K, H, W):
+    g = torch.Generator().manual_seed(N * 1000 + C)
+    x = torch.randn(N, C, H, W, generator=g)
+    w = torch.randn(K, C, 3, 3, generator=g) / math.sqrt(9 * C)
+    b = torch.randn(K, generator=g)
+    dy = torch.randn(N, K, H, W, generator=g)
+    xd, wd, bd = x.double().requires_grad_(), w.double().requires_grad_(), b.double().requires_grad_()
+    y_ref = F.conv2d(xd, wd, bd, padding=1)
+    y_ref.backward(dy.double())
+
+    xg, wg = _nhwc(x), _nhwc(w)
+    y = ops.conv3x3_forward(xg, wg, b.cuda())
+    assert y.is_contiguous(memory_format=torch.channels_last)
+    torch.testing.assert_close(y.cpu().double(), y_ref.detach(), rtol=1e-5, atol=4e-7 * math.sqrt(9 * C) * 4)
+    dx = ops.conv3x3_input_grad(_nhwc(dy), wg)
+    torch.testing.assert_close(dx.cpu().double(), xd.grad, rtol=1e-5, atol=4e-7 * math.sqrt(9 * K) * 4)
+    dw, db = ops.conv3x3_weight_grad(xg, _nhwc(dy))
+    R = N * H * W
+    torch.testing.assert_close(dw.cpu().double(), wd.grad, rtol=1e-5, atol=4e-7 * math.sqrt(R) * 4)
+    torch.testing.assert_close(db.cpu().double(), bd.grad, rtol=1e-5, atol=4e-7 * math.sqrt(R) * 4)
+
+
+def test_fused_relu_and_no_bias():
+    g = torch.Generator().manual_seed(7)
+    x = torch.randn(2, 16, 12, 12, generator=g)
+    w = torch.randn(24, 16, 3, 3, generator=g) / 12
+    y = ops.conv3x3_forward(_nhwc(x), _nhwc(w), None, relu=True)
+    want = F.conv2d(x.double(), w.double(), None, padding=1).clamp_min(0)
+    torch.testing.assert_close(y.cpu().double(), want, rtol=1e-5, atol=1e-5)
+    dw, db = ops.conv3x3_weight_grad(_nhwc(x), y, with_bias=False)
+    assert db is None
+
+
+def test_identity_filter_is_exact():
+    # a centre-tap identity filter must reproduce the input bit for bit
+    x = torch.randn(2, 32, 20, 20)
+    w = torch.zeros(32, 32, 3, 3)
+    for c in range(32):
+        w[c, c, 1, 1] = 1.0
+    y = ops.conv3x3_forward(_nhwc(x), _nhwc(w))
+    assert torch.equal(y.cpu(), x)
+    # shifting filter: tap (r=0,s=2) reads x[y-1, x+1]
+    w = torch.zeros(32, 32, 3, 3)
+    for c in range(32):
+        w[c, c, 0, 2] = 1.0
+    y = ops.conv3x3_forward(_nhwc(x), _nhwc(w)).cpu()
+    want = torch.zeros_like(x)
+    want[:, :, 1:, :-1] = x[:, :, :-1, 1:]
+    assert torch.equal(y, want)
+
+
+def test_conv_layer_module_matches_torch_nn():
+    torch.manual_seed(11)
+    ref = torch.nn.Conv2d(8, 16, 3, padding=1)
+    mine = layers.Conv2d(8, 16, relu=True)
+    mine.load_state_dict(ref.state_dict())
+    assert mine.weight.is_contiguous(memory_format=torch.channels_last)
+    mine = mine.cuda()
+    x = torch.randn(2, 8, 10, 10, requires_grad=True)
+    xg = x.detach().cuda().requires_grad_(True)
+    y_ref = torch.relu(ref(x))
+    y = mine(xg)
+    torch.testing.assert_close(y.cpu(), y_ref.detach(), rtol=1e-5, atol=1e-5)
+    dy = torch.randn(y_ref.shape)
+    y_ref.backward(dy)
+    y.backward(dy.cuda())
+    torch.testing.assert_close(xg.grad.cpu(), x.grad, rtol=1e-5, atol=1e-5)
+    torch.testing.assert_close(mine.weight.grad.cpu(), ref.weight.grad, rtol=1e-5, atol=1e-5)
+    torch.testing.assert_close(mine.bias.grad.cpu(), ref.bias.grad, rtol=1e-5, atol=1e-5)
+    assert list(mine.state_dict().keys()) == list(ref.state_dict().keys())
+
+
+def test_conv_rejects_bad_operands():
+    x = torch.randn(1, 4, 6, 6).cuda()           # NCHW memory order
+    w = _nhwc(torch.randn(8, 4, 3, 3))
+    with pytest.raises(ValueError, match="NHWC"):
+        ops.conv3x3_forward(x, w)
+    with pytest.raises(ValueError, match="channels"):
+        ops.conv3x3_forward(_nhwc(torch.randn(1, 5, 6, 6)), w)
+    with pytest.raises(NotImplementedError):
+        layers.Conv2d(4, 8, kernel_size=5, padding=2)
