@@ -1,0 +1,243 @@
+#!/usr/bin/env python3
+"""Headline benchmark: samples/s of one PipeDream stage's steady-state 1F1B step
+(forward + backward + stashed SGD update) on one MI355X.
+
+Workload (N=1): VGG16 conv1_1..pool2, batch 64 fp32, synthetic N(0,1) images, He-normal
+weights, weight-stash depth 4 (3 warm-up forwards in flight), SGD momentum 0.9 lr 0.01
+wd 5e-4; the stage is driven through StageRuntime / SGDWithWeightStashing and this script
+plays its downstream neighbour (consumes the sent activation, queues a synthetic upstream
+gradient ~ N(0,1)*1e-3).  All inputs are resident in HBM before the timed region.
+
+Prints ONE JSON line (see the keys below).  `roofline` covers the dominant kernel, the
+MFMA fp32 3x3 convolution (`conv3x3_fwd_kernel<.,.,16>`, used for forward and input
+gradient): algorithmic flop of its launches in the timed region / their summed duration,
+both measured with HIP events around every launch on the launch stream.
+`cpu_baseline` times the CPU oracle (torch.nn on the host cores) on a bounded sample of
+the same workload.
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+BATCH = 64
+STASH_DEPTH = 4
+SGD_KW = dict(lr=0.01, momentum=0.9, weight_decay=5e-4)
+PEAK_FP32_MFMA_TFLOPS = 157.3
+
+
+def build_stage():
+    import torch
+    from pipedream_amd import handoff, runtime, sgd
+    from pipedream_amd.layers import CrossEntropyLoss
+    from pipedream_amd.stages import vgg16
+
+    handoff.reset_fabrics()
+    torch.manual_seed(0)
+
+    class Rest(torch.nn.Module):     # placeholder for the stages that follow; never run
+        def forward(self, x):
+            raise RuntimeError("downstream stages are played by the benchmark")
+
+    model = [(vgg16.FrontStage(), ["input0"], ["out0"]), (Rest(), ["out0"], ["out1"]),
+             (CrossEntropyLoss(), ["out1"], ["loss"])]
+    shapes = {"input0": (BATCH, 3, 224, 224), "target": (BATCH,), "out0": (BATCH, 128, 56, 56)}
+    dtypes = {"input0": torch.float32, "target": torch.int64, "out0": torch.float32}
+    r = runtime.StageRuntime(
+        model=model, distributed_backend="gloo", fp16=False, loss_scale=1.0,
+        training_tensor_shapes=shapes, eval_tensor_shapes=dict(shapes), training_tensor_dtypes=dtypes,
+        inputs_module_destinations={"input": 0}, target_tensor_names={"target"},
+        configuration_maps={"module_to_stage_map": [0, 1, 1], "stage_to_rank_map": {"0": [0], "1": [1]},
+                            "stage_to_depth_map": {"0": STASH_DEPTH - 1, "1": 0}},
+        master_addr="127.0.0.1", rank=0, local_rank=0, num_ranks_in_server=2, verbose_freq=0,
+        model_type=runtime.IMAGE_CLASSIFICATION)
+    opt = sgd.SGDWithWeightStashing(r.modules(), r.master_parameters, r.model_parameters, 1.0,
+                                    num_versions=r.num_warmup_minibatches + 1, **SGD_KW)
+    return r, opt
+
+
+class Downstream(object):
+    """The next stage as seen from the hand-off queues."""
+
+    def __init__(self, r, grads):
+        self.fabric = r.comm_handler.fabric
+        self.grads = grads
+        self.i = 0
+
+    def after_forward(self):
+        self.fabric.queue("out0", 1, False).popleft()
+        self.fabric.queue("target", 1, False).popleft()
+        self.fabric.queue("out0", 0, True).append(self.grads[self.i % len(self.grads)])
+        self.i += 1
+
+
+def gpu_run(steps, warmup):
+    import torch
+    from pipedream_amd import ops
+
+    r, opt = build_stage()
+    g = torch.Generator().manual_seed(0)
+    n_data = 4
+    images = [torch.randn(BATCH, 3, 224, 224, generator=g).cuda().contiguous(memory_format=torch.channels_last)
+              for _ in range(n_data)]
+    targets = [torch.randint(0, 1000, (BATCH,), generator=g).cuda() for _ in range(n_data)]
+    grads = [(torch.randn(BATCH, 128, 56, 56, generator=g) * 1e-3).cuda().contiguous(
+        memory_format=torch.channels_last) for _ in range(n_data)]
+
+    def loader():
+        i = 0
+        while True:
+            yield images[i % n_data], targets[i % n_data]
+            i += 1
+
+    total = warmup + steps + r.num_warmup_minibatches
+    r.train(total)
+    r.set_loader(loader())
+    down = Downstream(r, grads)
+
+    def forward():
+        r.run_forward()
+        down.after_forward()
+
+    def step():
+        forward()
+        opt.zero_grad()
+        opt.load_old_params()
+        r.run_backward()
+        opt.load_new_params()
+        opt.step()
+
+    for _ in range(r.num_warmup_minibatches):     # fill the pipeline: 3 forwards in flight
+        forward()
+    for _ in range(warmup):
+        step()
+    torch.cuda.synchronize()
+    ops.kernel_timer = {}
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        step()
+    torch.cuda.synchronize()
+    elapsed = time.perf_counter() - t0
+    timer, ops.kernel_timer = ops.kernel_timer, None
+
+    stats = {}
+    for name, recs in timer.items():
+        ms = sum(s.elapsed_time(e) for s, e, _ in recs)
+        stats[name] = {"launches": len(recs), "avg_us": 1e3 * ms / len(recs),
+                       "work_per_launch": sum(w for _, _, w in recs) / len(recs),
+                       "rate": sum(w for _, _, w in recs) / (ms * 1e-3)}
+    done = warmup + steps
+    assert opt.queue.versions() == [done - (STASH_DEPTH - 1) + i for i in range(STASH_DEPTH)], opt.queue.versions()
+    return elapsed, stats, opt
+
+
+def optimizer_bandwidth():
+    """Fused stash+SGD step on a VGG16-sized flat parameter set (138 357 544 fp32 values,
+    20 algorithmic bytes each), timed with HIP events on the launch stream."""
+    import torch
+    from pipedream_amd import _cabi
+    n = 138357544
+    t = [torch.randn(n, device="cuda") for _ in range(3)]
+    out = torch.empty(n, device="cuda")
+    d = (_cabi.TensorDesc * 1)()
+    d[0].grad, d[0].p_in, d[0].p_out = t[0].data_ptr(), t[1].data_ptr(), out.data_ptr()
+    d[0].state0, d[0].state1, d[0].bf16_out, d[0].n = t[2].data_ptr(), None, None, n
+    lib, s = _cabi.lib(), _cabi.stream_ptr()
+    run = lambda: lib.pd_sgd_step(d, 1, 0.01, 0.9, 0.0, 5e-4, 0, 0, 1.0, 1.0, s)
+    for _ in range(3):
+        run()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    reps = 20
+    e0.record()
+    for _ in range(reps):
+        run()
+    e1.record()
+    torch.cuda.synchronize()
+    sec = e0.elapsed_time(e1) * 1e-3 / reps
+    return {"kernel": "pd_optim_kernel<SGD>", "params": n, "bytes_per_param": 20, "avg_us": sec * 1e6,
+            "achieved_GBps": 20.0 * n / sec / 1e9, "peak_GBps": 8000.0, "frac": 20.0 * n / sec / 1e9 / 8000.0}
+
+
+def cpu_baseline(timed_steps=2):
+    """The CPU oracle (torch.nn modules, state_dict-copy weight stashing, torch.optim.SGD)
+    on the same workload: 1 warm-up + `timed_steps` steady-state steps at batch 64."""
+    import torch
+    from oracle import models, stash_oracle
+    torch.manual_seed(0)
+    m = models.VggFrontStage()
+    opt = stash_oracle.StashingOptimizerOracle("SGD", [m], m.parameters(), STASH_DEPTH, **SGD_KW)
+    g = torch.Generator().manual_seed(0)
+    x = torch.randn(BATCH, 3, 224, 224, generator=g)
+    grad = torch.randn(BATCH, 128, 56, 56, generator=g) * 1e-3
+    pending = [m(x) for _ in range(STASH_DEPTH - 1)]
+
+    def step():
+        pending.append(m(x))
+        opt.zero_grad()
+        opt.load_old_params()
+        pending.pop(0).backward(grad)
+        opt.load_new_params()
+        opt.step()
+
+    step()
+    t0 = time.perf_counter()
+    for _ in range(timed_steps):
+        step()
+    sec = (time.perf_counter() - t0) / timed_steps
+    return {"value": BATCH / sec, "unit": "samples/s", "cores": torch.get_num_threads(), "kind": "port",
+            "sample": "%d steady-state steps at batch 64 after 1 warm-up step (%.1f s/step)" % (timed_steps, sec)}
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        sys.exit("bench.py: this build measures one GPU only (one stage's share of the pipeline at its "
+                 "real shape); --gpus %d is not supported" % args.gpus)
+    import torch
+    if not torch.cuda.is_available():
+        sys.exit("bench.py: no HIP device; the product path has no CPU fallback")
+
+    elapsed, stats, _ = gpu_run(args.steps, args.warmup)
+    conv = stats["conv3x3_fwd_kernel"]
+    achieved = conv["rate"] / 1e12
+    out = {
+        "metric": "samples/sec per stage (fwd+bwd+stashed update), VGG16 bs64; optimizer HBM GB/s",
+        "value": BATCH * args.steps / elapsed,
+        "unit": "samples/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": 1e3 * elapsed / args.steps,
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "f32",
+        "data": "synthetic",
+        "config": {"workload": "VGG16 stage 0 (conv1_1..pool2), batch 64, fp32, stash depth 4, SGD momentum 0.9, "
+                               "1F1B with 4 minibatches in flight",
+                   "global_batch": BATCH, "parallelism": "1 stage on 1 GPU"},
+        "roofline": {"bound": "mfma", "achieved": achieved, "peak": PEAK_FP32_MFMA_TFLOPS, "unit": "TFLOP/s",
+                     "frac": achieved / PEAK_FP32_MFMA_TFLOPS, "traffic": None,
+                     "kernel": "conv3x3_fwd_kernel<.,.,16> (forward + input gradient)",
+                     "launches": conv["launches"], "avg_us": conv["avg_us"],
+                     "flop_per_launch": conv["work_per_launch"]},
+        "kernels": {k: {"launches": v["launches"], "avg_us": round(v["avg_us"], 1),
+                        "TFLOP/s": round(v["rate"] / 1e12, 2)} for k, v in stats.items()},
+        "optimizer_hbm": optimizer_bandwidth(),
+    }
+    if not args.no_cpu_baseline:
+        out["cpu_baseline"] = cpu_baseline()
+    print(json.dumps(out))
+
+
+if __name__ == "__main__":
+    main()

@@ -144,10 +144,16 @@ int pd_colsum_f32(const float* x, float* out, uint64_t M, int N, uint64_t ld, in
 int pd_relu_fwd_f32(const float* x, float* y, uint64_t n, void* stream);
 int pd_relu_bwd_f32(const float* dy, const float* y, float* dx, uint64_t n, void* stream);
 
+/* torch.nn.Dropout (stage3.py:20,23) given its keep-mask (one byte per element, 0/1):
+ * y = mask ? x*scale : 0, scale = 1/(1-p); the same call applied to dy is the backward. */
+int pd_mask_scale_f32(const float* x, const uint8_t* mask, float* y, uint64_t n, float scale, void* stream);
+
 /* torch.nn.MaxPool2d(kernel_size=2, stride=2) on NHWC tensors (stage1.py:11).
- * y is [N, H/2, W/2, C].  Backward writes all of dx; first maximum wins ties.
- * relu_mask != 0 additionally zeroes dx where x <= 0 (fused ReLU backward). */
-int pd_maxpool2x2_fwd_nhwc_f32(const float* x, float* y, int N, int H, int W, int C, void* stream);
+ * y is [N, H/2, W/2, C].  relu != 0 applies a ReLU to the pooled value, which equals
+ * pooling a ReLU'd input (the ReLU + MaxPool2d pair at the head of stage1.py:10-11).
+ * Backward writes all of dx; first maximum wins ties.
+ * relu_mask != 0 additionally zeroes dx where the window maximum is <= 0. */
+int pd_maxpool2x2_fwd_nhwc_f32(const float* x, float* y, int N, int H, int W, int C, int relu, void* stream);
 int pd_maxpool2x2_bwd_nhwc_f32(const float* x, const float* dy, float* dx, int N, int H, int W, int C,
                                int relu_mask, void* stream);
 

@@ -35,3 +35,118 @@ class MlpStage1(torch.nn.Module):
 
     def forward(self, input0):
         return self.layer3(input0)
+
+
+# --------------------------------------------------------------------------------------
+# VGG16 (layer lists of vgg16/gpus=4_straight/stage0-3.py and vgg16/gpus=2/stage0.py)
+# --------------------------------------------------------------------------------------
+def _vgg_init(module):
+    """stage0.py:22-33"""
+    for m in module.modules():
+        if isinstance(m, torch.nn.Conv2d):
+            torch.nn.init.kaiming_normal_(m.weight, mode='fan_out', nonlinearity='relu')
+            if m.bias is not None:
+                torch.nn.init.constant_(m.bias, 0)
+        elif isinstance(m, torch.nn.Linear):
+            torch.nn.init.normal_(m.weight, 0, 0.01)
+            torch.nn.init.constant_(m.bias, 0)
+
+
+def _conv(cin, cout):
+    return torch.nn.Conv2d(cin, cout, kernel_size=(3, 3), stride=(1, 1), padding=(1, 1))
+
+
+class VggFrontStage(torch.nn.Module):
+    """conv1_1 .. pool2"""
+
+    def __init__(self):
+        super(VggFrontStage, self).__init__()
+        self.layer2 = _conv(3, 64)
+        self.layer4 = _conv(64, 64)
+        self.layer7 = _conv(64, 128)
+        self.layer9 = _conv(128, 128)
+        _vgg_init(self)
+
+    def forward(self, x):
+        F = torch.nn.functional
+        x = F.relu(self.layer4(F.relu(self.layer2(x))))
+        x = F.max_pool2d(x, 2, 2)
+        x = F.relu(self.layer9(F.relu(self.layer7(x))))
+        return F.max_pool2d(x, 2, 2)
+
+
+class VggStage0(torch.nn.Module):
+    def __init__(self):
+        super(VggStage0, self).__init__()
+        self.layer2 = _conv(3, 64)
+        self.layer4 = _conv(64, 64)
+        _vgg_init(self)
+
+    def forward(self, x):
+        return self.layer4(torch.relu(self.layer2(x)))
+
+
+class VggStage1(torch.nn.Module):
+    def __init__(self):
+        super(VggStage1, self).__init__()
+        self.layer3 = _conv(64, 128)
+        self.layer5 = _conv(128, 128)
+        self.layer8 = _conv(128, 256)
+        _vgg_init(self)
+
+    def forward(self, x):
+        F = torch.nn.functional
+        x = F.max_pool2d(F.relu(x), 2, 2)
+        x = F.relu(self.layer5(F.relu(self.layer3(x))))
+        return F.relu(self.layer8(F.max_pool2d(x, 2, 2)))
+
+
+class VggStage2(torch.nn.Module):
+    def __init__(self):
+        super(VggStage2, self).__init__()
+        self.layer1 = _conv(256, 256)
+        self.layer3 = _conv(256, 256)
+        self.layer6 = _conv(256, 512)
+        self.layer8 = _conv(512, 512)
+        self.layer10 = _conv(512, 512)
+        _vgg_init(self)
+
+    def forward(self, x):
+        F = torch.nn.functional
+        x = F.relu(self.layer3(F.relu(self.layer1(x))))
+        x = F.max_pool2d(x, 2, 2)
+        return F.relu(self.layer10(F.relu(self.layer8(F.relu(self.layer6(x))))))
+
+
+class VggStage3(torch.nn.Module):
+    """``masks``: optional callable (name, tensor) -> 0/1 keep-mask, so that a parity run can
+    feed both sides the same dropout masks; without it dropout is torch's own."""
+
+    def __init__(self, dropout=0.5, num_classes=1000, masks=None):
+        super(VggStage3, self).__init__()
+        self.layer2 = _conv(512, 512)
+        self.layer4 = _conv(512, 512)
+        self.layer6 = _conv(512, 512)
+        self.layer11 = torch.nn.Linear(25088, 4096)
+        self.layer14 = torch.nn.Linear(4096, 4096)
+        self.layer17 = torch.nn.Linear(4096, num_classes)
+        self.p = dropout
+        self.masks = masks
+        _vgg_init(self)
+
+    def _drop(self, name, x):
+        if not self.training or self.p == 0:
+            return x
+        if self.masks is None:
+            return torch.nn.functional.dropout(x, self.p, True)
+        return x * self.masks(name, x).to(x.dtype) * (1.0 / (1.0 - self.p))
+
+    def forward(self, x):
+        F = torch.nn.functional
+        x = F.max_pool2d(x, 2, 2)
+        x = F.relu(self.layer6(F.relu(self.layer4(F.relu(self.layer2(x))))))
+        x = F.max_pool2d(x, 2, 2)
+        x = x.reshape(x.size(0), -1)
+        x = self._drop("layer13", F.relu(self.layer11(x)))
+        x = self._drop("layer16", F.relu(self.layer14(x)))
+        return self.layer17(x)

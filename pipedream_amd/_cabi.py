@@ -66,7 +66,8 @@ SIGNATURES = {
     "pd_colsum_f32": (_i, [_vp, _vp, _u64, _i, _u64, _i, _f, _vp], True),
     "pd_relu_fwd_f32": (_i, [_vp, _vp, _u64, _vp], True),
     "pd_relu_bwd_f32": (_i, [_vp, _vp, _vp, _u64, _vp], True),
-    "pd_maxpool2x2_fwd_nhwc_f32": (_i, [_vp, _vp, _i, _i, _i, _i, _vp], True),
+    "pd_mask_scale_f32": (_i, [_vp, _vp, _vp, _u64, _f, _vp], True),
+    "pd_maxpool2x2_fwd_nhwc_f32": (_i, [_vp, _vp, _i, _i, _i, _i, _i, _vp], True),
     "pd_maxpool2x2_bwd_nhwc_f32": (_i, [_vp, _vp, _vp, _i, _i, _i, _i, _i, _vp], True),
     "pd_xent_fwd_f32": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i64, _vp], True),
     "pd_conv3x3_fwd_nhwc_f32": (_i, [_vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _vp], True),

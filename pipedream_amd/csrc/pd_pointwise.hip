@@ -47,6 +47,14 @@ __global__ __launch_bounds__(PW_THREADS) void relu_bwd_kernel(const float* __res
     }
 }
 
+// ---- dropout: y = x * mask * scale (mask is 0/1 bytes) --------------------------------
+__global__ __launch_bounds__(PW_THREADS) void mask_scale_kernel(const float* __restrict__ x,
+                                                                const uint8_t* __restrict__ mask,
+                                                                float* __restrict__ y, uint64_t n, float scale) {
+    uint64_t i = (uint64_t)blockIdx.x * PW_THREADS + threadIdx.x;
+    if (i < n) y[i] = mask[i] ? x[i] * scale : 0.f;
+}
+
 // ---- 2x2 / stride-2 max pooling, NHWC ---------------------------------------------
 // One thread handles 4 consecutive channels of one output pixel.  Ties go to the first
 // maximum in window scan order (dy=0,dx=0 -> 0,1 -> 1,0 -> 1,1) and NaNs win, which is
@@ -54,7 +62,7 @@ __global__ __launch_bounds__(PW_THREADS) void relu_bwd_kernel(const float* __res
 __device__ __forceinline__ bool pool_better(float v, float best) { return v > best || v != v; }
 
 __global__ __launch_bounds__(PW_THREADS) void maxpool2_fwd_kernel(const float* __restrict__ x, float* __restrict__ y,
-                                                                  int N, int H, int W, int C) {
+                                                                  int N, int H, int W, int C, int relu) {
     const int Ho = H / 2, Wo = W / 2, C4 = C / 4;
     uint64_t id = (uint64_t)blockIdx.x * PW_THREADS + threadIdx.x;
     uint64_t total = (uint64_t)N * Ho * Wo * C4;
@@ -75,6 +83,8 @@ __global__ __launch_bounds__(PW_THREADS) void maxpool2_fwd_kernel(const float* _
         if (pool_better(v1[k], best[k])) best[k] = v1[k];
         if (pool_better(v2[k], best[k])) best[k] = v2[k];
         if (pool_better(v3[k], best[k])) best[k] = v3[k];
+        // ReLU commutes with max: relu(max(window)) == max(relu(window))
+        if (relu && best[k] < 0.f) best[k] = 0.f;
     }
     *(float4_t*)(y + (((uint64_t)n * Ho + oy) * Wo + ox) * C + c4 * 4) = best;
 }
@@ -279,7 +289,18 @@ extern "C" int pd_relu_bwd_f32(const float* dy, const float* y, float* dx, uint6
     return PD_OK;
 }
 
-extern "C" int pd_maxpool2x2_fwd_nhwc_f32(const float* x, float* y, int N, int H, int W, int C, void* stream) {
+extern "C" int pd_mask_scale_f32(const float* x, const uint8_t* mask, float* y, uint64_t n, float scale, void* stream) {
+    if (n == 0) return PD_OK;
+    PD_REQUIRE(x && mask && y, PD_EINVAL, "pd_mask_scale_f32: NULL pointer");
+    unsigned blocks;
+    PD_REQUIRE(blocks_for(n, &blocks) == 0, PD_ESHAPE, "pd_mask_scale_f32: too large");
+    mask_scale_kernel<<<dim3(blocks), dim3(PW_THREADS), 0, (hipStream_t)stream>>>(x, mask, y, n, scale);
+    PD_CHECK_LAUNCH("pd_mask_scale_f32");
+    return PD_OK;
+}
+
+extern "C" int pd_maxpool2x2_fwd_nhwc_f32(const float* x, float* y, int N, int H, int W, int C, int relu,
+                                          void* stream) {
     PD_REQUIRE(N >= 0 && H >= 0 && W >= 0 && C >= 0, PD_ESHAPE, "pd_maxpool2x2_fwd: negative dimension");
     PD_REQUIRE(C % 4 == 0, PD_ESHAPE, "pd_maxpool2x2_fwd: channels must be a multiple of 4 (got %d)", C);
     uint64_t total = (uint64_t)N * (H / 2) * (W / 2) * (C / 4);
@@ -288,7 +309,7 @@ extern "C" int pd_maxpool2x2_fwd_nhwc_f32(const float* x, float* y, int N, int H
     PD_REQUIRE(pd_aligned(x, 16) && pd_aligned(y, 16), PD_EINVAL, "pd_maxpool2x2_fwd: pointers must be 16-byte aligned");
     unsigned blocks;
     PD_REQUIRE(blocks_for(total, &blocks) == 0, PD_ESHAPE, "pd_maxpool2x2_fwd: too large");
-    maxpool2_fwd_kernel<<<dim3(blocks), dim3(PW_THREADS), 0, (hipStream_t)stream>>>(x, y, N, H, W, C);
+    maxpool2_fwd_kernel<<<dim3(blocks), dim3(PW_THREADS), 0, (hipStream_t)stream>>>(x, y, N, H, W, C, relu);
     PD_CHECK_LAUNCH("pd_maxpool2x2_fwd");
     return PD_OK;
 }

@@ -162,31 +162,69 @@ class ReLU(torch.nn.Module):
 
 class _MaxPool2x2Fn(torch.autograd.Function):
     @staticmethod
-    def forward(ctx, x, after_relu):
+    def forward(ctx, x, relu):
         x = ops.to_nhwc(x)
-        y = ops.maxpool2x2(x)
-        ctx.after_relu = after_relu
+        y = ops.maxpool2x2(x, relu=relu)
+        ctx.relu = relu
         ctx.save_for_backward(x)
         return y
 
     @staticmethod
     def backward(ctx, dy):
         (x,) = ctx.saved_tensors
-        return ops.maxpool2x2_backward(x, dy, relu_mask=False), None
+        return ops.maxpool2x2_backward(x, dy, relu_mask=ctx.relu), None
 
 
 class MaxPool2d(torch.nn.Module):
     """``torch.nn.MaxPool2d(kernel_size=2, stride=2)`` on NHWC activations."""
 
-    def __init__(self, kernel_size=2, stride=2, padding=0, dilation=1, ceil_mode=False):
+    def __init__(self, kernel_size=2, stride=2, padding=0, dilation=1, ceil_mode=False, relu=False):
         super(MaxPool2d, self).__init__()
+        self.relu = relu  # a ReLU in front of the pooling (stage1.py:10-11), fused
         ks = kernel_size if isinstance(kernel_size, int) else kernel_size[0]
         st = ks if stride is None else (stride if isinstance(stride, int) else stride[0])
         if ks != 2 or st != 2 or padding not in (0, (0, 0)) or dilation not in (1, (1, 1)) or ceil_mode:
             raise NotImplementedError("only MaxPool2d(kernel_size=2, stride=2) has a HIP kernel")
 
     def forward(self, x):
-        return _MaxPool2x2Fn.apply(x, False)
+        return _MaxPool2x2Fn.apply(x, self.relu)
+
+
+class _DropoutFn(torch.autograd.Function):
+    @staticmethod
+    def forward(ctx, x, mask, scale):
+        ctx.scale = scale
+        ctx.save_for_backward(mask)
+        return ops.mask_scale(x, mask, scale)
+
+    @staticmethod
+    def backward(ctx, dy):
+        (mask,) = ctx.saved_tensors
+        if dy.stride() != mask.stride():
+            dy = dy.contiguous()
+        return ops.mask_scale(dy, mask, ctx.scale), None, None
+
+
+class Dropout(torch.nn.Module):
+    """``torch.nn.Dropout(p)``.  The keep-mask comes from ``mask_fn(x) -> uint8 tensor`` when
+    one is set (parity runs inject host-generated masks so that both sides drop the same
+    elements), otherwise from torch's device generator; applying it is a HIP kernel."""
+
+    def __init__(self, p=0.5, inplace=False):
+        super(Dropout, self).__init__()
+        if p < 0 or p >= 1:
+            raise ValueError("dropout probability has to be in [0, 1), got {}".format(p))
+        self.p = p
+        self.mask_fn = None
+
+    def forward(self, x):
+        if not self.training or self.p == 0:
+            return x
+        if self.mask_fn is not None:
+            mask = self.mask_fn(x)
+        else:
+            mask = (torch.rand_like(x) >= self.p).to(torch.uint8)
+        return _DropoutFn.apply(x, mask, 1.0 / (1.0 - self.p))
 
 
 class Flatten(torch.nn.Module):

@@ -13,6 +13,31 @@ from . import _cabi
 
 _vp = ctypes.c_void_p
 
+# Optional per-launch timing: when `kernel_timer` is a dict, every timed launch appends a
+# (start, end, work) triple of HIP events recorded on the launch stream under the kernel's
+# name; `work` is the algorithmic flop (or byte) count of that launch.
+kernel_timer = None
+
+
+class _timed(object):
+    __slots__ = ("name", "work", "start")
+
+    def __init__(self, name, work):
+        self.name = name
+        self.work = work
+
+    def __enter__(self):
+        if kernel_timer is not None:
+            self.start = torch.cuda.Event(enable_timing=True)
+            self.start.record()
+
+    def __exit__(self, *exc):
+        if kernel_timer is not None:
+            end = torch.cuda.Event(enable_timing=True)
+            end.record()
+            kernel_timer.setdefault(self.name, []).append((self.start, end, self.work))
+        return False
+
 
 def _ptr(t):
     return _vp(t.data_ptr()) if t is not None else None
@@ -113,6 +138,19 @@ def relu_backward(dy, y):
     return dx
 
 
+def mask_scale(x, mask, scale):
+    """y = x * mask * scale with a uint8 0/1 mask of x's shape and memory order."""
+    _check(x, "x")
+    _check(mask, "mask", torch.uint8)
+    if not _is_dense(x):
+        x = x.contiguous()
+    if not _dense_same_order(mask, x):
+        raise ValueError("mask_scale: mask must have the shape and memory order of x")
+    y = torch.empty_like(x)
+    _cabi.lib().pd_mask_scale_f32(_ptr(x), _ptr(mask), _ptr(y), x.numel(), float(scale), _cabi.stream_ptr())
+    return y
+
+
 def to_nhwc(x):
     """A logically-NCHW 4-D tensor whose memory order is N,H,W,C."""
     if x.dim() != 4:
@@ -127,13 +165,14 @@ def _nhwc_dims(x):
     return n, h, w, c
 
 
-def maxpool2x2(x):
+def maxpool2x2(x, relu=False):
+    """2x2/stride-2 max pooling; ``relu=True`` pools a (virtual) ReLU of ``x``."""
     _check(x, "x")
     x = to_nhwc(x)
     n, h, w, c = _nhwc_dims(x)
     y = torch.empty((n, c, h // 2, w // 2), dtype=torch.float32, device=x.device,
                     memory_format=torch.channels_last)
-    _cabi.lib().pd_maxpool2x2_fwd_nhwc_f32(_ptr(x), _ptr(y), n, h, w, c, _cabi.stream_ptr())
+    _cabi.lib().pd_maxpool2x2_fwd_nhwc_f32(_ptr(x), _ptr(y), n, h, w, c, int(relu), _cabi.stream_ptr())
     return y
 
 
@@ -203,8 +242,9 @@ def conv3x3_forward(x, w, bias=None, relu=False):
         if bias.numel() != k or not bias.is_contiguous():
             raise ValueError("conv3x3: bias must be a contiguous vector of K=%d" % k)
     y = torch.empty((n, k, h, wd), dtype=torch.float32, device=x.device, memory_format=torch.channels_last)
-    _cabi.lib().pd_conv3x3_fwd_nhwc_f32(_ptr(x), _ptr(w), _ptr(bias), _ptr(y), n, h, wd, c, k, int(relu),
-                                        _cabi.stream_ptr())
+    with _timed("conv3x3_fwd_kernel" if c > 8 else "conv3x3_fwd_kernel_smallc", 18.0 * c * k * n * h * wd):
+        _cabi.lib().pd_conv3x3_fwd_nhwc_f32(_ptr(x), _ptr(w), _ptr(bias), _ptr(y), n, h, wd, c, k, int(relu),
+                                            _cabi.stream_ptr())
     return y
 
 
@@ -220,7 +260,8 @@ def conv3x3_input_grad(dy, w):
     wr = torch.empty((c, k, 3, 3), dtype=torch.float32, device=w.device, memory_format=torch.channels_last)
     lib.pd_conv3x3_filter_rot180_f32(_ptr(w), _ptr(wr), k, c, _cabi.stream_ptr())
     dx = torch.empty((n, c, h, wd), dtype=torch.float32, device=dy.device, memory_format=torch.channels_last)
-    lib.pd_conv3x3_fwd_nhwc_f32(_ptr(dy), _ptr(wr), None, _ptr(dx), n, h, wd, k, c, 0, _cabi.stream_ptr())
+    with _timed("conv3x3_fwd_kernel" if k > 8 else "conv3x3_fwd_kernel_smallc", 18.0 * c * k * n * h * wd):
+        lib.pd_conv3x3_fwd_nhwc_f32(_ptr(dy), _ptr(wr), None, _ptr(dx), n, h, wd, k, c, 0, _cabi.stream_ptr())
     return dx
 
 
@@ -238,6 +279,7 @@ def conv3x3_weight_grad(x, dy, with_bias=True):
     ws = torch.empty(nbytes.value, dtype=torch.uint8, device=x.device)
     dw = torch.empty((k, c, 3, 3), dtype=torch.float32, device=x.device, memory_format=torch.channels_last)
     db = torch.empty(k, dtype=torch.float32, device=x.device) if with_bias else None
-    lib.pd_conv3x3_wgrad_nhwc_f32(_ptr(x), _ptr(dy), _ptr(dw), _ptr(db), _ptr(ws), nbytes.value, n, h, wd, c, k,
-                                  _cabi.stream_ptr())
+    with _timed("conv3x3_wgrad", 18.0 * c * k * n * h * wd):
+        lib.pd_conv3x3_wgrad_nhwc_f32(_ptr(x), _ptr(dy), _ptr(dw), _ptr(db), _ptr(ws), nbytes.value, n, h, wd, c, k,
+                                      _cabi.stream_ptr())
     return dw, db

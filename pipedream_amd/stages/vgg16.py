@@ -1,0 +1,143 @@
+"""VGG16 stage definitions.
+
+``model(criterion)`` / ``Stage0..Stage3`` follow the reference's 4-stage straight split
+(runtime/image_classification/models/vgg16/gpus=4_straight/__init__.py:13-20,
+stage0.py:10-33, stage1.py:8-32, stage2.py:8-36, stage3.py:10-46 and mp_conf.json): the
+same layers in the same stages, the same attribute names for every layer that owns
+parameters (so ``state_dict()`` keys match), the same initialisation.  A ReLU that
+follows a convolution or a Linear layer inside a stage is fused into that layer's
+epilogue, and the ReLU + MaxPool pair at the head of stages 1 is fused into the pooling
+kernel, so those ReLU attributes do not exist as separate modules.
+
+``FrontStage`` is the "conv1_1 .. pool2" stage of the headline benchmark configuration;
+the reference never cuts exactly there (its 2-GPU split keeps conv1_1..conv2_2 in
+vgg16/gpus=2/stage0.py:10-17 and puts the following ReLU + MaxPool at the head of
+stage1.py:10-11), the layer names follow gpus=2/stage0.py.
+"""
+import torch
+
+from .. import layers
+
+
+def _initialize_weights(module):
+    """stage0.py:22-33: conv kaiming-normal (fan_out, relu), biases 0, Linear N(0, 0.01)."""
+    for m in module.modules():
+        if isinstance(m, layers.Conv2d):
+            w = torch.empty(m.weight.shape)
+            torch.nn.init.kaiming_normal_(w, mode='fan_out', nonlinearity='relu')
+            with torch.no_grad():
+                m.weight.copy_(w)
+                if m.bias is not None:
+                    m.bias.zero_()
+        elif isinstance(m, layers.Linear):
+            torch.nn.init.normal_(m.weight, 0, 0.01)
+            torch.nn.init.constant_(m.bias, 0)
+
+
+class FrontStage(torch.nn.Module):
+    """conv1_1, conv1_2, pool1, conv2_1, conv2_2, pool2 (ReLU after every convolution)."""
+
+    def __init__(self):
+        super(FrontStage, self).__init__()
+        self.layer2 = layers.Conv2d(3, 64, relu=True)
+        self.layer4 = layers.Conv2d(64, 64, relu=True)
+        self.layer6 = layers.MaxPool2d(2, 2)
+        self.layer7 = layers.Conv2d(64, 128, relu=True)
+        self.layer9 = layers.Conv2d(128, 128, relu=True)
+        self.layer11 = layers.MaxPool2d(2, 2)
+        _initialize_weights(self)
+
+    def forward(self, input0):
+        out = self.layer4(self.layer2(input0))
+        out = self.layer6(out)
+        out = self.layer9(self.layer7(out))
+        return self.layer11(out)
+
+
+class Stage0(torch.nn.Module):
+    def __init__(self):
+        super(Stage0, self).__init__()
+        self.layer2 = layers.Conv2d(3, 64, relu=True)      # + layer3 ReLU
+        self.layer4 = layers.Conv2d(64, 64)
+        _initialize_weights(self)
+
+    def forward(self, input0):
+        return self.layer4(self.layer2(input0))
+
+
+class Stage1(torch.nn.Module):
+    def __init__(self):
+        super(Stage1, self).__init__()
+        self.layer2 = layers.MaxPool2d(2, 2, relu=True)    # layer1 ReLU + layer2 MaxPool
+        self.layer3 = layers.Conv2d(64, 128, relu=True)    # + layer4
+        self.layer5 = layers.Conv2d(128, 128, relu=True)   # + layer6
+        self.layer7 = layers.MaxPool2d(2, 2)
+        self.layer8 = layers.Conv2d(128, 256, relu=True)   # + layer9
+        _initialize_weights(self)
+
+    def forward(self, input0):
+        out = self.layer2(input0)
+        out = self.layer5(self.layer3(out))
+        return self.layer8(self.layer7(out))
+
+
+class Stage2(torch.nn.Module):
+    def __init__(self):
+        super(Stage2, self).__init__()
+        self.layer1 = layers.Conv2d(256, 256, relu=True)   # + layer2
+        self.layer3 = layers.Conv2d(256, 256, relu=True)   # + layer4
+        self.layer5 = layers.MaxPool2d(2, 2)
+        self.layer6 = layers.Conv2d(256, 512, relu=True)   # + layer7
+        self.layer8 = layers.Conv2d(512, 512, relu=True)   # + layer9
+        self.layer10 = layers.Conv2d(512, 512, relu=True)  # + layer11
+        _initialize_weights(self)
+
+    def forward(self, input0):
+        out = self.layer3(self.layer1(input0))
+        out = self.layer5(out)
+        return self.layer10(self.layer8(self.layer6(out)))
+
+
+class Stage3(torch.nn.Module):
+    def __init__(self, dropout=0.5, num_classes=1000):
+        super(Stage3, self).__init__()
+        self.layer1 = layers.MaxPool2d(2, 2)
+        self.layer2 = layers.Conv2d(512, 512, relu=True)   # + layer3
+        self.layer4 = layers.Conv2d(512, 512, relu=True)   # + layer5
+        self.layer6 = layers.Conv2d(512, 512, relu=True)   # + layer7
+        self.layer8 = layers.MaxPool2d(2, 2)
+        self.flatten = layers.Flatten()
+        self.layer11 = layers.Linear(25088, 4096, relu=True)   # + layer12
+        self.layer13 = layers.Dropout(p=dropout)
+        self.layer14 = layers.Linear(4096, 4096, relu=True)    # + layer15
+        self.layer16 = layers.Dropout(p=dropout)
+        self.layer17 = layers.Linear(4096, num_classes)
+        _initialize_weights(self)
+
+    def forward(self, input0):
+        out = self.layer1(input0)
+        out = self.layer6(self.layer4(self.layer2(out)))
+        out = self.flatten(self.layer8(out))
+        out = self.layer13(self.layer11(out))
+        out = self.layer16(self.layer14(out))
+        return self.layer17(out)
+
+
+def arch():
+    return "vgg16"
+
+
+def model(criterion, dropout=0.5):
+    return [
+        (Stage0(), ["input0"], ["out0"]),
+        (Stage1(), ["out0"], ["out1"]),
+        (Stage2(), ["out1"], ["out2"]),
+        (Stage3(dropout=dropout), ["out2"], ["out3"]),
+        (criterion, ["out3"], ["loss"]),
+    ]
+
+
+def conf():
+    """vgg16/gpus=4_straight/mp_conf.json"""
+    return {"module_to_stage_map": [0, 1, 2, 3, 3],
+            "stage_to_rank_map": {"0": [0], "1": [1], "2": [2], "3": [3]}}
