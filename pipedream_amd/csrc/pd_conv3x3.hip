@@ -48,14 +48,83 @@ struct ConvArgs {
     int c_vec;          // C % 4 == 0 and x/w 16-byte aligned: 128-bit global loads
 };
 
+// Global -> register staging of one reduction chunk (input halo tile + filter slice).
+// All loads of a chunk are issued back to back (fixed trip counts, no divergent
+// branches: out-of-range elements read a safe address and are zeroed by a select), so
+// a thread has ~15 128-bit loads in flight instead of one.
+template <int TH, int TW, int CC>
+struct FwdStage {
+    static constexpr int HW_ = TW + 2;
+    static constexpr int HALO = (TH + 2) * (TW + 2);
+    static constexpr int CP = CC + 4;
+    static constexpr int Q = CC / 4;
+    static constexpr int IN_ITERS = (HALO * Q + CONV_THREADS - 1) / CONV_THREADS;
+    static constexpr int W_ITERS = (9 * BN * Q + CONV_THREADS - 1) / CONV_THREADS;
+
+    float4_t rin[IN_ITERS];
+    float4_t rw[W_ITERS];
+
+    __device__ __forceinline__ void load(const ConvArgs& a, const float* __restrict__ xn, int y0, int x0, int k0,
+                                         int c0, int tid) {
+        const float4_t zero = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int it = 0; it < IN_ITERS; ++it) {
+            const int id = tid + it * CONV_THREADS;
+            const int p = id / Q, q4 = (id % Q) * 4;
+            const int gy = y0 + p / HW_ - 1, gx = x0 + p % HW_ - 1;
+            const int c = c0 + q4;
+            const bool ok = id < HALO * Q && gy >= 0 && gy < a.H && gx >= 0 && gx < a.W && c < a.C;
+            const float* src = ok ? xn + ((size_t)gy * a.W + gx) * a.C + c : xn;
+            float4_t v;
+            if (a.c_vec) {
+                v = *(const float4_t*)src;
+            } else {
+#pragma unroll
+                for (int j = 0; j < 4; ++j) v[j] = (ok && c + j < a.C) ? src[j] : 0.f;
+            }
+            rin[it] = ok ? v : zero;
+        }
+#pragma unroll
+        for (int it = 0; it < W_ITERS; ++it) {
+            const int id = tid + it * CONV_THREADS;
+            const int row = id / Q, q4 = (id % Q) * 4;
+            const int tap = row / BN, k = k0 + row % BN;
+            const int c = c0 + q4;
+            const bool ok = id < 9 * BN * Q && k < a.K && c < a.C;
+            const float* src = ok ? a.w + ((size_t)k * 9 + tap) * a.C + c : a.w;
+            float4_t v;
+            if (a.c_vec) {
+                v = *(const float4_t*)src;
+            } else {
+#pragma unroll
+                for (int j = 0; j < 4; ++j) v[j] = (ok && c + j < a.C) ? src[j] : 0.f;
+            }
+            rw[it] = ok ? v : zero;
+        }
+    }
+
+    __device__ __forceinline__ void store(float* in_tile, float* w_tile, int tid) const {
+#pragma unroll
+        for (int it = 0; it < IN_ITERS; ++it) {
+            const int id = tid + it * CONV_THREADS;
+            if (id < HALO * Q) *(float4_t*)(in_tile + (id / Q) * CP + (id % Q) * 4) = rin[it];
+        }
+#pragma unroll
+        for (int it = 0; it < W_ITERS; ++it) {
+            const int id = tid + it * CONV_THREADS;
+            if (id < 9 * BN * Q) *(float4_t*)(w_tile + (id / Q) * CP + (id % Q) * 4) = rw[it];
+        }
+    }
+};
+
 template <int TH, int TW, int CC>
 __global__ __launch_bounds__(CONV_THREADS, 2) void conv3x3_fwd_kernel(const ConvArgs a) {
     static_assert(TH * TW == 256, "a block owns 256 pixels");
     static_assert(TW == 8 || TW == 16 || TW == 32, "an MFMA row tile is 32/TW rows of TW pixels");
-    constexpr int HW_ = TW + 2;                  // halo tile width
-    constexpr int HALO = (TH + 2) * (TW + 2);    // halo pixels
-    constexpr int CP = CC + 4;                   // LDS pitch per pixel / per filter row
-    constexpr int Q = CC / 4;                    // float4 per pixel per chunk
+    using Stage = FwdStage<TH, TW, CC>;
+    constexpr int HW_ = Stage::HW_;
+    constexpr int HALO = Stage::HALO;
+    constexpr int CP = Stage::CP;
     __shared__ __attribute__((aligned(16))) float in_tile[HALO * CP];
     __shared__ __attribute__((aligned(16))) float w_tile[9 * BN * CP];
 
@@ -90,45 +159,15 @@ __global__ __launch_bounds__(CONV_THREADS, 2) void conv3x3_fwd_kernel(const Conv
 
     const float* xn = a.x + (size_t)n * a.H * a.W * a.C;
 
+    // Software pipeline over the reduction chunks: the global loads of chunk i+1 are in
+    // flight while chunk i is multiplied out of LDS.
+    Stage st;
+    st.load(a, xn, y0, x0, k0, 0, tid);
     for (int c0 = 0; c0 < a.C; c0 += CC) {
         __syncthreads();  // everyone is done reading the previous chunk
-        // ---- input halo tile: pixel p, channel quad q ---------------------------------
-        for (int id = tid; id < HALO * Q; id += CONV_THREADS) {
-            const int p = id / Q, q4 = (id % Q) * 4;
-            const int gy = y0 + p / HW_ - 1, gx = x0 + p % HW_ - 1;
-            const int c = c0 + q4;
-            float4_t v = {0.f, 0.f, 0.f, 0.f};
-            if (gy >= 0 && gy < a.H && gx >= 0 && gx < a.W && c < a.C) {
-                const float* src = xn + ((size_t)gy * a.W + gx) * a.C + c;
-                if (a.c_vec) {
-                    v = *(const float4_t*)src;
-                } else {
-#pragma unroll
-                    for (int j = 0; j < 4; ++j)
-                        if (c + j < a.C) v[j] = src[j];
-                }
-            }
-            *(float4_t*)(in_tile + p * CP + q4) = v;
-        }
-        // ---- filter slice: row = tap*64 + out channel ----------------------------------
-        for (int id = tid; id < 9 * BN * Q; id += CONV_THREADS) {
-            const int row = id / Q, q4 = (id % Q) * 4;
-            const int tap = row / BN, k = k0 + row % BN;
-            const int c = c0 + q4;
-            float4_t v = {0.f, 0.f, 0.f, 0.f};
-            if (k < a.K && c < a.C) {
-                const float* src = a.w + ((size_t)k * 9 + tap) * a.C + c;
-                if (a.c_vec) {
-                    v = *(const float4_t*)src;
-                } else {
-#pragma unroll
-                    for (int j = 0; j < 4; ++j)
-                        if (c + j < a.C) v[j] = src[j];
-                }
-            }
-            *(float4_t*)(w_tile + row * CP + q4) = v;
-        }
+        st.store(in_tile, w_tile, tid);
         __syncthreads();
+        if (c0 + CC < a.C) st.load(a, xn, y0, x0, k0, c0 + CC, tid);
         // ---- 9 taps x CC/8 k-groups x (4 LDS reads + 16 MFMAs) ---------------------------
 #pragma unroll
         for (int tap = 0; tap < 9; ++tap) {
@@ -232,40 +271,71 @@ __global__ __launch_bounds__(CONV_THREADS, 2) void conv3x3_wgrad_kernel(const Wg
         const float* xn = a.x + (size_t)n * a.H * a.W * a.C;
         const float* dyn = a.dy + (size_t)n * a.H * a.W * a.K;
 
-        __syncthreads();
-        for (int id = tid; id < PIX * (CS / 4); id += CONV_THREADS) {
+        // The tile's global loads are issued in two batches (dY + first part of X, then the
+        // rest of X): fixed trip counts and selects instead of branches, so a thread has
+        // 8-12 128-bit loads in flight at a time without outgrowing the register file
+        // next to the 144 accumulators.
+        constexpr int DY_ITERS = (PIX * (CS / 4) + CONV_THREADS - 1) / CONV_THREADS;
+        constexpr int X_ITERS = (HALO * (CS / 4) + CONV_THREADS - 1) / CONV_THREADS;
+        constexpr int X_SPLIT = X_ITERS / 3;
+        const float4_t zero = {0.f, 0.f, 0.f, 0.f};
+        auto load_x = [&](int it) -> float4_t {
+            const int id = tid + it * CONV_THREADS;
             const int p = id / (CS / 4), q4 = (id % (CS / 4)) * 4;
-            const int gy = y0 + p / TW, gx = x0 + p % TW;
-            const int k = k0 + q4;
-            float4_t v = {0.f, 0.f, 0.f, 0.f};
-            if (gy < a.H && gx < a.W && k < a.K) {
-                const float* src = dyn + ((size_t)gy * a.W + gx) * a.K + k;
+            const int gy = y0 + p / HW_ - 1, gx = x0 + p % HW_ - 1;
+            const int c = c0 + q4;
+            const bool ok = id < HALO * (CS / 4) && gy >= 0 && gy < a.H && gx >= 0 && gx < a.W && c < a.C;
+            const float* src = ok ? xn + ((size_t)gy * a.W + gx) * a.C + c : xn;
+            float4_t v;
+            if (a.c_vec) {
+                v = *(const float4_t*)src;
+            } else {
+#pragma unroll
+                for (int j = 0; j < 4; ++j) v[j] = (ok && c + j < a.C) ? src[j] : 0.f;
+            }
+            return ok ? v : zero;
+        };
+        auto store_x = [&](int it, float4_t v) {
+            const int id = tid + it * CONV_THREADS;
+            if (id < HALO * (CS / 4)) *(float4_t*)(x_tile + (id / (CS / 4)) * CS + (id % (CS / 4)) * 4) = v;
+        };
+        {
+            float4_t rdy[DY_ITERS], rx[X_SPLIT];
+#pragma unroll
+            for (int it = 0; it < DY_ITERS; ++it) {
+                const int id = tid + it * CONV_THREADS;
+                const int p = id / (CS / 4), q4 = (id % (CS / 4)) * 4;
+                const int gy = y0 + p / TW, gx = x0 + p % TW;
+                const int k = k0 + q4;
+                const bool ok = id < PIX * (CS / 4) && gy < a.H && gx < a.W && k < a.K;
+                const float* src = ok ? dyn + ((size_t)gy * a.W + gx) * a.K + k : dyn;
+                float4_t v;
                 if (a.k_vec) {
                     v = *(const float4_t*)src;
                 } else {
 #pragma unroll
-                    for (int j = 0; j < 4; ++j)
-                        if (k + j < a.K) v[j] = src[j];
+                    for (int j = 0; j < 4; ++j) v[j] = (ok && k + j < a.K) ? src[j] : 0.f;
                 }
+                rdy[it] = ok ? v : zero;
             }
-            *(float4_t*)(dy_tile + p * CS + q4) = v;
-        }
-        for (int id = tid; id < HALO * (CS / 4); id += CONV_THREADS) {
-            const int p = id / (CS / 4), q4 = (id % (CS / 4)) * 4;
-            const int gy = y0 + p / HW_ - 1, gx = x0 + p % HW_ - 1;
-            const int c = c0 + q4;
-            float4_t v = {0.f, 0.f, 0.f, 0.f};
-            if (gy >= 0 && gy < a.H && gx >= 0 && gx < a.W && c < a.C) {
-                const float* src = xn + ((size_t)gy * a.W + gx) * a.C + c;
-                if (a.c_vec) {
-                    v = *(const float4_t*)src;
-                } else {
 #pragma unroll
-                    for (int j = 0; j < 4; ++j)
-                        if (c + j < a.C) v[j] = src[j];
-                }
+            for (int it = 0; it < X_SPLIT; ++it) rx[it] = load_x(it);
+            __syncthreads();  // everyone is done reading the previous tile
+#pragma unroll
+            for (int it = 0; it < DY_ITERS; ++it) {
+                const int id = tid + it * CONV_THREADS;
+                if (id < PIX * (CS / 4))
+                    *(float4_t*)(dy_tile + (id / (CS / 4)) * CS + (id % (CS / 4)) * 4) = rdy[it];
             }
-            *(float4_t*)(x_tile + p * CS + q4) = v;
+#pragma unroll
+            for (int it = 0; it < X_SPLIT; ++it) store_x(it, rx[it]);
+        }
+        {
+            float4_t rx[X_ITERS - X_SPLIT];
+#pragma unroll
+            for (int it = X_SPLIT; it < X_ITERS; ++it) rx[it - X_SPLIT] = load_x(it);
+#pragma unroll
+            for (int it = X_SPLIT; it < X_ITERS; ++it) store_x(it, rx[it - X_SPLIT]);
         }
         __syncthreads();
         if (wave_active) {
