@@ -185,6 +185,28 @@ int pd_conv3x3_wgrad_nhwc_f32(const float* x, const float* dy, float* dw, float*
                               void* workspace, uint64_t workspace_bytes,
                               int N, int H, int W, int C, int K, void* stream);
 
+/* torch.nn.LSTM cell (gnmt_large/gpus=4/stage0.py:14-19), gate order i,f,g,o.
+ * Forward, one time step: gates[B][4H] holds x W_ih^T + h_prev W_hh^T on entry (from
+ * pd_gemm_f32) and the activated gates on exit; biases and c_prev may be NULL (= 0).
+ * c = f*c_prev + i*g, h = o*tanh(c). */
+int pd_lstm_cell_fwd_f32(float* gates, const float* b_ih, const float* b_hh, const float* c_prev,
+                         float* c_out, float* h_out, int B, int H, void* stream);
+/* Backward of that step: dh = dy (+ dh_rec if not NULL); dc_io holds dL/dc_t from the next
+ * step on entry (ignored when first_step != 0, i.e. for the last time step) and dL/dc_prev
+ * on exit; dgates[B][4H] = gradients of the gate pre-activations. */
+int pd_lstm_cell_bwd_f32(const float* gates, const float* c_prev, const float* c, const float* dy,
+                         const float* dh_rec, float* dc_io, float* dgates, int B, int H, int first_step,
+                         void* stream);
+/* y = a + b: the residual connections `out13 = out13 + out10` (stage0.py:32, 36). */
+int pd_add_f32(const float* a, const float* b, float* y, uint64_t n, void* stream);
+/* torch.nn.Embedding (stage0.py:10): out[p][:] = weight[ids[p]][:].  Backward writes the
+ * whole dense dweight[V][D] (zeros for unused rows and for padding_idx; pass -1 for none),
+ * summing duplicates in position order. */
+int pd_embedding_fwd_f32(const int64_t* ids, const float* weight, float* out, int n_tokens, int D, int64_t V,
+                         void* stream);
+int pd_embedding_bwd_f32(const int64_t* ids, const float* dout, float* dweight, int n_tokens, int D, int64_t V,
+                         int64_t padding_idx, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -150,3 +150,28 @@ class VggStage3(torch.nn.Module):
         x = self._drop("layer13", F.relu(self.layer11(x)))
         x = self._drop("layer16", F.relu(self.layer14(x)))
         return self.layer17(x)
+
+
+# --------------------------------------------------------------------------------------
+# GNMT-style stage (gnmt_large/gpus=4/stage0.py:10-40 without the bidirectional layer)
+# --------------------------------------------------------------------------------------
+class GnmtStage0(torch.nn.Module):
+    def __init__(self, vocab=32320, hidden=1024, dropout=0.2):
+        super(GnmtStage0, self).__init__()
+        self.layer6 = torch.nn.Embedding(vocab, hidden, padding_idx=0)
+        self.layer7 = torch.nn.LSTM(hidden, hidden)
+        self.layer8 = torch.nn.Dropout(p=dropout)
+        self.layer9 = torch.nn.LSTM(hidden, hidden)
+        self.layer11 = torch.nn.Dropout(p=dropout)
+        self.layer12 = torch.nn.LSTM(hidden, hidden)
+        self.layer15 = torch.nn.Dropout(p=dropout)
+        self.layer16 = torch.nn.LSTM(hidden, hidden)
+
+    def forward(self, input0):
+        out6 = self.layer6(input0)
+        out7 = self.layer7(out6)[0]
+        out9 = self.layer9(self.layer8(out7))[0]
+        out12 = self.layer12(self.layer11(out9))[0]
+        out13 = out12 + out9
+        out16 = self.layer16(self.layer15(out13))[0]
+        return out16 + out13

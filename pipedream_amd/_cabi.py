@@ -74,6 +74,11 @@ SIGNATURES = {
     "pd_conv3x3_filter_rot180_f32": (_i, [_vp, _vp, _i, _i, _vp], True),
     "pd_conv3x3_wgrad_workspace_bytes": (_i, [_i, _i, _i, _i, _i, ctypes.POINTER(ctypes.c_uint64)], True),
     "pd_conv3x3_wgrad_nhwc_f32": (_i, [_vp, _vp, _vp, _vp, _vp, _u64, _i, _i, _i, _i, _i, _vp], True),
+    "pd_lstm_cell_fwd_f32": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _vp], True),
+    "pd_lstm_cell_bwd_f32": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _vp], True),
+    "pd_add_f32": (_i, [_vp, _vp, _vp, _u64, _vp], True),
+    "pd_embedding_fwd_f32": (_i, [_vp, _vp, _vp, _i, _i, _i64, _vp], True),
+    "pd_embedding_bwd_f32": (_i, [_vp, _vp, _vp, _i, _i, _i64, _i64, _vp], True),
     "pd_xent_bwd_f32": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i64, _vp], True),
 }
 

@@ -375,21 +375,25 @@ __global__ __launch_bounds__(CONV_THREADS, 2) void conv3x3_wgrad_kernel(const Wg
     }
 }
 
-// out[i] = sum_b part[b][i]  (fixed order -> deterministic)
+// out[i] = sum_b part[b][i] in a fixed order (deterministic).  A block owns 64 outputs;
+// its 4 waves each sum a quarter of the partials, then combine through LDS.
 __global__ __launch_bounds__(256) void reduce_partials_kernel(const float* __restrict__ part, float* __restrict__ out,
                                                               int n_part, int n) {
-    const int i = blockIdx.x * 256 + threadIdx.x;
-    if (i >= n) return;
-    float s0 = 0.f, s1 = 0.f, s2 = 0.f, s3 = 0.f;
-    int b = 0;
-    for (; b + 3 < n_part; b += 4) {
-        s0 += part[(size_t)b * n + i];
-        s1 += part[(size_t)(b + 1) * n + i];
-        s2 += part[(size_t)(b + 2) * n + i];
-        s3 += part[(size_t)(b + 3) * n + i];
+    __shared__ float red[4][64];
+    const int lane = threadIdx.x % 64, w = threadIdx.x / 64;
+    const int i = blockIdx.x * 64 + lane;
+    float s0 = 0.f, s1 = 0.f;
+    if (i < n) {
+        int b = w;
+        for (; b + 4 < n_part; b += 8) {
+            s0 += part[(size_t)b * n + i];
+            s1 += part[(size_t)(b + 4) * n + i];
+        }
+        if (b < n_part) s0 += part[(size_t)b * n + i];
     }
-    for (; b < n_part; ++b) s0 += part[(size_t)b * n + i];
-    out[i] = (s0 + s1) + (s2 + s3);
+    red[w][lane] = s0 + s1;
+    __syncthreads();
+    if (w == 0 && i < n) out[i] = (red[0][lane] + red[1][lane]) + (red[2][lane] + red[3][lane]);
 }
 
 struct TileShape {
@@ -504,10 +508,10 @@ extern "C" int pd_conv3x3_wgrad_nhwc_f32(const float* x, const float* dy, float*
     conv3x3_wgrad_kernel<WGRAD_TH, WGRAD_TW><<<grid, CONV_THREADS, 0, s>>>(a);
     PD_CHECK_LAUNCH("pd_conv3x3_wgrad_nhwc_f32");
     const int nw = K * 9 * C;
-    reduce_partials_kernel<<<dim3((nw + 255) / 256), dim3(256), 0, s>>>(a.part_w, dw, nb, nw);
+    reduce_partials_kernel<<<dim3((nw + 63) / 64), dim3(256), 0, s>>>(a.part_w, dw, nb, nw);
     PD_CHECK_LAUNCH("pd_conv3x3_wgrad_nhwc_f32(reduce)");
     if (dbias) {
-        reduce_partials_kernel<<<dim3((K + 255) / 256), dim3(256), 0, s>>>(a.part_b, dbias, nb, K);
+        reduce_partials_kernel<<<dim3((K + 63) / 64), dim3(256), 0, s>>>(a.part_b, dbias, nb, K);
         PD_CHECK_LAUNCH("pd_conv3x3_wgrad_nhwc_f32(reduce bias)");
     }
     return PD_OK;

@@ -1,0 +1,238 @@
+// LSTM cell (gate non-linearities + state update) and embedding lookup, forward and
+// backward: the HBM-bound parts of the GNMT-style stage.  The matrix products around
+// them (input projection for all time steps, the per-step recurrent product, the weight
+// gradients) run on the fp32 MFMA GEMM.
+//
+// They stand in for torch.nn.LSTM / torch.nn.Embedding of the reference's translation
+// stages (runtime/translation/models/gnmt_large/gpus=4/stage0.py:10-19; gate order and
+// parameter layout are torch's: rows [i | f | g | o] of weight_ih / weight_hh / bias).
+//
+// Algorithmic traffic per (batch row, hidden unit) and time step:
+//   forward : read 4 gate pre-activations + c_prev, write 4 activated gates + c + h = 44 B
+//   backward: read 4 gates + c_prev + c + dh (+dy) + dc, write 4 dgates + dc        = 60-64 B
+#include "pd_internal.h"
+
+typedef float float4_t __attribute__((ext_vector_type(4)));
+
+namespace {
+
+constexpr int LSTM_THREADS = 256;
+
+__device__ __forceinline__ float sigmoidf_(float x) { return 1.0f / (1.0f + expf(-x)); }
+
+// gates: [B][4H] pre-activations (x W_ih^T + h W_hh^T), overwritten with the ACTIVATED
+// gates i,f,g,o which the backward pass needs.  One thread = 4 consecutive hidden units.
+__global__ __launch_bounds__(LSTM_THREADS) void lstm_cell_fwd_kernel(float* __restrict__ gates,
+                                                                     const float* __restrict__ b_ih,
+                                                                     const float* __restrict__ b_hh,
+                                                                     const float* __restrict__ c_prev,
+                                                                     float* __restrict__ c_out,
+                                                                     float* __restrict__ h_out, int B, int H) {
+    const int H4 = H / 4;
+    const int id = blockIdx.x * LSTM_THREADS + threadIdx.x;
+    if (id >= B * H4) return;
+    const int b = id / H4, j = (id % H4) * 4;
+    float* g = gates + (size_t)b * 4 * H;
+    float4_t gi = *(const float4_t*)(g + j);
+    float4_t gf = *(const float4_t*)(g + H + j);
+    float4_t gg = *(const float4_t*)(g + 2 * H + j);
+    float4_t go = *(const float4_t*)(g + 3 * H + j);
+    if (b_ih) {
+        gi += *(const float4_t*)(b_ih + j) + *(const float4_t*)(b_hh + j);
+        gf += *(const float4_t*)(b_ih + H + j) + *(const float4_t*)(b_hh + H + j);
+        gg += *(const float4_t*)(b_ih + 2 * H + j) + *(const float4_t*)(b_hh + 2 * H + j);
+        go += *(const float4_t*)(b_ih + 3 * H + j) + *(const float4_t*)(b_hh + 3 * H + j);
+    }
+    float4_t cp = {0.f, 0.f, 0.f, 0.f};
+    if (c_prev) cp = *(const float4_t*)(c_prev + (size_t)b * H + j);
+    float4_t c, h;
+#pragma unroll
+    for (int k = 0; k < 4; ++k) {
+        gi[k] = sigmoidf_(gi[k]);
+        gf[k] = sigmoidf_(gf[k]);
+        gg[k] = tanhf(gg[k]);
+        go[k] = sigmoidf_(go[k]);
+        c[k] = gf[k] * cp[k] + gi[k] * gg[k];
+        h[k] = go[k] * tanhf(c[k]);
+    }
+    *(float4_t*)(g + j) = gi;
+    *(float4_t*)(g + H + j) = gf;
+    *(float4_t*)(g + 2 * H + j) = gg;
+    *(float4_t*)(g + 3 * H + j) = go;
+    *(float4_t*)(c_out + (size_t)b * H + j) = c;
+    *(float4_t*)(h_out + (size_t)b * H + j) = h;
+}
+
+// dh = dy (+ dh_rec); dc = dc_next + dh*o*(1-tanh(c)^2); dgates are gradients with respect
+// to the pre-activations; dc_next is overwritten with the gradient for c_prev.
+__global__ __launch_bounds__(LSTM_THREADS) void lstm_cell_bwd_kernel(const float* __restrict__ gates,
+                                                                     const float* __restrict__ c_prev,
+                                                                     const float* __restrict__ c,
+                                                                     const float* __restrict__ dy,
+                                                                     const float* __restrict__ dh_rec,
+                                                                     float* __restrict__ dc_io,
+                                                                     float* __restrict__ dgates, int B, int H,
+                                                                     int first_step) {
+    const int H4 = H / 4;
+    const int id = blockIdx.x * LSTM_THREADS + threadIdx.x;
+    if (id >= B * H4) return;
+    const int b = id / H4, j = (id % H4) * 4;
+    const float* g = gates + (size_t)b * 4 * H;
+    const float4_t gi = *(const float4_t*)(g + j);
+    const float4_t gf = *(const float4_t*)(g + H + j);
+    const float4_t gg = *(const float4_t*)(g + 2 * H + j);
+    const float4_t go = *(const float4_t*)(g + 3 * H + j);
+    const size_t o = (size_t)b * H + j;
+    float4_t cp = {0.f, 0.f, 0.f, 0.f};
+    if (c_prev) cp = *(const float4_t*)(c_prev + o);
+    const float4_t ct = *(const float4_t*)(c + o);
+    float4_t dh = *(const float4_t*)(dy + o);
+    if (dh_rec) dh += *(const float4_t*)(dh_rec + o);
+    float4_t dc = {0.f, 0.f, 0.f, 0.f};
+    if (!first_step) dc = *(const float4_t*)(dc_io + o);
+    float4_t di, df, dg, dO, dcp;
+#pragma unroll
+    for (int k = 0; k < 4; ++k) {
+        const float tc = tanhf(ct[k]);
+        const float dck = dc[k] + dh[k] * go[k] * (1.0f - tc * tc);
+        dO[k] = dh[k] * tc * go[k] * (1.0f - go[k]);
+        di[k] = dck * gg[k] * gi[k] * (1.0f - gi[k]);
+        df[k] = dck * cp[k] * gf[k] * (1.0f - gf[k]);
+        dg[k] = dck * gi[k] * (1.0f - gg[k] * gg[k]);
+        dcp[k] = dck * gf[k];
+    }
+    float* d = dgates + (size_t)b * 4 * H;
+    *(float4_t*)(d + j) = di;
+    *(float4_t*)(d + H + j) = df;
+    *(float4_t*)(d + 2 * H + j) = dg;
+    *(float4_t*)(d + 3 * H + j) = dO;
+    *(float4_t*)(dc_io + o) = dcp;
+}
+
+// y = a + b  (the residual connections between LSTM layers)
+__global__ __launch_bounds__(LSTM_THREADS) void add_kernel(const float* __restrict__ a, const float* __restrict__ b,
+                                                           float* __restrict__ y, uint64_t n, bool vec) {
+    uint64_t i = ((uint64_t)blockIdx.x * LSTM_THREADS + threadIdx.x) * 4;
+    if (i >= n) return;
+    if (vec && i + 3 < n) {
+        *(float4_t*)(y + i) = *(const float4_t*)(a + i) + *(const float4_t*)(b + i);
+    } else {
+        for (uint64_t k = i; k < n && k < i + 4; ++k) y[k] = a[k] + b[k];
+    }
+}
+
+// out[p][:] = weight[ids[p]][:]; one block per token, 4 floats per thread per pass.
+__global__ __launch_bounds__(LSTM_THREADS) void embedding_fwd_kernel(const int64_t* __restrict__ ids,
+                                                                     const float* __restrict__ weight,
+                                                                     float* __restrict__ out, int D, int64_t V) {
+    const int64_t v = ids[blockIdx.x];
+    const float* src = weight + (size_t)(v < 0 || v >= V ? 0 : v) * D;
+    float* dst = out + (size_t)blockIdx.x * D;
+    for (int j = threadIdx.x * 4; j < D; j += LSTM_THREADS * 4) *(float4_t*)(dst + j) = *(const float4_t*)(src + j);
+}
+
+// dweight[v][:] = sum over positions p with ids[p] == v of dout[p][:], positions in
+// increasing order (deterministic, no atomics); rows without a hit and the padding row
+// are written as zeros, so dweight needs no prior clearing.  One block per vocabulary row;
+// the ids are scanned 64 at a time with a ballot.
+__global__ __launch_bounds__(LSTM_THREADS) void embedding_bwd_kernel(const int64_t* __restrict__ ids,
+                                                                     const float* __restrict__ dout,
+                                                                     float* __restrict__ dweight, int n_tokens, int D,
+                                                                     int64_t padding_idx) {
+    const int64_t v = blockIdx.x;
+    const int lane = threadIdx.x % 64;
+    // every thread owns D/(4*256) float4 columns; D <= 4096 supported by the accumulators below
+    float4_t acc[4];
+#pragma unroll
+    for (int r = 0; r < 4; ++r) acc[r] = (float4_t){0.f, 0.f, 0.f, 0.f};
+    if (v != padding_idx) {
+        for (int p0 = 0; p0 < n_tokens; p0 += 64) {
+            const int p = p0 + lane;
+            const bool hit = p < n_tokens && ids[p] == v;
+            unsigned long long m = __ballot(hit);
+            while (m) {
+                const int bit = __ffsll((long long)m) - 1;
+                m &= m - 1;
+                const float* src = dout + (size_t)(p0 + bit) * D;
+#pragma unroll
+                for (int r = 0; r < 4; ++r) {
+                    const int j = (r * LSTM_THREADS + threadIdx.x) * 4;
+                    if (j < D) acc[r] += *(const float4_t*)(src + j);
+                }
+            }
+        }
+    }
+    float* dst = dweight + (size_t)v * D;
+#pragma unroll
+    for (int r = 0; r < 4; ++r) {
+        const int j = (r * LSTM_THREADS + threadIdx.x) * 4;
+        if (j < D) *(float4_t*)(dst + j) = acc[r];
+    }
+}
+
+}  // namespace
+
+extern "C" int pd_lstm_cell_fwd_f32(float* gates, const float* b_ih, const float* b_hh, const float* c_prev,
+                                    float* c_out, float* h_out, int B, int H, void* stream) {
+    PD_REQUIRE(B > 0 && H > 0 && H % 4 == 0, PD_ESHAPE, "pd_lstm_cell_fwd_f32: need B > 0 and H a positive multiple of 4");
+    PD_REQUIRE(gates && c_out && h_out, PD_EINVAL, "pd_lstm_cell_fwd_f32: NULL pointer");
+    PD_REQUIRE((b_ih == nullptr) == (b_hh == nullptr), PD_EINVAL, "pd_lstm_cell_fwd_f32: pass both biases or neither");
+    PD_REQUIRE(pd_aligned(gates, 16) && pd_aligned(c_out, 16) && pd_aligned(h_out, 16) &&
+                   (!c_prev || pd_aligned(c_prev, 16)) && (!b_ih || (pd_aligned(b_ih, 16) && pd_aligned(b_hh, 16))),
+               PD_EINVAL, "pd_lstm_cell_fwd_f32: pointers must be 16-byte aligned");
+    const int total = B * (H / 4);
+    lstm_cell_fwd_kernel<<<dim3((total + LSTM_THREADS - 1) / LSTM_THREADS), dim3(LSTM_THREADS), 0,
+                           (hipStream_t)stream>>>(gates, b_ih, b_hh, c_prev, c_out, h_out, B, H);
+    PD_CHECK_LAUNCH("pd_lstm_cell_fwd_f32");
+    return PD_OK;
+}
+
+extern "C" int pd_lstm_cell_bwd_f32(const float* gates, const float* c_prev, const float* c, const float* dy,
+                                    const float* dh_rec, float* dc_io, float* dgates, int B, int H, int first_step,
+                                    void* stream) {
+    PD_REQUIRE(B > 0 && H > 0 && H % 4 == 0, PD_ESHAPE, "pd_lstm_cell_bwd_f32: need B > 0 and H a positive multiple of 4");
+    PD_REQUIRE(gates && c && dy && dc_io && dgates, PD_EINVAL, "pd_lstm_cell_bwd_f32: NULL pointer");
+    PD_REQUIRE(pd_aligned(gates, 16) && pd_aligned(c, 16) && pd_aligned(dy, 16) && pd_aligned(dc_io, 16) &&
+                   pd_aligned(dgates, 16) && (!c_prev || pd_aligned(c_prev, 16)) && (!dh_rec || pd_aligned(dh_rec, 16)),
+               PD_EINVAL, "pd_lstm_cell_bwd_f32: pointers must be 16-byte aligned");
+    const int total = B * (H / 4);
+    lstm_cell_bwd_kernel<<<dim3((total + LSTM_THREADS - 1) / LSTM_THREADS), dim3(LSTM_THREADS), 0,
+                           (hipStream_t)stream>>>(gates, c_prev, c, dy, dh_rec, dc_io, dgates, B, H, first_step);
+    PD_CHECK_LAUNCH("pd_lstm_cell_bwd_f32");
+    return PD_OK;
+}
+
+extern "C" int pd_add_f32(const float* a, const float* b, float* y, uint64_t n, void* stream) {
+    if (n == 0) return PD_OK;
+    PD_REQUIRE(a && b && y, PD_EINVAL, "pd_add_f32: NULL pointer");
+    const uint64_t blocks = ((n + 3) / 4 + LSTM_THREADS - 1) / LSTM_THREADS;
+    PD_REQUIRE(blocks <= 0x7fffffffull, PD_ESHAPE, "pd_add_f32: too large");
+    const bool vec = pd_aligned(a, 16) && pd_aligned(b, 16) && pd_aligned(y, 16);
+    add_kernel<<<dim3((unsigned)blocks), dim3(LSTM_THREADS), 0, (hipStream_t)stream>>>(a, b, y, n, vec);
+    PD_CHECK_LAUNCH("pd_add_f32");
+    return PD_OK;
+}
+
+extern "C" int pd_embedding_fwd_f32(const int64_t* ids, const float* weight, float* out, int n_tokens, int D,
+                                    int64_t V, void* stream) {
+    PD_REQUIRE(n_tokens >= 0 && D > 0 && D % 4 == 0 && V > 0, PD_ESHAPE,
+               "pd_embedding_fwd_f32: need D a positive multiple of 4 and V > 0");
+    if (n_tokens == 0) return PD_OK;
+    PD_REQUIRE(ids && weight && out, PD_EINVAL, "pd_embedding_fwd_f32: NULL pointer");
+    PD_REQUIRE(pd_aligned(weight, 16) && pd_aligned(out, 16), PD_EINVAL, "pd_embedding_fwd_f32: 16-byte alignment");
+    embedding_fwd_kernel<<<dim3(n_tokens), dim3(LSTM_THREADS), 0, (hipStream_t)stream>>>(ids, weight, out, D, V);
+    PD_CHECK_LAUNCH("pd_embedding_fwd_f32");
+    return PD_OK;
+}
+
+extern "C" int pd_embedding_bwd_f32(const int64_t* ids, const float* dout, float* dweight, int n_tokens, int D,
+                                    int64_t V, int64_t padding_idx, void* stream) {
+    PD_REQUIRE(n_tokens >= 0 && D > 0 && D % 4 == 0 && D <= 4096 && V > 0 && V <= 0x7fffffff, PD_ESHAPE,
+               "pd_embedding_bwd_f32: need D a multiple of 4 in (0, 4096] and 0 < V < 2^31");
+    PD_REQUIRE(dweight && (n_tokens == 0 || (ids && dout)), PD_EINVAL, "pd_embedding_bwd_f32: NULL pointer");
+    PD_REQUIRE(pd_aligned(dweight, 16) && pd_aligned(dout, 16), PD_EINVAL, "pd_embedding_bwd_f32: 16-byte alignment");
+    embedding_bwd_kernel<<<dim3((unsigned)V), dim3(LSTM_THREADS), 0, (hipStream_t)stream>>>(ids, dout, dweight,
+                                                                                          n_tokens, D, padding_idx);
+    PD_CHECK_LAUNCH("pd_embedding_bwd_f32");
+    return PD_OK;
+}

@@ -236,6 +236,94 @@ class Flatten(torch.nn.Module):
 
 
 # --------------------------------------------------------------------------------------
+# Embedding / LSTM / residual add
+# --------------------------------------------------------------------------------------
+class _EmbeddingFn(torch.autograd.Function):
+    @staticmethod
+    def forward(ctx, ids, weight, padding_idx):
+        ctx.padding_idx = padding_idx
+        ctx.num_embeddings = weight.shape[0]
+        ctx.save_for_backward(ids)
+        return ops.embedding_forward(ids, weight)
+
+    @staticmethod
+    def backward(ctx, dout):
+        (ids,) = ctx.saved_tensors
+        return None, ops.embedding_backward(ids, dout, ctx.num_embeddings, ctx.padding_idx), None
+
+
+class Embedding(torch.nn.Module):
+    """``torch.nn.Embedding(num_embeddings, embedding_dim, padding_idx)`` with a dense
+    weight gradient (torch's default)."""
+
+    def __init__(self, num_embeddings, embedding_dim, padding_idx=None):
+        super(Embedding, self).__init__()
+        self.num_embeddings = num_embeddings
+        self.embedding_dim = embedding_dim
+        self.padding_idx = padding_idx
+        self.weight = torch.nn.Parameter(torch.empty(num_embeddings, embedding_dim))
+        torch.nn.init.normal_(self.weight)
+        if padding_idx is not None:
+            with torch.no_grad():
+                self.weight[padding_idx].fill_(0)
+
+    def forward(self, ids):
+        return _EmbeddingFn.apply(ids, self.weight, self.padding_idx)
+
+
+class _LSTMFn(torch.autograd.Function):
+    @staticmethod
+    def forward(ctx, x, w_ih, w_hh, b_ih, b_hh):
+        y, (gates, c) = ops.lstm_forward(x, w_ih, w_hh, b_ih, b_hh)
+        ctx.save_for_backward(x, y, gates, c, w_ih, w_hh)
+        return y
+
+    @staticmethod
+    def backward(ctx, dy):
+        x, y, gates, c, w_ih, w_hh = ctx.saved_tensors
+        dx, dw_ih, dw_hh, db = ops.lstm_backward(dy, x, y, gates, c, w_ih, w_hh, need_dx=ctx.needs_input_grad[0])
+        return dx, dw_ih, dw_hh, db, db.clone()
+
+
+class LSTM(torch.nn.Module):
+    """Single-layer uni-directional ``torch.nn.LSTM(input_size, hidden_size)`` on
+    sequence-first input ``[T, B, I]`` from zero initial state; returns ``(output, None)``
+    so that ``lstm(x)[0]`` reads like the reference's stages (stage0.py:28-29).  Parameter
+    names and layout are torch's (``weight_ih_l0`` ... ``bias_hh_l0``, gates i,f,g,o)."""
+
+    def __init__(self, input_size, hidden_size, num_layers=1, bias=True, batch_first=False, dropout=0,
+                 bidirectional=False):
+        super(LSTM, self).__init__()
+        if num_layers != 1 or not bias or batch_first or dropout or bidirectional:
+            raise NotImplementedError("only LSTM(input_size, hidden_size) with torch's other defaults is built")
+        self.input_size = input_size
+        self.hidden_size = hidden_size
+        k = 1.0 / math.sqrt(hidden_size)
+        self.weight_ih_l0 = torch.nn.Parameter(torch.empty(4 * hidden_size, input_size).uniform_(-k, k))
+        self.weight_hh_l0 = torch.nn.Parameter(torch.empty(4 * hidden_size, hidden_size).uniform_(-k, k))
+        self.bias_ih_l0 = torch.nn.Parameter(torch.empty(4 * hidden_size).uniform_(-k, k))
+        self.bias_hh_l0 = torch.nn.Parameter(torch.empty(4 * hidden_size).uniform_(-k, k))
+
+    def forward(self, x):
+        return _LSTMFn.apply(x, self.weight_ih_l0, self.weight_hh_l0, self.bias_ih_l0, self.bias_hh_l0), None
+
+
+class _AddFn(torch.autograd.Function):
+    @staticmethod
+    def forward(ctx, a, b):
+        return ops.add(a, b)
+
+    @staticmethod
+    def backward(ctx, dy):
+        return dy, dy
+
+
+def add(a, b):
+    """Residual connection ``a + b`` on the HIP add kernel."""
+    return _AddFn.apply(a, b)
+
+
+# --------------------------------------------------------------------------------------
 # Criterion
 # --------------------------------------------------------------------------------------
 class _CrossEntropyFn(torch.autograd.Function):

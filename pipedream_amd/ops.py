@@ -283,3 +283,98 @@ def conv3x3_weight_grad(x, dy, with_bias=True):
         lib.pd_conv3x3_wgrad_nhwc_f32(_ptr(x), _ptr(dy), _ptr(dw), _ptr(db), _ptr(ws), nbytes.value, n, h, wd, c, k,
                                       _cabi.stream_ptr())
     return dw, db
+
+
+# --------------------------------------------------------------------------------------
+# LSTM / embedding / residual add
+# --------------------------------------------------------------------------------------
+def add(a, b):
+    _check(a, "a")
+    _check(b, "b")
+    if a.shape != b.shape:
+        raise ValueError("add: shapes differ (%s vs %s)" % (tuple(a.shape), tuple(b.shape)))
+    if not _is_dense(a):
+        a = a.contiguous()
+    if b.stride() != a.stride():
+        b2 = torch.empty_like(a)
+        b2.copy_(b)
+        b = b2
+    y = torch.empty_like(a)
+    _cabi.lib().pd_add_f32(_ptr(a), _ptr(b), _ptr(y), a.numel(), _cabi.stream_ptr())
+    return y
+
+
+def lstm_forward(x, w_ih, w_hh, b_ih, b_hh):
+    """Single-layer, uni-directional LSTM over x[T,B,I] from zero state.
+    Returns (y[T,B,H], saved) where saved = (gates[T,B,4H] activated, c[T,B,H])."""
+    _check(x, "x")
+    if x.dim() != 3:
+        raise ValueError("lstm: input must be [T, B, I]")
+    T, B, I = x.shape
+    H = w_hh.shape[1]
+    if tuple(w_ih.shape) != (4 * H, I) or tuple(w_hh.shape) != (4 * H, H):
+        raise ValueError("lstm: weight shapes %s / %s do not fit input %d, hidden %d"
+                         % (tuple(w_ih.shape), tuple(w_hh.shape), I, H))
+    x2 = x.contiguous().view(T * B, I)
+    lib, s = _cabi.lib(), _cabi.stream_ptr
+    # input projection of all time steps at once
+    gates = gemm(x2, w_ih, trans_b=True).view(T, B, 4 * H)
+    y = torch.empty((T, B, H), dtype=torch.float32, device=x.device)
+    c = torch.empty((T, B, H), dtype=torch.float32, device=x.device)
+    for t in range(T):
+        if t > 0:
+            gemm(y[t - 1], w_hh, trans_b=True, out=gates[t], beta=1.0)
+        lib.pd_lstm_cell_fwd_f32(_ptr(gates[t]), _ptr(b_ih), _ptr(b_hh), _ptr(c[t - 1]) if t > 0 else None,
+                                 _ptr(c[t]), _ptr(y[t]), B, H, s())
+    return y, (gates, c)
+
+
+def lstm_backward(dy, x, y, gates, c, w_ih, w_hh, need_dx=True):
+    """Gradients of lstm_forward: (dx or None, dw_ih, dw_hh, db) with db = db_ih = db_hh."""
+    T, B, I = x.shape
+    H = w_hh.shape[1]
+    dy = dy.contiguous()
+    lib, s = _cabi.lib(), _cabi.stream_ptr
+    dgates = torch.empty((T, B, 4 * H), dtype=torch.float32, device=x.device)
+    dc = torch.empty((B, H), dtype=torch.float32, device=x.device)
+    dh_rec = None
+    for t in range(T - 1, -1, -1):
+        lib.pd_lstm_cell_bwd_f32(_ptr(gates[t]), _ptr(c[t - 1]) if t > 0 else None, _ptr(c[t]), _ptr(dy[t]),
+                                 _ptr(dh_rec), _ptr(dc), _ptr(dgates[t]), B, H, int(t == T - 1), s())
+        if t > 0:
+            dh_rec = gemm(dgates[t], w_hh)                      # [B,4H] @ [4H,H]
+    dg2 = dgates.view(T * B, 4 * H)
+    x2 = x.contiguous().view(T * B, I)
+    dw_ih = gemm(dg2, x2, trans_a=True)
+    # h_{t-1} for t >= 1 is y[t-1]; the t = 0 term has h = 0
+    if T > 1:
+        dw_hh = gemm(dgates[1:].view((T - 1) * B, 4 * H), y[:-1].view((T - 1) * B, H), trans_a=True)
+    else:
+        dw_hh = torch.zeros_like(w_hh)
+    db = colsum(dg2)
+    dx = gemm(dg2, w_ih).view(T, B, I) if need_dx else None
+    return dx, dw_ih, dw_hh, db
+
+
+def embedding_forward(ids, weight):
+    _check(ids, "ids", torch.int64)
+    _check(weight, "weight")
+    if weight.dim() != 2 or not weight.is_contiguous():
+        raise ValueError("embedding: weight must be a contiguous [V, D] matrix")
+    flat = ids.contiguous().view(-1)
+    V, D = weight.shape
+    out = torch.empty((flat.numel(), D), dtype=torch.float32, device=weight.device)
+    _cabi.lib().pd_embedding_fwd_f32(_ptr(flat), _ptr(weight), _ptr(out), flat.numel(), D, V, _cabi.stream_ptr())
+    return out.view(*ids.shape, D)
+
+
+def embedding_backward(ids, dout, num_embeddings, padding_idx=None):
+    _check(ids, "ids", torch.int64)
+    _check(dout, "dout")
+    flat = ids.contiguous().view(-1)
+    D = dout.shape[-1]
+    d2 = dout.contiguous().view(-1, D)
+    dw = torch.empty((num_embeddings, D), dtype=torch.float32, device=dout.device)
+    _cabi.lib().pd_embedding_bwd_f32(_ptr(flat), _ptr(d2), _ptr(dw), flat.numel(), D, num_embeddings,
+                                     -1 if padding_idx is None else int(padding_idx), _cabi.stream_ptr())
+    return dw
