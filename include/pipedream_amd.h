@@ -207,6 +207,50 @@ int pd_embedding_fwd_f32(const int64_t* ids, const float* weight, float* out, in
 int pd_embedding_bwd_f32(const int64_t* ids, const float* dout, float* dweight, int n_tokens, int D, int64_t V,
                          int64_t padding_idx, void* stream);
 
+/* ------------------------------------------------------------------------- *
+ * bf16 transformer stage (6 pre-LN layers, bf16 compute, fp32 master weights).
+ * The reference's checked-out branch has no such stage (PipeDream-2BW is on another
+ * branch, README.md:7-8); these entry points do for it what cuBLAS / ATen do for the
+ * torch.nn layers of the reference's stages (runtime/runtime.py:529-530, :606-608).
+ * bf16 tensors are passed as uint16_t*.
+ * ------------------------------------------------------------------------- */
+
+/* Strided-batched bf16 GEMM, fp32 accumulation on MFMA:
+ *   C = alpha * op(A) op(B) (+ bias[N]) (+ residual) (+ beta*C, fp32 output only)
+ * Layout flags as pd_gemm_f32.  C is bf16 (out_f32 = 0) or fp32.  Batch entry
+ * (o, i), o < batch_outer, i < batch_inner, offsets the operands by
+ * strides = {sa_o, sa_i, sb_o, sb_i, sc_o, sc_i} elements (NULL when unbatched); the
+ * residual shares C's offsets.  Leading dimensions, contiguous extents and A/B batch
+ * strides must be multiples of 8 elements. */
+int pd_gemm_bf16(int trans_a, int trans_b, int M, int N, int K,
+                 const uint16_t* A, int lda, const uint16_t* B, int ldb,
+                 void* C, int ldc, int out_f32, float alpha, float beta,
+                 const float* bias, const uint16_t* residual, int ldr,
+                 int batch_outer, int batch_inner, const int64_t* strides, void* stream);
+
+/* LayerNorm over the last dimension H (multiple of 8, <= 2048): bf16 in/out, fp32 affine
+ * parameters and statistics.  Backward writes dx and per-block partial sums of
+ * dgamma / dbeta, [pd_layernorm_bwd_partials(M)][H] each, to be summed with pd_colsum_f32. */
+int pd_layernorm_fwd_bf16(const uint16_t* x, const float* gamma, const float* beta, uint16_t* y,
+                          float* mean, float* rstd, int M, int H, float eps, void* stream);
+int pd_layernorm_bwd_partials(int M);
+int pd_layernorm_bwd_bf16(const uint16_t* dy, const uint16_t* x, const float* gamma, const float* mean,
+                          const float* rstd, uint16_t* dx, float* part_dgamma, float* part_dbeta,
+                          int M, int H, void* stream);
+
+/* Row softmax (row length multiple of 8, <= 2048) and its backward dx = y*(dy - sum(dy*y)). */
+int pd_softmax_fwd_bf16(const uint16_t* x, uint16_t* y, int64_t rows, int n, void* stream);
+int pd_softmax_bwd_bf16(const uint16_t* y, const uint16_t* dy, uint16_t* dx, int64_t rows, int n, void* stream);
+
+/* Exact (erf) GELU and its backward dx = dy * gelu'(x); element-wise add; casts; column sums
+ * of a bf16 matrix into fp32 partials out[splits][N]. */
+int pd_gelu_fwd_bf16(const uint16_t* x, uint16_t* y, uint64_t n, void* stream);
+int pd_gelu_bwd_bf16(const uint16_t* x, const uint16_t* dy, uint16_t* dx, uint64_t n, void* stream);
+int pd_add_bf16(const uint16_t* a, const uint16_t* b, uint16_t* y, uint64_t n, void* stream);
+int pd_cast_f32_to_bf16(const float* x, uint16_t* y, uint64_t n, void* stream);
+int pd_cast_bf16_to_f32(const uint16_t* x, float* y, uint64_t n, void* stream);
+int pd_colsum_bf16(const uint16_t* x, float* out, uint64_t M, int N, uint64_t ld, int splits, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

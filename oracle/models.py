@@ -175,3 +175,53 @@ class GnmtStage0(torch.nn.Module):
         out13 = out12 + out9
         out16 = self.layer16(self.layer15(out13))[0]
         return out16 + out13
+
+
+# --------------------------------------------------------------------------------------
+# bf16 pre-LN transformer stage (fp32 master parameters, bf16 activations and products)
+# --------------------------------------------------------------------------------------
+class TransformerLayerOracle(torch.nn.Module):
+    """Same parameter names as pipedream_amd.layers.TransformerLayer.  Every product takes
+    bf16 operands (weights rounded from the fp32 masters at use time); LayerNorm, softmax
+    and GELU are evaluated by torch's bf16 CPU kernels (fp32 internally, bf16 results)."""
+
+    def __init__(self, hidden, heads, ffn, eps=1e-5):
+        super(TransformerLayerOracle, self).__init__()
+        self.heads = heads
+        self.ln1 = torch.nn.LayerNorm(hidden, eps=eps)
+        self.qkv = torch.nn.Linear(hidden, 3 * hidden)
+        self.proj = torch.nn.Linear(hidden, hidden)
+        self.ln2 = torch.nn.LayerNorm(hidden, eps=eps)
+        self.fc1 = torch.nn.Linear(hidden, ffn)
+        self.fc2 = torch.nn.Linear(ffn, hidden)
+
+    @staticmethod
+    def _lin(x, m):
+        return torch.nn.functional.linear(x, m.weight.bfloat16(), m.bias.bfloat16())
+
+    @staticmethod
+    def _ln(x, m):
+        return torch.nn.functional.layer_norm(x.float(), x.shape[-1:], m.weight, m.bias, m.eps).bfloat16()
+
+    def forward(self, x):
+        B, S, H = x.shape
+        d = H // self.heads
+        qkv = self._lin(self._ln(x, self.ln1), self.qkv)
+        q, k, v = [t.reshape(B, S, self.heads, d).transpose(1, 2) for t in qkv.split(H, dim=-1)]
+        p = torch.softmax((q @ k.transpose(-1, -2)) * (1.0 / d ** 0.5), dim=-1)
+        att = (p @ v).transpose(1, 2).reshape(B, S, H)
+        x = self._lin(att, self.proj) + x
+        f = torch.nn.functional.gelu(self._lin(self._ln(x, self.ln2), self.fc1))
+        return self._lin(f, self.fc2) + x
+
+
+class TransformerStage0(torch.nn.Module):
+    def __init__(self, n_layers=6, hidden=1024, heads=16, ffn=4096):
+        super(TransformerStage0, self).__init__()
+        self.layers = torch.nn.ModuleList([TransformerLayerOracle(hidden, heads, ffn) for _ in range(n_layers)])
+
+    def forward(self, x):
+        x = x.bfloat16()
+        for layer in self.layers:
+            x = layer(x)
+        return x

@@ -79,6 +79,19 @@ SIGNATURES = {
     "pd_add_f32": (_i, [_vp, _vp, _vp, _u64, _vp], True),
     "pd_embedding_fwd_f32": (_i, [_vp, _vp, _vp, _i, _i, _i64, _vp], True),
     "pd_embedding_bwd_f32": (_i, [_vp, _vp, _vp, _i, _i, _i64, _i64, _vp], True),
+    "pd_gemm_bf16": (_i, [_i, _i, _i, _i, _i, _vp, _i, _vp, _i, _vp, _i, _i, _f, _f, _vp, _vp, _i, _i, _i,
+                          ctypes.POINTER(ctypes.c_int64), _vp], True),
+    "pd_layernorm_fwd_bf16": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _f, _vp], True),
+    "pd_layernorm_bwd_partials": (_i, [_i], False),
+    "pd_layernorm_bwd_bf16": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _vp], True),
+    "pd_softmax_fwd_bf16": (_i, [_vp, _vp, _i64, _i, _vp], True),
+    "pd_softmax_bwd_bf16": (_i, [_vp, _vp, _vp, _i64, _i, _vp], True),
+    "pd_gelu_fwd_bf16": (_i, [_vp, _vp, _u64, _vp], True),
+    "pd_gelu_bwd_bf16": (_i, [_vp, _vp, _vp, _u64, _vp], True),
+    "pd_add_bf16": (_i, [_vp, _vp, _vp, _u64, _vp], True),
+    "pd_cast_f32_to_bf16": (_i, [_vp, _vp, _u64, _vp], True),
+    "pd_cast_bf16_to_f32": (_i, [_vp, _vp, _u64, _vp], True),
+    "pd_colsum_bf16": (_i, [_vp, _vp, _u64, _i, _u64, _i, _vp], True),
     "pd_xent_bwd_f32": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i64, _vp], True),
 }
 

@@ -65,7 +65,7 @@ def _is_dense(t):
 class WeightArena(object):
     """``num_versions`` flat slots + the integer ring that orders them."""
 
-    def __init__(self, modules, master_parameters, num_versions):
+    def __init__(self, modules, master_parameters, num_versions, bf16_image=False):
         self._lib = _cabi.lib()
         self.modules = list(modules)
         self.num_versions = int(num_versions)
@@ -164,6 +164,26 @@ class WeightArena(object):
                 e.tensor.data = live
         self._lib.pd_ring_broadcast(self._ring, self.live_slot, self.slot_bytes, _cabi.stream_ptr())
         self._point_live_at(self.live_slot)
+
+        # Optional bf16 image of the master section, one per slot, with the same element
+        # offsets: what bf16-compute layers multiply with.  The fused optimizer step keeps
+        # it current (it writes the bf16 value next to every fp32 parameter it produces).
+        self.bf16_image = None
+        if bf16_image:
+            n = self.master_bytes // 4
+            self.bf16_image = [torch.empty(n, dtype=torch.bfloat16, device=device) for _ in range(self.num_versions)]
+            for s in range(self.num_versions):
+                self._lib.pd_cast_f32_to_bf16(ctypes.c_void_p(self.slot_ptr(s)),
+                                              ctypes.c_void_p(self.bf16_image[s].data_ptr()), n, _cabi.stream_ptr())
+            for e in self.masters:
+                lo = e.offset // 4
+                views = []
+                for s in range(self.num_versions):
+                    flat = self.bf16_image[s][lo:lo + e.numel]
+                    views.append(flat.view(e.shape) if e.tensor.is_contiguous() else flat.as_strided(e.shape, e.stride))
+                # layers look these up through the parameter object
+                e.tensor._pd_bf16_views = views
+                e.tensor._pd_arena = self
 
     def __del__(self):
         ring = getattr(self, "_ring", None)

@@ -41,7 +41,7 @@ class _FusedOptimizer(torch.optim.Optimizer):
         # flat state buffers share the slot layout of the master section
         self._flat_state = [torch.zeros(n, dtype=torch.float32, device=device) for _ in self._state_names]
         self._descs = (_cabi.TensorDesc * max(1, len(masters)))()
-        self.bf16_copy = None  # optional flat bf16 image of the master section (set by the wrapper)
+        self.bf16_copy = arena.bf16_image  # per-slot flat bf16 images of the master section, or None
 
     # -- helpers -----------------------------------------------------------------------
     def _state_view(self, which, p):
@@ -155,7 +155,13 @@ class SGD(_FusedOptimizer):
             for p in group["params"]:
                 if p.grad is None:
                     e = self._index[id(p)]
-                    e.views[out_slot].copy_(e.views[in_slot])
+                    self._lib.pd_copy(ctypes.c_void_p(e.views[out_slot].data_ptr()),
+                                      ctypes.c_void_p(e.views[in_slot].data_ptr()), e.nbytes, _cabi.stream_ptr())
+                    if self.bf16_copy is not None:
+                        views = e.tensor._pd_bf16_views
+                        self._lib.pd_cast_f32_to_bf16(ctypes.c_void_p(e.views[out_slot].data_ptr()),
+                                                      ctypes.c_void_p(views[out_slot].data_ptr()), e.numel,
+                                                      _cabi.stream_ptr())
 
 
 class Adam(_FusedOptimizer):

@@ -324,6 +324,123 @@ def add(a, b):
 
 
 # --------------------------------------------------------------------------------------
+# bf16 pre-LN transformer layer (fp32 master parameters, bf16 compute)
+# --------------------------------------------------------------------------------------
+def _accumulate(p, fresh_fn, acc_fn):
+    """Weight-gradient accumulation fused into the producing kernel: the first micro-batch
+    of an update interval creates ``p.grad`` (fp32), later ones add into it in the GEMM /
+    column-sum epilogue, so no separate accumulate pass runs."""
+    if p.grad is None:
+        p.grad = fresh_fn()
+    else:
+        acc_fn(p.grad)
+
+
+class _TransformerLayerFn(torch.autograd.Function):
+    """x -> x + Attn(LN1(x)) -> . + FFN(LN2(.)), hand-written backward; every matrix product is
+    the bf16 MFMA GEMM, every reduction / pointwise op one of the bf16 HIP kernels."""
+
+    @staticmethod
+    def forward(ctx, x, heads, eps, ln1_w, ln1_b, qkv_w, qkv_b, o_w, o_b, ln2_w, ln2_b, fc1_w, fc1_b, fc2_w, fc2_b):
+        B, S, H = x.shape
+        x2d = x.contiguous().view(B * S, H)
+        bw = ops.bf16_weight
+        h1, mean1, rstd1 = ops.layernorm_forward(x2d, ln1_w, ln1_b, eps)
+        qkv = ops.gemm_bf16(h1, bw(qkv_w), trans_b=True, bias=qkv_b)
+        att, probs = ops.attention_forward(qkv, B, S, heads)
+        x2 = ops.gemm_bf16(att, bw(o_w), trans_b=True, bias=o_b, residual=x2d)
+        h2, mean2, rstd2 = ops.layernorm_forward(x2, ln2_w, ln2_b, eps)
+        f = ops.gemm_bf16(h2, bw(fc1_w), trans_b=True, bias=fc1_b)
+        g = ops.gelu(f)
+        y = ops.gemm_bf16(g, bw(fc2_w), trans_b=True, bias=fc2_b, residual=x2)
+        ctx.dims = (B, S, H, heads)
+        ctx.params = (ln1_w, ln1_b, qkv_w, qkv_b, o_w, o_b, ln2_w, ln2_b, fc1_w, fc1_b, fc2_w, fc2_b)
+        ctx.save_for_backward(x2d, h1, mean1, rstd1, qkv, probs, att, x2, h2, mean2, rstd2, f, g)
+        return y.view(B, S, H)
+
+    @staticmethod
+    def backward(ctx, dy):
+        B, S, H, heads = ctx.dims
+        x2d, h1, mean1, rstd1, qkv, probs, att, x2, h2, mean2, rstd2, f, g = ctx.saved_tensors
+        ln1_w, ln1_b, qkv_w, qkv_b, o_w, o_b, ln2_w, ln2_b, fc1_w, fc1_b, fc2_w, fc2_b = ctx.params
+        bw = ops.bf16_weight
+        dy2 = dy.contiguous().view(B * S, H)
+
+        def linear_backward(d_out, inp, w, b):
+            # parameters are read (and their bf16 image taken) at backward time: the version
+            # load_old_params made current
+            _accumulate(w, lambda: ops.gemm_bf16(d_out, inp, trans_a=True, out_f32=True),
+                        lambda acc: ops.gemm_bf16(d_out, inp, trans_a=True, out=acc, beta=1.0))
+            _accumulate(b, lambda: ops.colsum_bf16(d_out), lambda acc: ops.colsum_bf16(d_out, acc))
+            return ops.gemm_bf16(d_out, bw(w))
+
+        def layernorm_backward(d_out, inp, w, b, mean, rstd):
+            if w.grad is None:
+                dx, dg, db = ops.layernorm_backward(d_out, inp, w, mean, rstd)
+                w.grad, b.grad = dg, db
+            else:
+                dx, _, _ = ops.layernorm_backward(d_out, inp, w, mean, rstd, w.grad, b.grad)
+            return dx
+
+        # y = fc2(gelu(fc1(LN2(x2)))) + x2
+        dg = linear_backward(dy2, g, fc2_w, fc2_b)
+        df = ops.gelu_backward(f, dg)
+        dh2 = linear_backward(df, h2, fc1_w, fc1_b)
+        dx2 = ops.add_bf16(layernorm_backward(dh2, x2, ln2_w, ln2_b, mean2, rstd2), dy2)
+        # x2 = o(attn(qkv(LN1(x)))) + x
+        datt = linear_backward(dx2, att, o_w, o_b)
+        dqkv = ops.attention_backward(datt, qkv, probs, B, S, heads)
+        dh1 = linear_backward(dqkv, h1, qkv_w, qkv_b)
+        dx = ops.add_bf16(layernorm_backward(dh1, x2d, ln1_w, ln1_b, mean1, rstd1), dx2)
+        return (dx.view(B, S, H), None, None) + (None,) * 12
+
+
+class TransformerLayer(torch.nn.Module):
+    """Pre-LayerNorm transformer layer: multi-head self-attention (no mask) and a GELU
+    feed-forward block, each with a residual connection.  Parameters are fp32 masters
+    (``ln1``, ``qkv``, ``proj``, ``ln2``, ``fc1``, ``fc2`` with torch's ``weight``/``bias``
+    names); activations are bf16 ``[batch, seq, hidden]``.  Weight gradients are produced in
+    fp32 and accumulated across micro-batches inside the producing kernels, so autograd
+    sees only the activation path."""
+
+    def __init__(self, hidden, heads, ffn, eps=1e-5):
+        super(TransformerLayer, self).__init__()
+        self.hidden, self.heads, self.ffn, self.eps = hidden, heads, ffn, eps
+        self.ln1 = torch.nn.LayerNorm(hidden, eps=eps)
+        self.qkv = torch.nn.Linear(hidden, 3 * hidden)
+        self.proj = torch.nn.Linear(hidden, hidden)
+        self.ln2 = torch.nn.LayerNorm(hidden, eps=eps)
+        self.fc1 = torch.nn.Linear(hidden, ffn)
+        self.fc2 = torch.nn.Linear(ffn, hidden)
+
+    def forward(self, x):
+        # the torch.nn members are parameter containers only; their forward is never called
+        return _TransformerLayerFn.apply(
+            x, self.heads, self.eps, self.ln1.weight, self.ln1.bias, self.qkv.weight, self.qkv.bias,
+            self.proj.weight, self.proj.bias, self.ln2.weight, self.ln2.bias, self.fc1.weight, self.fc1.bias,
+            self.fc2.weight, self.fc2.bias)
+
+
+class _CastFn(torch.autograd.Function):
+    @staticmethod
+    def forward(ctx, x, to_bf16):
+        ctx.to_bf16 = to_bf16
+        return ops.cast_bf16(x) if to_bf16 else ops.cast_f32(x)
+
+    @staticmethod
+    def backward(ctx, dy):
+        return (ops.cast_f32(dy) if ctx.to_bf16 else ops.cast_bf16(dy)), None
+
+
+def to_bf16(x):
+    return x if x.dtype == torch.bfloat16 else _CastFn.apply(x, True)
+
+
+def to_f32(x):
+    return x if x.dtype == torch.float32 else _CastFn.apply(x, False)
+
+
+# --------------------------------------------------------------------------------------
 # Criterion
 # --------------------------------------------------------------------------------------
 class _CrossEntropyFn(torch.autograd.Function):

@@ -378,3 +378,194 @@ def embedding_backward(ids, dout, num_embeddings, padding_idx=None):
     _cabi.lib().pd_embedding_bwd_f32(_ptr(flat), _ptr(d2), _ptr(dw), flat.numel(), D, num_embeddings,
                                      -1 if padding_idx is None else int(padding_idx), _cabi.stream_ptr())
     return dw
+
+
+# --------------------------------------------------------------------------------------
+# bf16 transformer ops
+# --------------------------------------------------------------------------------------
+BF16 = torch.bfloat16
+
+
+def cast_bf16(x):
+    _check(x, "x")
+    x = x.contiguous()
+    y = torch.empty(x.shape, dtype=BF16, device=x.device)
+    _cabi.lib().pd_cast_f32_to_bf16(_ptr(x), _ptr(y), x.numel(), _cabi.stream_ptr())
+    return y
+
+
+def cast_f32(x):
+    _check(x, "x", BF16)
+    x = x.contiguous()
+    y = torch.empty(x.shape, dtype=torch.float32, device=x.device)
+    _cabi.lib().pd_cast_bf16_to_f32(_ptr(x), _ptr(y), x.numel(), _cabi.stream_ptr())
+    return y
+
+
+def bf16_weight(p):
+    """bf16 image of a master parameter: the ring's image of the loaded slot when the
+    optimizer keeps one, otherwise a fresh cast."""
+    views = getattr(p, "_pd_bf16_views", None)
+    if views is not None:
+        return views[p._pd_arena.live_slot]
+    return cast_bf16(p.detach())
+
+
+def _mat_bf16(t, name):
+    _check(t, name, BF16)
+    if t.dim() != 2 or t.stride(1) != 1:
+        raise ValueError("%s must be a row-major 2-D bf16 matrix" % name)
+    return t
+
+
+def gemm_bf16(a, b, trans_a=False, trans_b=False, out=None, out_f32=False, alpha=1.0, beta=0.0, bias=None,
+              residual=None):
+    """out[M,N] = alpha * op(a) op(b) (+bias) (+residual) (+beta*out for fp32 out)."""
+    _mat_bf16(a, "a")
+    _mat_bf16(b, "b")
+    M, K = (a.size(1), a.size(0)) if trans_a else (a.size(0), a.size(1))
+    Kb, N = (b.size(1), b.size(0)) if trans_b else (b.size(0), b.size(1))
+    if K != Kb:
+        raise ValueError("gemm_bf16: inner dimensions differ (%d vs %d)" % (K, Kb))
+    if out is None:
+        out = torch.empty((M, N), dtype=torch.float32 if out_f32 else BF16, device=a.device)
+    else:
+        out_f32 = out.dtype == torch.float32
+        if tuple(out.shape) != (M, N) or out.stride(1) != 1 or not out.is_cuda:
+            raise ValueError("gemm_bf16: bad out tensor")
+    if residual is not None:
+        _mat_bf16(residual, "residual")
+        if tuple(residual.shape) != (M, N):
+            raise ValueError("gemm_bf16: residual shape")
+    if bias is not None:
+        _check(bias, "bias")
+    _cabi.lib().pd_gemm_bf16(int(trans_a), int(trans_b), M, N, K, _ptr(a), a.stride(0), _ptr(b), b.stride(0),
+                             _ptr(out), out.stride(0), int(out_f32), float(alpha), float(beta), _ptr(bias),
+                             _ptr(residual), residual.stride(0) if residual is not None else 0, 1, 1, None,
+                             _cabi.stream_ptr())
+    return out
+
+
+def _batched(ta, tb, M, N, K, A, a_off, lda, B, b_off, ldb, C, c_off, ldc, alpha, bo, bi, strides):
+    arr = (ctypes.c_int64 * 6)(*strides)
+    es = 2
+    _cabi.lib().pd_gemm_bf16(int(ta), int(tb), M, N, K, _vp(A.data_ptr() + a_off * es), lda,
+                             _vp(B.data_ptr() + b_off * es), ldb, _vp(C.data_ptr() + c_off * es), ldc, 0,
+                             float(alpha), 0.0, None, None, 0, bo, bi, arr, _cabi.stream_ptr())
+
+
+def attention_forward(qkv, batch, seq, heads):
+    """qkv: [batch*seq, 3H] bf16 (Q | K | V, heads contiguous inside each).  Returns
+    (ctx [batch*seq, H], probs [batch, heads, seq, seq])."""
+    _mat_bf16(qkv, "qkv")
+    H = qkv.size(1) // 3
+    d = H // heads
+    if qkv.size(0) != batch * seq or H * 3 != qkv.size(1) or d * heads != H or not qkv.is_contiguous():
+        raise ValueError("attention: qkv shape %s does not fit batch %d seq %d heads %d"
+                         % (tuple(qkv.shape), batch, seq, heads))
+    dev = qkv.device
+    probs = torch.empty((batch, heads, seq, seq), dtype=BF16, device=dev)
+    ctx = torch.empty((batch * seq, H), dtype=BF16, device=dev)
+    scale = 1.0 / (d ** 0.5)
+    ld = 3 * H
+    # scores = scale * Q K^T
+    _batched(0, 1, seq, seq, d, qkv, 0, ld, qkv, H, ld, probs, 0, seq, scale, batch, heads,
+             (seq * ld, d, seq * ld, d, heads * seq * seq, seq * seq))
+    _cabi.lib().pd_softmax_fwd_bf16(_ptr(probs), _ptr(probs), batch * heads * seq, seq, _cabi.stream_ptr())
+    # ctx = P V
+    _batched(0, 0, seq, d, seq, probs, 0, seq, qkv, 2 * H, ld, ctx, 0, H, 1.0, batch, heads,
+             (heads * seq * seq, seq * seq, seq * ld, d, seq * H, d))
+    return ctx, probs
+
+
+def attention_backward(dctx, qkv, probs, batch, seq, heads):
+    """Gradient with respect to qkv."""
+    _mat_bf16(dctx, "dctx")
+    H = qkv.size(1) // 3
+    d = H // heads
+    dctx = dctx.contiguous()
+    dev = qkv.device
+    ld = 3 * H
+    scale = 1.0 / (d ** 0.5)
+    dqkv = torch.empty_like(qkv)
+    dP = torch.empty_like(probs)
+    sP = (heads * seq * seq, seq * seq)
+    # dP = dctx V^T
+    _batched(0, 1, seq, seq, d, dctx, 0, H, qkv, 2 * H, ld, dP, 0, seq, 1.0, batch, heads,
+             (seq * H, d, seq * ld, d) + sP)
+    # dV = P^T dctx
+    _batched(1, 0, seq, d, seq, probs, 0, seq, dctx, 0, H, dqkv, 2 * H, ld, 1.0, batch, heads,
+             sP + (seq * H, d, seq * ld, d))
+    # dS = P * (dP - sum(dP * P)), in place
+    _cabi.lib().pd_softmax_bwd_bf16(_ptr(probs), _ptr(dP), _ptr(dP), batch * heads * seq, seq, _cabi.stream_ptr())
+    # dQ = scale * dS K ; dK = scale * dS^T Q
+    _batched(0, 0, seq, d, seq, dP, 0, seq, qkv, H, ld, dqkv, 0, ld, scale, batch, heads,
+             sP + (seq * ld, d, seq * ld, d))
+    _batched(1, 0, seq, d, seq, dP, 0, seq, qkv, 0, ld, dqkv, H, ld, scale, batch, heads,
+             sP + (seq * ld, d, seq * ld, d))
+    return dqkv
+
+
+def layernorm_forward(x, gamma, beta, eps=1e-5):
+    _mat_bf16(x, "x")
+    M, H = x.shape
+    y = torch.empty_like(x)
+    mean = torch.empty(M, dtype=torch.float32, device=x.device)
+    rstd = torch.empty(M, dtype=torch.float32, device=x.device)
+    _cabi.lib().pd_layernorm_fwd_bf16(_ptr(x), _ptr(gamma), _ptr(beta), _ptr(y), _ptr(mean), _ptr(rstd), M, H,
+                                      float(eps), _cabi.stream_ptr())
+    return y, mean, rstd
+
+
+def layernorm_backward(dy, x, gamma, mean, rstd, dgamma_acc=None, dbeta_acc=None):
+    """Returns dx; dgamma/dbeta are added to the given fp32 accumulators or returned fresh."""
+    M, H = x.shape
+    lib = _cabi.lib()
+    nb = lib.pd_layernorm_bwd_partials(M)
+    dx = torch.empty_like(x)
+    pg = torch.empty((nb, H), dtype=torch.float32, device=x.device)
+    pb = torch.empty((nb, H), dtype=torch.float32, device=x.device)
+    lib.pd_layernorm_bwd_bf16(_ptr(dy), _ptr(x), _ptr(gamma), _ptr(mean), _ptr(rstd), _ptr(dx), _ptr(pg), _ptr(pb),
+                              M, H, _cabi.stream_ptr())
+    outs = []
+    for part, acc in ((pg, dgamma_acc), (pb, dbeta_acc)):
+        if acc is None:
+            acc = torch.empty(H, dtype=torch.float32, device=x.device)
+            lib.pd_colsum_f32(_ptr(part), _ptr(acc), nb, H, H, 1, 0.0, _cabi.stream_ptr())
+        else:
+            lib.pd_colsum_f32(_ptr(part), _ptr(acc), nb, H, H, 1, 1.0, _cabi.stream_ptr())
+        outs.append(acc)
+    return dx, outs[0], outs[1]
+
+
+def gelu(x):
+    y = torch.empty_like(x)
+    _cabi.lib().pd_gelu_fwd_bf16(_ptr(x), _ptr(y), x.numel(), _cabi.stream_ptr())
+    return y
+
+
+def gelu_backward(x, dy):
+    dx = torch.empty_like(x)
+    _cabi.lib().pd_gelu_bwd_bf16(_ptr(x), _ptr(dy), _ptr(dx), x.numel(), _cabi.stream_ptr())
+    return dx
+
+
+def add_bf16(a, b):
+    y = torch.empty_like(a)
+    _cabi.lib().pd_add_bf16(_ptr(a), _ptr(b), _ptr(y), a.numel(), _cabi.stream_ptr())
+    return y
+
+
+def colsum_bf16(x, acc=None):
+    """fp32 column sums of a bf16 matrix; added to ``acc`` when given."""
+    M, N = x.shape
+    lib = _cabi.lib()
+    splits = min(256, max(1, M // 256))
+    part = torch.empty((splits, N), dtype=torch.float32, device=x.device)
+    lib.pd_colsum_bf16(_ptr(x), _ptr(part), M, N, x.stride(0), splits, _cabi.stream_ptr())
+    if acc is None:
+        acc = torch.empty(N, dtype=torch.float32, device=x.device)
+        lib.pd_colsum_f32(_ptr(part), _ptr(acc), splits, N, N, 1, 0.0, _cabi.stream_ptr())
+    else:
+        lib.pd_colsum_f32(_ptr(part), _ptr(acc), splits, N, N, 1, 1.0, _cabi.stream_ptr())
+    return acc

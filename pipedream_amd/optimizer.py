@@ -80,12 +80,13 @@ class OptimizerWithWeightStashing(torch.optim.Optimizer):
     selects the base optimizer: ``'SGD'`` or ``'Adam'`` (the two the reference's
     runtime/sgd.py and runtime/adam.py use).  ``update_interval`` (not in the
     reference) decouples gradient accumulation from ``num_versions`` for 2BW-style
-    double buffering; left at ``None`` it follows the reference rule.
+    double buffering; left at ``None`` it follows the reference rule.  ``bf16_image`` (not
+    in the reference) keeps a bf16 copy of every weight version for bf16-compute stages.
     """
 
     def __init__(self, optim_name, modules, master_parameters, model_parameters,
                  loss_scale, num_versions, verbose_freq=0, macrobatch=False,
-                 update_interval=None, **optimizer_args):
+                 update_interval=None, bf16_image=False, **optimizer_args):
         if optim_name not in BASE_OPTIMIZERS:
             raise NotImplementedError(
                 "optim_name %r has no fused HIP kernel (available: %s)" % (optim_name, sorted(BASE_OPTIMIZERS)))
@@ -109,7 +110,7 @@ class OptimizerWithWeightStashing(torch.optim.Optimizer):
                 flat_masters.extend(item["params"])
             else:
                 flat_masters.append(item)
-        self.arena = WeightArena(self.modules, flat_masters, num_versions)
+        self.arena = WeightArena(self.modules, flat_masters, num_versions, bf16_image=bf16_image)
         self.base_optimizer = BASE_OPTIMIZERS[optim_name](master_parameters, arena=self.arena, **optimizer_args)
         self.latest_version = Version()
         self.current_version = Version()

@@ -12,7 +12,7 @@ class SGDWithWeightStashing(OptimizerWithWeightStashing):
     def __init__(self, modules, master_parameters, model_parameters,
                  loss_scale, num_versions, lr=required, momentum=0,
                  dampening=0, weight_decay=0, nesterov=False, verbose_freq=0,
-                 macrobatch=False, update_interval=None):
+                 macrobatch=False, update_interval=None, bf16_image=False):
         super(SGDWithWeightStashing, self).__init__(
             optim_name='SGD',
             modules=modules, master_parameters=master_parameters,
@@ -20,5 +20,5 @@ class SGDWithWeightStashing(OptimizerWithWeightStashing):
             num_versions=num_versions, lr=lr, momentum=momentum,
             dampening=dampening, weight_decay=weight_decay,
             nesterov=nesterov, verbose_freq=verbose_freq,
-            macrobatch=macrobatch, update_interval=update_interval,
+            macrobatch=macrobatch, update_interval=update_interval, bf16_image=bf16_image,
         )
