@@ -28,6 +28,9 @@ BATCH = 64
 STASH_DEPTH = 4
 SGD_KW = dict(lr=0.01, momentum=0.9, weight_decay=5e-4)
 PEAK_FP32_MFMA_TFLOPS = 157.3
+# HBM bytes per launch of the dominant kernel, from the rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE
+# runs summarised under profiles/ (None until measured for the current kernel).
+MEASURED_TRAFFIC_BYTES = None
 
 
 def build_stage():
@@ -135,6 +138,25 @@ def gpu_run(steps, warmup):
     return elapsed, stats, opt
 
 
+def pmc_probe():
+    """Workload for `rocprofv3 --pmc FETCH_SIZE` / `--pmc WRITE_SIZE` runs: a plain copy of
+    known size (calibrates the counters: pd_copy_kernel moves 1 GiB in and 1 GiB out per
+    launch) followed by two steady-state steps of the benchmark stage, so the per-dispatch
+    counter values of conv3x3_fwd_kernel cover exactly the launch mix of the timed region."""
+    import ctypes
+    import torch
+    from pipedream_amd import _cabi
+    n = 1 << 30
+    src = torch.empty(n, dtype=torch.uint8, device="cuda").fill_(1)
+    dst = torch.empty(n, dtype=torch.uint8, device="cuda")
+    for _ in range(3):
+        _cabi.lib().pd_copy(ctypes.c_void_p(dst.data_ptr()), ctypes.c_void_p(src.data_ptr()), n, _cabi.stream_ptr())
+    torch.cuda.synchronize()
+    del src, dst
+    gpu_run(steps=2, warmup=1)
+    print("pmc probe done")
+
+
 def optimizer_bandwidth():
     """Fused stash+SGD step on a VGG16-sized flat parameter set (138 357 544 fp32 values,
     20 algorithmic bytes each), timed with HIP events on the launch stream."""
@@ -198,6 +220,10 @@ def main():
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--pmc-probe", action="store_true",
+                    help="run the counter-calibration copy and two benchmark steps, print no JSON")
+    ap.add_argument("--traffic-bytes", type=float, default=None,
+                    help="HBM bytes per launch of the dominant kernel from the PMC runs (see profiles/)")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this build measures one GPU only (one stage's share of the pipeline at its "
@@ -206,6 +232,9 @@ def main():
     if not torch.cuda.is_available():
         sys.exit("bench.py: no HIP device; the product path has no CPU fallback")
 
+    if args.pmc_probe:
+        pmc_probe()
+        return
     elapsed, stats, _ = gpu_run(args.steps, args.warmup)
     conv = stats["conv3x3_fwd_kernel"]
     achieved = conv["rate"] / 1e12
@@ -226,7 +255,8 @@ def main():
                                "1F1B with 4 minibatches in flight",
                    "global_batch": BATCH, "parallelism": "1 stage on 1 GPU"},
         "roofline": {"bound": "mfma", "achieved": achieved, "peak": PEAK_FP32_MFMA_TFLOPS, "unit": "TFLOP/s",
-                     "frac": achieved / PEAK_FP32_MFMA_TFLOPS, "traffic": None,
+                     "frac": achieved / PEAK_FP32_MFMA_TFLOPS,
+                     "traffic": args.traffic_bytes if args.traffic_bytes is not None else MEASURED_TRAFFIC_BYTES,
                      "kernel": "conv3x3_fwd_kernel<.,.,16> (forward + input gradient)",
                      "launches": conv["launches"], "avg_us": conv["avg_us"],
                      "flop_per_launch": conv["work_per_launch"]},

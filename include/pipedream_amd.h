@@ -175,13 +175,19 @@ int pd_xent_bwd_f32(const float* logits, const int64_t* target, const float* lse
 int pd_conv3x3_fwd_nhwc_f32(const float* x, const float* w, const float* bias, float* y,
                             int N, int H, int W, int C, int K, int relu, void* stream);
 /* out[c][r][s][k] = w[k][2-r][2-s][c]: with this filter the forward kernel computes the
- * input gradient, dX = conv3x3_fwd(dY, rot180(w)) (no bias, no ReLU). */
+ * input gradient. */
 int pd_conv3x3_filter_rot180_f32(const float* w, float* out, int K, int C, void* stream);
+/* Input gradient dx[N,H,W,C] = conv3x3(dy[N,H,W,K], w_rot[C][3][3][K]).  If relu_out is not
+ * NULL it is the forward output of the fused conv+ReLU layer and dy is taken as 0 where
+ * relu_out <= 0 (the ReLU backward applied while the tile is loaded). */
+int pd_conv3x3_dgrad_nhwc_f32(const float* dy, const float* w_rot, const float* relu_out, float* dx,
+                              int N, int H, int W, int K, int C, void* stream);
 /* Weight and (optional, dbias may be NULL) bias gradient of the same convolution:
  * dw[k][r][s][c] = sum_{n,y,x} dy[n,y,x,k] * x[n,y+r-1,x+s-1,c].  Deterministic two-pass
- * reduction through a caller-provided workspace of pd_conv3x3_wgrad_workspace_bytes(). */
+ * reduction through a caller-provided workspace of pd_conv3x3_wgrad_workspace_bytes().
+ * relu_out (may be NULL) masks dy as in pd_conv3x3_dgrad_nhwc_f32. */
 int pd_conv3x3_wgrad_workspace_bytes(int N, int H, int W, int C, int K, uint64_t* bytes);
-int pd_conv3x3_wgrad_nhwc_f32(const float* x, const float* dy, float* dw, float* dbias,
+int pd_conv3x3_wgrad_nhwc_f32(const float* x, const float* dy, const float* relu_out, float* dw, float* dbias,
                               void* workspace, uint64_t workspace_bytes,
                               int N, int H, int W, int C, int K, void* stream);
 

@@ -41,18 +41,23 @@ struct ConvArgs {
     const float* x;     // [N,H,W,C]
     const float* w;     // [K,3,3,C]
     const float* bias;  // [K] or null
+    const float* mask;  // [N,H,W,C] or null: x is taken as 0 where mask <= 0 (fused ReLU backward)
     float* y;           // [N,H,W,K]
     int N, H, W, C, K;
     int relu;
     int tiles_x, tiles_y;
+    int n_tiles, k_blocks, tiles_per_xcd;
     int c_vec;          // C % 4 == 0 and x/w 16-byte aligned: 128-bit global loads
 };
+
+constexpr int N_XCD = 8;  // MI355X: 8 accelerator dies, each with its own L2; workgroups are
+                          // handed to them round-robin by linear workgroup id
 
 // Global -> register staging of one reduction chunk (input halo tile + filter slice).
 // All loads of a chunk are issued back to back (fixed trip counts, no divergent
 // branches: out-of-range elements read a safe address and are zeroed by a select), so
 // a thread has ~15 128-bit loads in flight instead of one.
-template <int TH, int TW, int CC>
+template <int TH, int TW, int CC, bool MASK>
 struct FwdStage {
     static constexpr int HW_ = TW + 2;
     static constexpr int HALO = (TH + 2) * (TW + 2);
@@ -64,8 +69,8 @@ struct FwdStage {
     float4_t rin[IN_ITERS];
     float4_t rw[W_ITERS];
 
-    __device__ __forceinline__ void load(const ConvArgs& a, const float* __restrict__ xn, int y0, int x0, int k0,
-                                         int c0, int tid) {
+    __device__ __forceinline__ void load(const ConvArgs& a, const float* __restrict__ xn,
+                                         const float* __restrict__ mn, int y0, int x0, int k0, int c0, int tid) {
         const float4_t zero = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
         for (int it = 0; it < IN_ITERS; ++it) {
@@ -74,13 +79,27 @@ struct FwdStage {
             const int gy = y0 + p / HW_ - 1, gx = x0 + p % HW_ - 1;
             const int c = c0 + q4;
             const bool ok = id < HALO * Q && gy >= 0 && gy < a.H && gx >= 0 && gx < a.W && c < a.C;
-            const float* src = ok ? xn + ((size_t)gy * a.W + gx) * a.C + c : xn;
+            const size_t off = ok ? ((size_t)gy * a.W + gx) * a.C + c : 0;
+            const float* src = xn + off;
             float4_t v;
             if (a.c_vec) {
                 v = *(const float4_t*)src;
             } else {
 #pragma unroll
                 for (int j = 0; j < 4; ++j) v[j] = (ok && c + j < a.C) ? src[j] : 0.f;
+            }
+            if (MASK) {
+                // gradient of a fused ReLU: dY counts only where the forward output was positive
+                const float* msrc = mn + off;
+                float4_t m;
+                if (a.c_vec) {
+                    m = *(const float4_t*)msrc;
+                } else {
+#pragma unroll
+                    for (int j = 0; j < 4; ++j) m[j] = (ok && c + j < a.C) ? msrc[j] : 0.f;
+                }
+#pragma unroll
+                for (int j = 0; j < 4; ++j) v[j] = m[j] > 0.f ? v[j] : 0.f;
             }
             rin[it] = ok ? v : zero;
         }
@@ -117,11 +136,11 @@ struct FwdStage {
     }
 };
 
-template <int TH, int TW, int CC>
+template <int TH, int TW, int CC, bool MASK>
 __global__ __launch_bounds__(CONV_THREADS, 2) void conv3x3_fwd_kernel(const ConvArgs a) {
     static_assert(TH * TW == 256, "a block owns 256 pixels");
     static_assert(TW == 8 || TW == 16 || TW == 32, "an MFMA row tile is 32/TW rows of TW pixels");
-    using Stage = FwdStage<TH, TW, CC>;
+    using Stage = FwdStage<TH, TW, CC, MASK>;
     constexpr int HW_ = Stage::HW_;
     constexpr int HALO = Stage::HALO;
     constexpr int CP = Stage::CP;
@@ -132,13 +151,18 @@ __global__ __launch_bounds__(CONV_THREADS, 2) void conv3x3_fwd_kernel(const Conv
     const int wave = tid / 64, lane = tid % 64;
     const int idx = lane % 32, h = lane / 32;
 
-    int b = blockIdx.x;
+    // XCD-aware tile order: workgroup id -> (die, sequence on that die).  Each die walks a
+    // contiguous range of pixel tiles, and the out-channel blocks of one tile follow each
+    // other on the same die, so halo rows/columns and re-read input tiles hit that die's L2.
+    const int xcd = blockIdx.x % N_XCD, seq = blockIdx.x / N_XCD;
+    int b = xcd * a.tiles_per_xcd + seq / a.k_blocks;
+    if (b >= a.n_tiles) return;
+    const int k0 = (seq % a.k_blocks) * BN;
     const int tx = b % a.tiles_x;
     b /= a.tiles_x;
     const int ty = b % a.tiles_y;
     const int n = b / a.tiles_y;
     const int y0 = ty * TH, x0 = tx * TW;
-    const int k0 = blockIdx.y * BN;
 
     float16_t acc[2][2];
 #pragma unroll
@@ -158,16 +182,17 @@ __global__ __launch_bounds__(CONV_THREADS, 2) void conv3x3_fwd_kernel(const Conv
     }
 
     const float* xn = a.x + (size_t)n * a.H * a.W * a.C;
+    const float* mn = MASK ? a.mask + (size_t)n * a.H * a.W * a.C : nullptr;
 
     // Software pipeline over the reduction chunks: the global loads of chunk i+1 are in
     // flight while chunk i is multiplied out of LDS.
     Stage st;
-    st.load(a, xn, y0, x0, k0, 0, tid);
+    st.load(a, xn, mn, y0, x0, k0, 0, tid);
     for (int c0 = 0; c0 < a.C; c0 += CC) {
         __syncthreads();  // everyone is done reading the previous chunk
         st.store(in_tile, w_tile, tid);
         __syncthreads();
-        if (c0 + CC < a.C) st.load(a, xn, y0, x0, k0, c0 + CC, tid);
+        if (c0 + CC < a.C) st.load(a, xn, mn, y0, x0, k0, c0 + CC, tid);
         // ---- 9 taps x CC/8 k-groups x (4 LDS reads + 16 MFMAs) ---------------------------
 #pragma unroll
         for (int tap = 0; tap < 9; ++tap) {
@@ -230,6 +255,7 @@ __global__ __launch_bounds__(256) void filter_rot180_kernel(const float* __restr
 struct WgradArgs {
     const float* x;    // [N,H,W,C]
     const float* dy;   // [N,H,W,K]
+    const float* mask; // [N,H,W,K] or null: dy is taken as 0 where mask <= 0 (fused ReLU backward)
     float* part_w;     // [gridDim.x][K][9][C]   per-block partial sums
     float* part_b;     // [gridDim.x][K]         (null: no bias gradient)
     int N, H, W, C, K;
@@ -308,13 +334,26 @@ __global__ __launch_bounds__(CONV_THREADS, 2) void conv3x3_wgrad_kernel(const Wg
                 const int gy = y0 + p / TW, gx = x0 + p % TW;
                 const int k = k0 + q4;
                 const bool ok = id < PIX * (CS / 4) && gy < a.H && gx < a.W && k < a.K;
-                const float* src = ok ? dyn + ((size_t)gy * a.W + gx) * a.K + k : dyn;
+                const size_t off = ok ? ((size_t)gy * a.W + gx) * a.K + k : 0;
+                const float* src = dyn + off;
                 float4_t v;
                 if (a.k_vec) {
                     v = *(const float4_t*)src;
                 } else {
 #pragma unroll
                     for (int j = 0; j < 4; ++j) v[j] = (ok && k + j < a.K) ? src[j] : 0.f;
+                }
+                if (a.mask) {
+                    const float* msrc = a.mask + (size_t)n * a.H * a.W * a.K + off;
+                    float4_t m;
+                    if (a.k_vec) {
+                        m = *(const float4_t*)msrc;
+                    } else {
+#pragma unroll
+                        for (int j = 0; j < 4; ++j) m[j] = (ok && k + j < a.K) ? msrc[j] : 0.f;
+                    }
+#pragma unroll
+                    for (int j = 0; j < 4; ++j) v[j] = m[j] > 0.f ? v[j] : 0.f;
                 }
                 rdy[it] = ok ? v : zero;
             }
@@ -433,28 +472,34 @@ int check_dims(const char* who, int N, int H, int W, int C, int K) {
 
 }  // namespace
 
-extern "C" int pd_conv3x3_fwd_nhwc_f32(const float* x, const float* w, const float* bias, float* y, int N, int H,
-                                       int W, int C, int K, int relu, void* stream) {
+static int conv3x3_fwd_launch(const float* x, const float* w, const float* bias, const float* mask, float* y, int N,
+                              int H, int W, int C, int K, int relu, void* stream) {
     int rc = check_dims("pd_conv3x3_fwd_nhwc_f32", N, H, W, C, K);
     if (rc != PD_OK) return rc;
     PD_REQUIRE(x && w && y, PD_EINVAL, "pd_conv3x3_fwd_nhwc_f32: NULL pointer");
     ConvArgs a;
-    a.x = x; a.w = w; a.bias = bias; a.y = y;
+    a.x = x; a.w = w; a.bias = bias; a.mask = mask; a.y = y;
     a.N = N; a.H = H; a.W = W; a.C = C; a.K = K;
     a.relu = relu != 0;
-    a.c_vec = (C % 4 == 0) && pd_aligned(x, 16) && pd_aligned(w, 16);
+    a.c_vec = (C % 4 == 0) && pd_aligned(x, 16) && pd_aligned(w, 16) && (!mask || pd_aligned(mask, 16));
     const TileShape t = pick_tile(H, W);
     a.tiles_x = (W + t.tw - 1) / t.tw;
     a.tiles_y = (H + t.th - 1) / t.th;
-    const long nblk = (long)N * a.tiles_x * a.tiles_y;
+    const long ntiles = (long)N * a.tiles_x * a.tiles_y;
+    a.k_blocks = (K + BN - 1) / BN;
+    a.tiles_per_xcd = (int)((ntiles + N_XCD - 1) / N_XCD);
+    const long nblk = (long)N_XCD * a.tiles_per_xcd * a.k_blocks;
     PD_REQUIRE(nblk <= 0x7fffffffL, PD_ESHAPE, "pd_conv3x3_fwd_nhwc_f32: too many tiles");
-    dim3 grid((unsigned)nblk, (K + BN - 1) / BN);
+    a.n_tiles = (int)ntiles;
+    dim3 grid((unsigned)nblk);
     hipStream_t s = (hipStream_t)stream;
     const bool small_c = C <= 8;
 #define PD_LAUNCH_FWD(TH_, TW_)                                                                        \
     do {                                                                                               \
-        if (small_c) conv3x3_fwd_kernel<TH_, TW_, 8><<<grid, CONV_THREADS, 0, s>>>(a);                 \
-        else conv3x3_fwd_kernel<TH_, TW_, 16><<<grid, CONV_THREADS, 0, s>>>(a);                        \
+        if (small_c && mask) conv3x3_fwd_kernel<TH_, TW_, 8, true><<<grid, CONV_THREADS, 0, s>>>(a);   \
+        else if (small_c) conv3x3_fwd_kernel<TH_, TW_, 8, false><<<grid, CONV_THREADS, 0, s>>>(a);     \
+        else if (mask) conv3x3_fwd_kernel<TH_, TW_, 16, true><<<grid, CONV_THREADS, 0, s>>>(a);        \
+        else conv3x3_fwd_kernel<TH_, TW_, 16, false><<<grid, CONV_THREADS, 0, s>>>(a);                 \
     } while (0)
     if (t.tw == 16) PD_LAUNCH_FWD(16, 16);
     else if (t.tw == 32) PD_LAUNCH_FWD(8, 32);
@@ -462,6 +507,18 @@ extern "C" int pd_conv3x3_fwd_nhwc_f32(const float* x, const float* w, const flo
 #undef PD_LAUNCH_FWD
     PD_CHECK_LAUNCH("pd_conv3x3_fwd_nhwc_f32");
     return PD_OK;
+}
+
+extern "C" int pd_conv3x3_fwd_nhwc_f32(const float* x, const float* w, const float* bias, float* y, int N, int H,
+                                       int W, int C, int K, int relu, void* stream) {
+    return conv3x3_fwd_launch(x, w, bias, nullptr, y, N, H, W, C, K, relu, stream);
+}
+
+extern "C" int pd_conv3x3_dgrad_nhwc_f32(const float* dy, const float* w_rot, const float* relu_out, float* dx, int N,
+                                         int H, int W, int K, int C, void* stream) {
+    // the forward kernel with the roles of the channel counts swapped: input = dy (K channels),
+    // filter = rot180(w) [C][3][3][K], output = dx (C channels)
+    return conv3x3_fwd_launch(dy, w_rot, nullptr, relu_out, dx, N, H, W, K, C, 0, stream);
 }
 
 extern "C" int pd_conv3x3_filter_rot180_f32(const float* w, float* out, int K, int C, void* stream) {
@@ -482,8 +539,9 @@ extern "C" int pd_conv3x3_wgrad_workspace_bytes(int N, int H, int W, int C, int 
     return PD_OK;
 }
 
-extern "C" int pd_conv3x3_wgrad_nhwc_f32(const float* x, const float* dy, float* dw, float* dbias, void* workspace,
-                                         uint64_t workspace_bytes, int N, int H, int W, int C, int K, void* stream) {
+extern "C" int pd_conv3x3_wgrad_nhwc_f32(const float* x, const float* dy, const float* relu_out, float* dw,
+                                         float* dbias, void* workspace, uint64_t workspace_bytes, int N, int H, int W,
+                                         int C, int K, void* stream) {
     int rc = check_dims("pd_conv3x3_wgrad_nhwc_f32", N, H, W, C, K);
     if (rc != PD_OK) return rc;
     PD_REQUIRE(x && dy && dw && workspace, PD_EINVAL, "pd_conv3x3_wgrad_nhwc_f32: NULL pointer");
@@ -493,7 +551,7 @@ extern "C" int pd_conv3x3_wgrad_nhwc_f32(const float* x, const float* dy, float*
                (unsigned long long)workspace_bytes, (unsigned long long)need);
     PD_REQUIRE(pd_aligned(workspace, 16), PD_EINVAL, "pd_conv3x3_wgrad_nhwc_f32: workspace must be 16-byte aligned");
     WgradArgs a;
-    a.x = x; a.dy = dy;
+    a.x = x; a.dy = dy; a.mask = relu_out;
     a.N = N; a.H = H; a.W = W; a.C = C; a.K = K;
     a.tiles_x = (W + WGRAD_TW - 1) / WGRAD_TW;
     a.tiles_y = (H + WGRAD_TH - 1) / WGRAD_TH;
@@ -502,7 +560,7 @@ extern "C" int pd_conv3x3_wgrad_nhwc_f32(const float* x, const float* dy, float*
     a.part_w = (float*)workspace;
     a.part_b = dbias ? a.part_w + (size_t)nb * K * 9 * C : nullptr;
     a.c_vec = (C % 4 == 0) && pd_aligned(x, 16);
-    a.k_vec = (K % 4 == 0) && pd_aligned(dy, 16);
+    a.k_vec = (K % 4 == 0) && pd_aligned(dy, 16) && (!relu_out || pd_aligned(relu_out, 16));
     hipStream_t s = (hipStream_t)stream;
     dim3 grid(nb, (K + 63) / 64, (C + 63) / 64);
     conv3x3_wgrad_kernel<WGRAD_TH, WGRAD_TW><<<grid, CONV_THREADS, 0, s>>>(a);

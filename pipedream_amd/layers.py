@@ -92,12 +92,14 @@ class _Conv3x3Fn(torch.autograd.Function):
     @staticmethod
     def backward(ctx, dy):
         x, weight, y = ctx.saved_tensors
-        dy = ops.relu_backward(dy, y) if ctx.relu else ops.to_nhwc(dy)
+        dy = ops.to_nhwc(dy)
+        # the ReLU backward (dy where y > 0) is applied by the gradient kernels while they
+        # load dy, so no masked copy of dy is ever written
         dx = dw = db = None
         if ctx.needs_input_grad[0]:
-            dx = ops.conv3x3_input_grad(dy, weight)
+            dx = ops.conv3x3_input_grad(dy, weight, relu_out=y)
         if ctx.needs_input_grad[1] or (ctx.has_bias and ctx.needs_input_grad[2]):
-            dw, db = ops.conv3x3_weight_grad(x, dy, with_bias=ctx.has_bias)
+            dw, db = ops.conv3x3_weight_grad(x, dy, with_bias=ctx.has_bias, relu_out=y)
         return dx, dw, db, None
 
 

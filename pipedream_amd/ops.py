@@ -248,9 +248,12 @@ def conv3x3_forward(x, w, bias=None, relu=False):
     return y
 
 
-def conv3x3_input_grad(dy, w):
-    """dx of conv3x3_forward: the forward kernel on dy with the 180-degree-rotated filter."""
+def conv3x3_input_grad(dy, w, relu_out=None):
+    """dx of conv3x3_forward: the forward kernel on dy with the 180-degree-rotated filter.
+    ``relu_out`` (the layer's fused-ReLU output) masks dy while it is loaded."""
     _check(dy, "dy")
+    if relu_out is not None and not _dense_same_order(relu_out, dy):
+        raise ValueError("conv3x3_input_grad: relu_out must have dy's shape and memory order")
     n, h, wd, k = _nhwc_dims(dy)
     kw, c = _filter_dims(w)
     if kw != k:
@@ -261,12 +264,16 @@ def conv3x3_input_grad(dy, w):
     lib.pd_conv3x3_filter_rot180_f32(_ptr(w), _ptr(wr), k, c, _cabi.stream_ptr())
     dx = torch.empty((n, c, h, wd), dtype=torch.float32, device=dy.device, memory_format=torch.channels_last)
     with _timed("conv3x3_fwd_kernel" if k > 8 else "conv3x3_fwd_kernel_smallc", 18.0 * c * k * n * h * wd):
-        lib.pd_conv3x3_fwd_nhwc_f32(_ptr(dy), _ptr(wr), None, _ptr(dx), n, h, wd, k, c, 0, _cabi.stream_ptr())
+        lib.pd_conv3x3_dgrad_nhwc_f32(_ptr(dy), _ptr(wr), _ptr(relu_out), _ptr(dx), n, h, wd, k, c,
+                                      _cabi.stream_ptr())
     return dx
 
 
-def conv3x3_weight_grad(x, dy, with_bias=True):
-    """(dw [K,C,3,3] channels_last, dbias [K] or None)."""
+def conv3x3_weight_grad(x, dy, with_bias=True, relu_out=None):
+    """(dw [K,C,3,3] channels_last, dbias [K] or None).  ``relu_out`` masks dy as in
+    conv3x3_input_grad."""
+    if relu_out is not None and not _dense_same_order(relu_out, dy):
+        raise ValueError("conv3x3_weight_grad: relu_out must have dy's shape and memory order")
     _check(x, "x")
     _check(dy, "dy")
     n, h, wd, c = _nhwc_dims(x)
@@ -280,8 +287,8 @@ def conv3x3_weight_grad(x, dy, with_bias=True):
     dw = torch.empty((k, c, 3, 3), dtype=torch.float32, device=x.device, memory_format=torch.channels_last)
     db = torch.empty(k, dtype=torch.float32, device=x.device) if with_bias else None
     with _timed("conv3x3_wgrad", 18.0 * c * k * n * h * wd):
-        lib.pd_conv3x3_wgrad_nhwc_f32(_ptr(x), _ptr(dy), _ptr(dw), _ptr(db), _ptr(ws), nbytes.value, n, h, wd, c, k,
-                                      _cabi.stream_ptr())
+        lib.pd_conv3x3_wgrad_nhwc_f32(_ptr(x), _ptr(dy), _ptr(relu_out), _ptr(dw), _ptr(db), _ptr(ws), nbytes.value,
+                                      n, h, wd, c, k, _cabi.stream_ptr())
     return dw, db
 
 

@@ -98,6 +98,21 @@ def test_fused_relu_and_no_bias():
     assert db is None
 
 
+def test_fused_relu_mask_in_gradient_kernels():
+    g = torch.Generator().manual_seed(8)
+    x = torch.randn(2, 24, 20, 28, generator=g)
+    w = torch.randn(40, 24, 3, 3, generator=g) / 15
+    dy = torch.randn(2, 40, 20, 28, generator=g)
+    y = ops.conv3x3_forward(_nhwc(x), _nhwc(w), None, relu=True)
+    masked = ops.relu_backward(_nhwc(dy), y)
+    dx_ref = ops.conv3x3_input_grad(masked, _nhwc(w))
+    dw_ref, db_ref = ops.conv3x3_weight_grad(_nhwc(x), masked)
+    dx = ops.conv3x3_input_grad(_nhwc(dy), _nhwc(w), relu_out=y)
+    dw, db = ops.conv3x3_weight_grad(_nhwc(x), _nhwc(dy), relu_out=y)
+    # same arithmetic on the same masked values: bit-identical
+    assert torch.equal(dx, dx_ref) and torch.equal(dw, dw_ref) and torch.equal(db, db_ref)
+
+
 def test_identity_filter_is_exact():
     # a centre-tap identity filter must reproduce the input bit for bit
     x = torch.randn(2, 32, 20, 20)
