@@ -414,6 +414,135 @@ __global__ __launch_bounds__(CONV_THREADS, 2) void conv3x3_wgrad_kernel(const Wg
     }
 }
 
+// Weight gradient for very few input channels (9*C <= 32, i.e. the first VGG layer with
+// C = 3): all 9*C (tap, channel) pairs fit the 32 columns of ONE MFMA tile, so a pixel pair
+// costs 2 MFMAs (two 32-row out-channel tiles) instead of 18.  The kernel is then bound by
+// reading dY.  Each of the 4 waves reduces a quarter of the tile's pixels and writes its own
+// partial sums ([gridDim.x * 4] partials).
+template <int TH, int TW>
+__global__ __launch_bounds__(CONV_THREADS, 2) void conv3x3_wgrad_smallc_kernel(const WgradArgs a) {
+    constexpr int PIX = TH * TW;
+    constexpr int HW_ = TW + 2;
+    constexpr int HALO = (TH + 2) * (TW + 2);
+    constexpr int CS = 64;
+    __shared__ __attribute__((aligned(16))) float dy_tile[PIX * CS];
+    __shared__ float x_tile[HALO * 4 + 4];   // [halo pixel][4], last slot stays 0 for unused columns
+
+    const int tid = threadIdx.x;
+    const int wave = tid / 64, lane = tid % 64;
+    const int idx = lane % 32, h = lane / 32;
+    const int k0 = blockIdx.y * 64;
+    const int C = a.C, NC = 9 * a.C;
+    // column idx of the MFMA tile = (tap, c); columns >= 9*C read the zero slot
+    const int tap = idx / C, c = idx % C;
+    const int col_off = idx < NC ? ((tap / 3) * HW_ + (tap % 3)) * 4 + c : -1;
+
+    float16_t acc[2];
+#pragma unroll
+    for (int t = 0; t < 2; ++t)
+#pragma unroll
+        for (int e = 0; e < 16; ++e) acc[t][e] = 0.f;
+    float bsum[2] = {0.f, 0.f};
+    if (tid == 0) x_tile[HALO * 4] = 0.f;
+
+    for (int tile = blockIdx.x; tile < a.n_tiles; tile += gridDim.x) {
+        int b = tile;
+        const int tx = b % a.tiles_x;
+        b /= a.tiles_x;
+        const int ty = b % a.tiles_y;
+        const int n = b / a.tiles_y;
+        const int y0 = ty * TH, x0 = tx * TW;
+        const float* xn = a.x + (size_t)n * a.H * a.W * C;
+        const float* dyn = a.dy + (size_t)n * a.H * a.W * a.K;
+        const float* mn = a.mask ? a.mask + (size_t)n * a.H * a.W * a.K : nullptr;
+
+        constexpr int DY_ITERS = PIX * (CS / 4) / CONV_THREADS;
+        const float4_t zero = {0.f, 0.f, 0.f, 0.f};
+        float4_t rdy[DY_ITERS];
+#pragma unroll
+        for (int it = 0; it < DY_ITERS; ++it) {
+            const int id = tid + it * CONV_THREADS;
+            const int p = id / (CS / 4), q4 = (id % (CS / 4)) * 4;
+            const int gy = y0 + p / TW, gx = x0 + p % TW;
+            const int k = k0 + q4;
+            const bool ok = gy < a.H && gx < a.W && k < a.K;
+            const size_t off = ok ? ((size_t)gy * a.W + gx) * a.K + k : 0;
+            float4_t v;
+            if (a.k_vec) {
+                v = *(const float4_t*)(dyn + off);
+            } else {
+#pragma unroll
+                for (int j = 0; j < 4; ++j) v[j] = (ok && k + j < a.K) ? dyn[off + j] : 0.f;
+            }
+            if (mn) {
+                float4_t m;
+                if (a.k_vec) {
+                    m = *(const float4_t*)(mn + off);
+                } else {
+#pragma unroll
+                    for (int j = 0; j < 4; ++j) m[j] = (ok && k + j < a.K) ? mn[off + j] : 0.f;
+                }
+#pragma unroll
+                for (int j = 0; j < 4; ++j) v[j] = m[j] > 0.f ? v[j] : 0.f;
+            }
+            rdy[it] = ok ? v : zero;
+        }
+        float rx[(HALO * 4 + CONV_THREADS - 1) / CONV_THREADS];
+#pragma unroll
+        for (int it = 0; it < (HALO * 4 + CONV_THREADS - 1) / CONV_THREADS; ++it) {
+            const int id = tid + it * CONV_THREADS;
+            const int p = id / 4, cc = id % 4;
+            const int gy = y0 + p / HW_ - 1, gx = x0 + p % HW_ - 1;
+            const bool ok = id < HALO * 4 && cc < C && gy >= 0 && gy < a.H && gx >= 0 && gx < a.W;
+            rx[it] = ok ? xn[((size_t)gy * a.W + gx) * C + cc] : 0.f;
+        }
+        __syncthreads();  // previous tile fully consumed
+#pragma unroll
+        for (int it = 0; it < DY_ITERS; ++it) {
+            const int id = tid + it * CONV_THREADS;
+            *(float4_t*)(dy_tile + (id / (CS / 4)) * CS + (id % (CS / 4)) * 4) = rdy[it];
+        }
+#pragma unroll
+        for (int it = 0; it < (HALO * 4 + CONV_THREADS - 1) / CONV_THREADS; ++it) {
+            const int id = tid + it * CONV_THREADS;
+            if (id < HALO * 4) x_tile[id] = rx[it];
+        }
+        __syncthreads();
+        // this wave's quarter of the pixels, two per MFMA
+#pragma unroll 4
+        for (int pp = 0; pp < PIX / 8; ++pp) {
+            const int p = wave * (PIX / 4) + 2 * pp + h;
+            const float a0 = dy_tile[p * CS + idx];
+            const float a1 = dy_tile[p * CS + 32 + idx];
+            bsum[0] += a0;
+            bsum[1] += a1;
+            const float bv = x_tile[col_off >= 0 ? ((p / TW) * HW_ + (p % TW)) * 4 + col_off : HALO * 4];
+            acc[0] = __builtin_amdgcn_mfma_f32_32x32x2f32(a0, bv, acc[0], 0, 0, 0);
+            acc[1] = __builtin_amdgcn_mfma_f32_32x32x2f32(a1, bv, acc[1], 0, 0, 0);
+        }
+    }
+
+    const int part = blockIdx.x * 4 + wave;
+    float* pw = a.part_w + (size_t)part * a.K * NC;
+    if (idx < NC) {
+#pragma unroll
+        for (int t = 0; t < 2; ++t)
+#pragma unroll
+            for (int e = 0; e < 16; ++e) {
+                const int k = k0 + t * 32 + 8 * (e / 4) + 4 * h + (e % 4);
+                if (k < a.K) pw[(size_t)k * NC + idx] = acc[t][e];
+            }
+    }
+    if (a.part_b) {
+#pragma unroll
+        for (int t = 0; t < 2; ++t) {
+            const float tot = bsum[t] + __shfl_xor(bsum[t], 32, 64);
+            const int k = k0 + t * 32 + idx;
+            if (h == 0 && k < a.K) a.part_b[(size_t)part * a.K + k] = tot;
+        }
+    }
+}
+
 // out[i] = sum_b part[b][i] in a fixed order (deterministic).  A block owns 64 outputs;
 // its 4 waves each sum a quarter of the partials, then combine through LDS.
 __global__ __launch_bounds__(256) void reduce_partials_kernel(const float* __restrict__ part, float* __restrict__ out,
@@ -534,7 +663,8 @@ extern "C" int pd_conv3x3_wgrad_workspace_bytes(int N, int H, int W, int C, int 
     int rc = check_dims("pd_conv3x3_wgrad_workspace_bytes", N, H, W, C, K);
     if (rc != PD_OK) return rc;
     PD_REQUIRE(bytes != nullptr, PD_EINVAL, "pd_conv3x3_wgrad_workspace_bytes: NULL pointer");
-    const uint64_t nb = (uint64_t)wgrad_blocks(N, H, W);
+    // the few-channel kernel writes one partial per wave (4 per block)
+    const uint64_t nb = (uint64_t)wgrad_blocks(N, H, W) * (9 * C <= 32 ? 4 : 1);
     *bytes = nb * ((uint64_t)K * 9 * C + (uint64_t)K) * sizeof(float);
     return PD_OK;
 }
@@ -556,14 +686,21 @@ extern "C" int pd_conv3x3_wgrad_nhwc_f32(const float* x, const float* dy, const 
     a.tiles_x = (W + WGRAD_TW - 1) / WGRAD_TW;
     a.tiles_y = (H + WGRAD_TH - 1) / WGRAD_TH;
     a.n_tiles = N * a.tiles_x * a.tiles_y;
-    const int nb = wgrad_blocks(N, H, W);
+    const bool small_c = 9 * C <= 32;
+    const int nblk = wgrad_blocks(N, H, W);
+    const int nb = nblk * (small_c ? 4 : 1);     // number of partial sums
     a.part_w = (float*)workspace;
     a.part_b = dbias ? a.part_w + (size_t)nb * K * 9 * C : nullptr;
     a.c_vec = (C % 4 == 0) && pd_aligned(x, 16);
     a.k_vec = (K % 4 == 0) && pd_aligned(dy, 16) && (!relu_out || pd_aligned(relu_out, 16));
     hipStream_t s = (hipStream_t)stream;
-    dim3 grid(nb, (K + 63) / 64, (C + 63) / 64);
-    conv3x3_wgrad_kernel<WGRAD_TH, WGRAD_TW><<<grid, CONV_THREADS, 0, s>>>(a);
+    if (small_c) {
+        dim3 grid(nblk, (K + 63) / 64);
+        conv3x3_wgrad_smallc_kernel<WGRAD_TH, WGRAD_TW><<<grid, CONV_THREADS, 0, s>>>(a);
+    } else {
+        dim3 grid(nblk, (K + 63) / 64, (C + 63) / 64);
+        conv3x3_wgrad_kernel<WGRAD_TH, WGRAD_TW><<<grid, CONV_THREADS, 0, s>>>(a);
+    }
     PD_CHECK_LAUNCH("pd_conv3x3_wgrad_nhwc_f32");
     const int nw = K * 9 * C;
     reduce_partials_kernel<<<dim3((nw + 63) / 64), dim3(256), 0, s>>>(a.part_w, dw, nb, nw);
