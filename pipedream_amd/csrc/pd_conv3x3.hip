@@ -48,8 +48,10 @@ struct ConvArgs {
     int tiles_x, tiles_y;
     int n_tiles, k_blocks, tiles_per_xcd;
     int c_vec;          // C % 4 == 0 and x/w 16-byte aligned: 128-bit global loads
+    int y_vec;          // K % 4 == 0 and y 16-byte aligned: 128-bit stores through the LDS transpose
 };
 
+constexpr int FWD_BLOCKS_PER_XCD = 64;  // 32 CUs per die x 2 resident blocks
 constexpr int N_XCD = 8;  // MI355X: 8 accelerator dies, each with its own L2; workgroups are
                           // handed to them round-robin by linear workgroup id
 
@@ -57,7 +59,7 @@ constexpr int N_XCD = 8;  // MI355X: 8 accelerator dies, each with its own L2; w
 // All loads of a chunk are issued back to back (fixed trip counts, no divergent
 // branches: out-of-range elements read a safe address and are zeroed by a select), so
 // a thread has ~15 128-bit loads in flight instead of one.
-template <int TH, int TW, int CC, bool MASK>
+template <int TH, int TW, int CC, bool MASK, bool VEC>
 struct FwdStage {
     static constexpr int HW_ = TW + 2;
     static constexpr int HALO = (TH + 2) * (TW + 2);
@@ -66,12 +68,19 @@ struct FwdStage {
     static constexpr int IN_ITERS = (HALO * Q + CONV_THREADS - 1) / CONV_THREADS;
     static constexpr int W_ITERS = (9 * BN * Q + CONV_THREADS - 1) / CONV_THREADS;
 
+    // Raw loaded values.  Nothing here is *used* before store(): zero-filling of out-of-range
+    // elements and the ReLU mask are applied when the registers are written to LDS, so the
+    // loads stay in flight across the whole multiply phase that sits between load() and
+    // store() (a use right after the load would force a wait for all of them).
     float4_t rin[IN_ITERS];
+    float4_t rm[MASK ? IN_ITERS : 1];
     float4_t rw[W_ITERS];
+    uint32_t ok_in, ok_w;   // bit it: element it is inside the tensor
 
     __device__ __forceinline__ void load(const ConvArgs& a, const float* __restrict__ xn,
                                          const float* __restrict__ mn, int y0, int x0, int k0, int c0, int tid) {
-        const float4_t zero = {0.f, 0.f, 0.f, 0.f};
+        ok_in = 0;
+        ok_w = 0;
 #pragma unroll
         for (int it = 0; it < IN_ITERS; ++it) {
             const int id = tid + it * CONV_THREADS;
@@ -79,29 +88,19 @@ struct FwdStage {
             const int gy = y0 + p / HW_ - 1, gx = x0 + p % HW_ - 1;
             const int c = c0 + q4;
             const bool ok = id < HALO * Q && gy >= 0 && gy < a.H && gx >= 0 && gx < a.W && c < a.C;
+            ok_in |= (uint32_t)ok << it;
             const size_t off = ok ? ((size_t)gy * a.W + gx) * a.C + c : 0;
-            const float* src = xn + off;
-            float4_t v;
-            if (a.c_vec) {
-                v = *(const float4_t*)src;
+            if (VEC) {
+                rin[it] = *(const float4_t*)(xn + off);
+                if (MASK) rm[it] = *(const float4_t*)(mn + off);
             } else {
 #pragma unroll
-                for (int j = 0; j < 4; ++j) v[j] = (ok && c + j < a.C) ? src[j] : 0.f;
-            }
-            if (MASK) {
-                // gradient of a fused ReLU: dY counts only where the forward output was positive
-                const float* msrc = mn + off;
-                float4_t m;
-                if (a.c_vec) {
-                    m = *(const float4_t*)msrc;
-                } else {
-#pragma unroll
-                    for (int j = 0; j < 4; ++j) m[j] = (ok && c + j < a.C) ? msrc[j] : 0.f;
+                for (int j = 0; j < 4; ++j) {
+                    const bool okj = ok && c + j < a.C;
+                    rin[it][j] = okj ? xn[off + j] : 0.f;
+                    if (MASK) rm[it][j] = okj ? mn[off + j] : 0.f;
                 }
-#pragma unroll
-                for (int j = 0; j < 4; ++j) v[j] = m[j] > 0.f ? v[j] : 0.f;
             }
-            rin[it] = ok ? v : zero;
         }
 #pragma unroll
         for (int it = 0; it < W_ITERS; ++it) {
@@ -110,67 +109,89 @@ struct FwdStage {
             const int tap = row / BN, k = k0 + row % BN;
             const int c = c0 + q4;
             const bool ok = id < 9 * BN * Q && k < a.K && c < a.C;
-            const float* src = ok ? a.w + ((size_t)k * 9 + tap) * a.C + c : a.w;
-            float4_t v;
-            if (a.c_vec) {
-                v = *(const float4_t*)src;
+            ok_w |= (uint32_t)ok << it;
+            const size_t off = ok ? ((size_t)k * 9 + tap) * a.C + c : 0;
+            if (VEC) {
+                rw[it] = *(const float4_t*)(a.w + off);
             } else {
 #pragma unroll
-                for (int j = 0; j < 4; ++j) v[j] = (ok && c + j < a.C) ? src[j] : 0.f;
+                for (int j = 0; j < 4; ++j) rw[it][j] = (ok && c + j < a.C) ? a.w[off + j] : 0.f;
             }
-            rw[it] = ok ? v : zero;
         }
     }
 
     __device__ __forceinline__ void store(float* in_tile, float* w_tile, int tid) const {
+        const float4_t zero = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
         for (int it = 0; it < IN_ITERS; ++it) {
             const int id = tid + it * CONV_THREADS;
-            if (id < HALO * Q) *(float4_t*)(in_tile + (id / Q) * CP + (id % Q) * 4) = rin[it];
+            float4_t v = rin[it];
+            if (MASK) {
+                // gradient of a fused ReLU: dY counts only where the forward output was positive
+#pragma unroll
+                for (int j = 0; j < 4; ++j) v[j] = rm[it][j] > 0.f ? v[j] : 0.f;
+            }
+            v = ((ok_in >> it) & 1u) ? v : zero;
+            if (id < HALO * Q) *(float4_t*)(in_tile + (id / Q) * CP + (id % Q) * 4) = v;
         }
 #pragma unroll
         for (int it = 0; it < W_ITERS; ++it) {
             const int id = tid + it * CONV_THREADS;
-            if (id < 9 * BN * Q) *(float4_t*)(w_tile + (id / Q) * CP + (id % Q) * 4) = rw[it];
+            const float4_t v = ((ok_w >> it) & 1u) ? rw[it] : zero;
+            if (id < 9 * BN * Q) *(float4_t*)(w_tile + (id / Q) * CP + (id % Q) * 4) = v;
         }
     }
 };
 
-template <int TH, int TW, int CC, bool MASK>
+// Decoded work item of the persistent forward kernel: one pixel tile x one block of 64 out
+// channels.
+struct FwdWork {
+    int n, y0, x0, k0;
+    bool valid;
+};
+
+template <int TH, int TW>
+__device__ __forceinline__ FwdWork fwd_work(const ConvArgs& a, int xcd, int w) {
+    // XCD-aware order: each die walks a contiguous range of pixel tiles, the out-channel
+    // blocks of one tile follow each other, and the blocks resident on a die at the same
+    // time work on neighbouring tiles -- halo rows/columns and re-read tiles hit that die's L2.
+    FwdWork r;
+    int b = xcd * a.tiles_per_xcd + w / a.k_blocks;
+    r.valid = w < a.tiles_per_xcd * a.k_blocks && b < a.n_tiles;
+    r.k0 = (w % a.k_blocks) * BN;
+    const int tx = b % a.tiles_x;
+    b /= a.tiles_x;
+    r.x0 = tx * TW;
+    r.y0 = (b % a.tiles_y) * TH;
+    r.n = b / a.tiles_y;
+    return r;
+}
+
+template <int TH, int TW, int CC, bool MASK, bool VEC>
 __global__ __launch_bounds__(CONV_THREADS, 2) void conv3x3_fwd_kernel(const ConvArgs a) {
     static_assert(TH * TW == 256, "a block owns 256 pixels");
     static_assert(TW == 8 || TW == 16 || TW == 32, "an MFMA row tile is 32/TW rows of TW pixels");
-    using Stage = FwdStage<TH, TW, CC, MASK>;
+    using Stage = FwdStage<TH, TW, CC, MASK, VEC>;
     constexpr int HW_ = Stage::HW_;
     constexpr int HALO = Stage::HALO;
     constexpr int CP = Stage::CP;
-    __shared__ __attribute__((aligned(16))) float in_tile[HALO * CP];
-    __shared__ __attribute__((aligned(16))) float w_tile[9 * BN * CP];
+    constexpr int STEPS = 9 * (CC / 8);   // (tap, k-group) pairs per chunk
+    constexpr int OP = BN + 4;            // pitch of the output staging tile
+    constexpr int LDS_FLOATS = (HALO * CP + 9 * BN * CP) > 256 * OP ? (HALO * CP + 9 * BN * CP) : 256 * OP;
+    __shared__ __attribute__((aligned(16))) float lds[LDS_FLOATS];
+    float* const in_tile = lds;
+    float* const w_tile = lds + HALO * CP;
 
     const int tid = threadIdx.x;
     const int wave = tid / 64, lane = tid % 64;
     const int idx = lane % 32, h = lane / 32;
 
-    // XCD-aware tile order: workgroup id -> (die, sequence on that die).  Each die walks a
-    // contiguous range of pixel tiles, and the out-channel blocks of one tile follow each
-    // other on the same die, so halo rows/columns and re-read input tiles hit that die's L2.
-    const int xcd = blockIdx.x % N_XCD, seq = blockIdx.x / N_XCD;
-    int b = xcd * a.tiles_per_xcd + seq / a.k_blocks;
-    if (b >= a.n_tiles) return;
-    const int k0 = (seq % a.k_blocks) * BN;
-    const int tx = b % a.tiles_x;
-    b /= a.tiles_x;
-    const int ty = b % a.tiles_y;
-    const int n = b / a.tiles_y;
-    const int y0 = ty * TH, x0 = tx * TW;
-
-    float16_t acc[2][2];
-#pragma unroll
-    for (int i = 0; i < 2; ++i)
-#pragma unroll
-        for (int j = 0; j < 2; ++j)
-#pragma unroll
-            for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.f;
+    // Persistent blocks: gridDim.x / N_XCD blocks per die, each striding over that die's work.
+    const int xcd = blockIdx.x % N_XCD;
+    const int per_xcd = gridDim.x / N_XCD;
+    int w = blockIdx.x / N_XCD;
+    FwdWork cur = fwd_work<TH, TW>(a, xcd, w);
+    if (!cur.valid) return;
 
     // LDS offsets of this lane's two pixel rows (tap 0,0) and two filter rows.
     int a_off[2], b_off[2];
@@ -180,30 +201,50 @@ __global__ __launch_bounds__(CONV_THREADS, 2) void conv3x3_fwd_kernel(const Conv
         a_off[i] = ((q / TW) * HW_ + (q % TW)) * CP + 4 * h;
         b_off[i] = (i * 32 + idx) * CP + 4 * h;
     }
+    auto read_frags = [&](int step, float4_t (&fa)[2], float4_t (&fb)[2]) {
+        const int tap = step / (CC / 8), g = step % (CC / 8);
+        const int shift = ((tap / 3) * HW_ + (tap % 3)) * CP;
+#pragma unroll
+        for (int i = 0; i < 2; ++i) fa[i] = *(const float4_t*)(in_tile + a_off[i] + shift + 8 * g);
+#pragma unroll
+        for (int j = 0; j < 2; ++j) fb[j] = *(const float4_t*)(w_tile + tap * BN * CP + b_off[j] + 8 * g);
+    };
 
-    const float* xn = a.x + (size_t)n * a.H * a.W * a.C;
-    const float* mn = MASK ? a.mask + (size_t)n * a.H * a.W * a.C : nullptr;
-
-    // Software pipeline over the reduction chunks: the global loads of chunk i+1 are in
-    // flight while chunk i is multiplied out of LDS.
+    const size_t img = (size_t)a.H * a.W * a.C;
+    // Software pipeline over (work item, reduction chunk): the global loads of the next chunk
+    // -- or of the next tile's first chunk -- are in flight while the current chunk is
+    // multiplied out of LDS, and the epilogue stores overlap the next tile's loads.
     Stage st;
-    st.load(a, xn, mn, y0, x0, k0, 0, tid);
-    for (int c0 = 0; c0 < a.C; c0 += CC) {
-        __syncthreads();  // everyone is done reading the previous chunk
-        st.store(in_tile, w_tile, tid);
-        __syncthreads();
-        if (c0 + CC < a.C) st.load(a, xn, mn, y0, x0, k0, c0 + CC, tid);
-        // ---- 9 taps x CC/8 k-groups x (4 LDS reads + 16 MFMAs) ---------------------------
+    st.load(a, a.x + cur.n * img, MASK ? a.mask + cur.n * img : nullptr, cur.y0, cur.x0, cur.k0, 0, tid);
+    while (true) {
+        float16_t acc[2][2];
 #pragma unroll
-        for (int tap = 0; tap < 9; ++tap) {
-            const int shift = ((tap / 3) * HW_ + (tap % 3)) * CP;
+        for (int i = 0; i < 2; ++i)
 #pragma unroll
-            for (int g = 0; g < CC / 8; ++g) {
+            for (int j = 0; j < 2; ++j)
+#pragma unroll
+                for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.f;
+        FwdWork nxt;
+        nxt.valid = false;
+        for (int c0 = 0; c0 < a.C; c0 += CC) {
+            __syncthreads();  // everyone is done reading the previous chunk
+            st.store(in_tile, w_tile, tid);
+            __syncthreads();
+            if (c0 + CC < a.C) {
+                st.load(a, a.x + cur.n * img, MASK ? a.mask + cur.n * img : nullptr, cur.y0, cur.x0, cur.k0,
+                        c0 + CC, tid);
+            } else {
+                w += per_xcd;
+                nxt = fwd_work<TH, TW>(a, xcd, w);
+                if (nxt.valid)
+                    st.load(a, a.x + nxt.n * img, MASK ? a.mask + nxt.n * img : nullptr, nxt.y0, nxt.x0, nxt.k0, 0,
+                            tid);
+            }
+            // ---- STEPS x (4 LDS reads + 16 MFMAs) ----------------------------------------------
+#pragma unroll
+            for (int step = 0; step < STEPS; ++step) {
                 float4_t fa[2], fb[2];
-#pragma unroll
-                for (int i = 0; i < 2; ++i) fa[i] = *(const float4_t*)(in_tile + a_off[i] + shift + 8 * g);
-#pragma unroll
-                for (int j = 0; j < 2; ++j) fb[j] = *(const float4_t*)(w_tile + tap * BN * CP + b_off[j] + 8 * g);
+                read_frags(step, fa, fb);
 #pragma unroll
                 for (int s = 0; s < 4; ++s)
 #pragma unroll
@@ -213,27 +254,58 @@ __global__ __launch_bounds__(CONV_THREADS, 2) void conv3x3_fwd_kernel(const Conv
                             acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(fa[i][s], fb[j][s], acc[i][j], 0, 0, 0);
             }
         }
-    }
 
-    // ---- epilogue: bias, ReLU, NHWC store (32 consecutive channels per lane group) ------
-    float* yn = a.y + (size_t)n * a.H * a.W * a.K;
+        // ---- epilogue: bias + ReLU, then the 256 x 64 result tile is transposed through LDS
+        //      (reusing the operand tiles) so that every lane writes 16 contiguous bytes and a
+        //      wave covers whole 256-byte pixel rows of the NHWC output -------------------------
+        float* yn = a.y + (size_t)cur.n * a.H * a.W * a.K;
+        if (a.y_vec) {
+            __syncthreads();  // all waves are done reading the operand tiles
 #pragma unroll
-    for (int j = 0; j < 2; ++j) {
-        const int k = k0 + j * 32 + idx;
-        if (k >= a.K) continue;
-        const float bv = a.bias ? a.bias[k] : 0.f;
+            for (int j = 0; j < 2; ++j) {
+                const int k = cur.k0 + j * 32 + idx;
+                const float bv = (a.bias && k < a.K) ? a.bias[k] : 0.f;
 #pragma unroll
-        for (int i = 0; i < 2; ++i)
+                for (int i = 0; i < 2; ++i)
 #pragma unroll
-            for (int e = 0; e < 16; ++e) {
-                const int q = (wave * 2 + i) * 32 + 8 * (e / 4) + 4 * h + (e % 4);
-                const int gy = y0 + q / TW, gx = x0 + q % TW;
-                if (gy < a.H && gx < a.W) {
-                    float v = acc[i][j][e] + bv;
-                    if (a.relu) v = v > 0.f ? v : 0.f;
-                    yn[((size_t)gy * a.W + gx) * a.K + k] = v;
-                }
+                    for (int e = 0; e < 16; ++e) {
+                        const int q = (wave * 2 + i) * 32 + 8 * (e / 4) + 4 * h + (e % 4);
+                        float v = acc[i][j][e] + bv;
+                        if (a.relu) v = v > 0.f ? v : 0.f;
+                        lds[q * OP + j * 32 + idx] = v;
+                    }
             }
+            __syncthreads();
+#pragma unroll
+            for (int it = 0; it < 256 * (BN / 4) / CONV_THREADS; ++it) {
+                const int id = tid + it * CONV_THREADS;
+                const int q = id / (BN / 4), k4 = (id % (BN / 4)) * 4;
+                const int gy = cur.y0 + q / TW, gx = cur.x0 + q % TW;
+                if (gy < a.H && gx < a.W && cur.k0 + k4 < a.K)
+                    *(float4_t*)(yn + ((size_t)gy * a.W + gx) * a.K + cur.k0 + k4) = *(const float4_t*)(lds + q * OP + k4);
+            }
+        } else {
+#pragma unroll
+            for (int j = 0; j < 2; ++j) {
+                const int k = cur.k0 + j * 32 + idx;
+                if (k >= a.K) continue;
+                const float bv = a.bias ? a.bias[k] : 0.f;
+#pragma unroll
+                for (int i = 0; i < 2; ++i)
+#pragma unroll
+                    for (int e = 0; e < 16; ++e) {
+                        const int q = (wave * 2 + i) * 32 + 8 * (e / 4) + 4 * h + (e % 4);
+                        const int gy = cur.y0 + q / TW, gx = cur.x0 + q % TW;
+                        if (gy < a.H && gx < a.W) {
+                            float v = acc[i][j][e] + bv;
+                            if (a.relu) v = v > 0.f ? v : 0.f;
+                            yn[((size_t)gy * a.W + gx) * a.K + k] = v;
+                        }
+                    }
+            }
+        }
+        if (!nxt.valid) break;
+        cur = nxt;
     }
 }
 
@@ -717,6 +789,7 @@ static int conv3x3_fwd_launch(const float* x, const float* w, const float* bias,
     a.N = N; a.H = H; a.W = W; a.C = C; a.K = K;
     a.relu = relu != 0;
     a.c_vec = (C % 4 == 0) && pd_aligned(x, 16) && pd_aligned(w, 16) && (!mask || pd_aligned(mask, 16));
+    a.y_vec = (K % 4 == 0) && pd_aligned(y, 16);
     const TileShape t = pick_tile(H, W);
     a.tiles_x = (W + t.tw - 1) / t.tw;
     a.tiles_y = (H + t.th - 1) / t.th;
@@ -726,16 +799,21 @@ static int conv3x3_fwd_launch(const float* x, const float* w, const float* bias,
     const long nblk = (long)N_XCD * a.tiles_per_xcd * a.k_blocks;
     PD_REQUIRE(nblk <= 0x7fffffffL, PD_ESHAPE, "pd_conv3x3_fwd_nhwc_f32: too many tiles");
     a.n_tiles = (int)ntiles;
-    dim3 grid((unsigned)nblk);
+    dim3 grid((unsigned)nblk);                       // one block per work item (few-channel kernel)
+    const long per_xcd_work = (long)a.tiles_per_xcd * a.k_blocks;
+    const int per_xcd_blocks = (int)(per_xcd_work < FWD_BLOCKS_PER_XCD ? per_xcd_work : FWD_BLOCKS_PER_XCD);
+    dim3 pgrid((unsigned)(N_XCD * per_xcd_blocks));  // persistent blocks
     hipStream_t s = (hipStream_t)stream;
     const bool small_c = C <= 8;
 #define PD_LAUNCH_FWD(TH_, TW_)                                                                        \
     do {                                                                                               \
         if (9 * C <= 32 && !mask) conv3x3_fwd_smallc_kernel<TH_, TW_><<<grid, CONV_THREADS, 0, s>>>(a); \
-        else if (small_c && mask) conv3x3_fwd_kernel<TH_, TW_, 8, true><<<grid, CONV_THREADS, 0, s>>>(a);   \
-        else if (small_c) conv3x3_fwd_kernel<TH_, TW_, 8, false><<<grid, CONV_THREADS, 0, s>>>(a);     \
-        else if (mask) conv3x3_fwd_kernel<TH_, TW_, 16, true><<<grid, CONV_THREADS, 0, s>>>(a);        \
-        else conv3x3_fwd_kernel<TH_, TW_, 16, false><<<grid, CONV_THREADS, 0, s>>>(a);                 \
+        else if (!a.c_vec && mask) conv3x3_fwd_kernel<TH_, TW_, 8, true, false><<<pgrid, CONV_THREADS, 0, s>>>(a); \
+        else if (!a.c_vec) conv3x3_fwd_kernel<TH_, TW_, 8, false, false><<<pgrid, CONV_THREADS, 0, s>>>(a);  \
+        else if (small_c && mask) conv3x3_fwd_kernel<TH_, TW_, 8, true, true><<<pgrid, CONV_THREADS, 0, s>>>(a); \
+        else if (small_c) conv3x3_fwd_kernel<TH_, TW_, 8, false, true><<<pgrid, CONV_THREADS, 0, s>>>(a); \
+        else if (mask) conv3x3_fwd_kernel<TH_, TW_, 16, true, true><<<pgrid, CONV_THREADS, 0, s>>>(a);  \
+        else conv3x3_fwd_kernel<TH_, TW_, 16, false, true><<<pgrid, CONV_THREADS, 0, s>>>(a);           \
     } while (0)
     if (t.tw == 16) PD_LAUNCH_FWD(16, 16);
     else if (t.tw == 32) PD_LAUNCH_FWD(8, 32);
