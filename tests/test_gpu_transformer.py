@@ -55,6 +55,54 @@ def test_gemm_bf16_epilogues():
         ops.gemm_bf16(a.cuda()[:, :60], b.cuda()[:, :60], trans_b=True)     # K not a multiple of 8
 
 
+@pytest.mark.parametrize("ta,tb", [(False, True), (False, False), (True, False), (True, True)])
+@pytest.mark.parametrize("M,N,K", [(4096, 3072, 128), (3992, 3600, 256), (4000, 3592, 224), (3584, 3584, 96)])
+def test_gemm_bf16_large_tiles(M, N, K, ta, tb):
+    """Shapes with >= 192 tiles of 256 x 256: K a multiple of 128 runs the direct-to-LDS ring
+    kernel (one and two ring rounds), other K the register-staged large-tile kernel; M and N
+    that are not tile multiples exercise the clamped loads and the masked vector stores.
+    The fp32 reference product is computed on the device by torch from the same bf16 inputs."""
+    from pipedream_amd import ops
+    g = torch.Generator().manual_seed(M + N + K)
+    a = torch.randn((K, M) if ta else (M, K), generator=g).to(BF).cuda()
+    b = torch.randn((N, K) if tb else (K, N), generator=g).to(BF).cuda()
+    want = (a.float().t() if ta else a.float()) @ (b.float().t() if tb else b.float())
+    got32 = ops.gemm_bf16(a, b, trans_a=ta, trans_b=tb, out_f32=True)
+    assert _rel(got32, want.cpu()) < 1e-5
+    torch.testing.assert_close(got32, want, rtol=1e-4, atol=2e-6 * math.sqrt(K) * 9)
+    got16 = ops.gemm_bf16(a, b, trans_a=ta, trans_b=tb)
+    assert torch.equal(got16, got32.to(BF))
+
+
+def test_gemm_bf16_large_tile_epilogues():
+    """bias + residual (single rounding), alpha, and fp32 accumulation (beta = 1) through the
+    vectorised LDS-transposed epilogue, and the element-wise fallback when C is not 16-byte
+    aligned."""
+    from pipedream_amd import ops
+    g = torch.Generator().manual_seed(1)
+    M, N, K = 4096, 4096, 128
+    a = torch.randn(M, K, generator=g).to(BF).cuda()
+    b = torch.randn(N, K, generator=g).to(BF).cuda()
+    bias = torch.randn(N, generator=g).cuda()
+    res = torch.randn(M, N, generator=g).to(BF).cuda()
+    prod = a.float() @ b.float().t()
+    got = ops.gemm_bf16(a, b, trans_b=True, alpha=0.5, bias=bias, residual=res)
+    want = (0.5 * prod + bias + res.float()).to(BF)
+    # fp32 summation order inside the product differs from torch's, so a value within rounding of a
+    # bf16 tie may round the other way: at most one bf16 ulp, and rarely
+    diff = (got.float() - want.float()).abs()
+    assert float(diff.max()) <= float(want.float().abs().max()) * 2 ** -7
+    assert float((diff > 0).float().mean()) < 1e-3
+    acc = torch.ones(M, N).cuda()
+    ops.gemm_bf16(a, b, trans_b=True, out=acc, beta=1.0)
+    assert _rel(acc, (prod + 1).cpu()) < 1e-5
+    # C shifted by one element: 16-byte vector stores are impossible, the element-wise path must agree
+    buf = torch.zeros(M * N + 8, dtype=BF).cuda()
+    shifted = buf[1:1 + M * N].view(M, N)
+    ops.gemm_bf16(a, b, trans_b=True, out=shifted)
+    assert torch.equal(shifted, ops.gemm_bf16(a, b, trans_b=True))
+
+
 def test_layernorm_softmax_gelu_vs_torch():
     from pipedream_amd import ops
     g = torch.Generator().manual_seed(1)
