@@ -541,7 +541,7 @@ struct DmaGemm {
 };
 
 template <int BM, int BN, bool A_KC, bool B_KC>
-__global__ __launch_bounds__(256) void pd_gemm_bf16_dma_kernel(const GemmBf16Args a) {
+__global__ __launch_bounds__(256, (BM * BN <= 128 * 128 ? 2 : 1)) void pd_gemm_bf16_dma_kernel(const GemmBf16Args a) {
     using G = DmaGemm<BM, BN, A_KC, B_KC>;
     using TA = typename G::TA;
     using TB = typename G::TB;
@@ -699,7 +699,8 @@ extern "C" int pd_gemm_bf16(int trans_a, int trans_b, int M, int N, int K, const
     const long tiles128 = (long)((M + 127) / 128) * ((N + 127) / 128) * batch;
     // direct-to-LDS kernel: whole ring rounds of k, and per-lane byte offsets that fit 32 bits
     const bool dma_ok = K % (DK * NS) == 0 && (long long)256 * (lda > ldb ? lda : ldb) * 2 < (1ll << 31);
-    if (tiles256 >= 192 && dma_ok) return launch_gemm_bf16_dma<256, 256>(trans_a, trans_b, g, batch, s);
+    if (dma_ok && tiles256 >= 256) return launch_gemm_bf16_dma<256, 256>(trans_a, trans_b, g, batch, s);
+    if (dma_ok && M >= 128 && N >= 128) return launch_gemm_bf16_dma<128, 128>(trans_a, trans_b, g, batch, s);
     if (tiles256 >= 192) return launch_gemm_bf16<256, 256, 2, 4>(trans_a, trans_b, g, batch, s);
     if (tiles128 >= 128) return launch_gemm_bf16<128, 128, 2, 2>(trans_a, trans_b, g, batch, s);
     return launch_gemm_bf16<64, 64, 2, 2>(trans_a, trans_b, g, batch, s);

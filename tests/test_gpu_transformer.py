@@ -56,11 +56,13 @@ def test_gemm_bf16_epilogues():
 
 
 @pytest.mark.parametrize("ta,tb", [(False, True), (False, False), (True, False), (True, True)])
-@pytest.mark.parametrize("M,N,K", [(4096, 3072, 128), (3992, 3600, 256), (4000, 3592, 224), (3584, 3584, 96)])
+@pytest.mark.parametrize("M,N,K", [(4096, 4096, 128), (4088, 4104, 256), (4096, 3072, 128), (3992, 3600, 256),
+                                   (1000, 1016, 384), (4000, 3592, 224), (3584, 3584, 96)])
 def test_gemm_bf16_large_tiles(M, N, K, ta, tb):
-    """Shapes with >= 192 tiles of 256 x 256: K a multiple of 128 runs the direct-to-LDS ring
-    kernel (one and two ring rounds), other K the register-staged large-tile kernel; M and N
-    that are not tile multiples exercise the clamped loads and the masked vector stores.
+    """K a multiple of 128 runs the direct-to-LDS ring kernel (one to three ring rounds): with
+    256 x 256 tiles when there are at least 256 of them, else with 128 x 128 tiles; other K
+    the register-staged large-tile kernel; M and N that are not tile multiples exercise the
+    clamped loads and the masked vector stores.
     The fp32 reference product is computed on the device by torch from the same bf16 inputs."""
     from pipedream_amd import ops
     g = torch.Generator().manual_seed(M + N + K)
