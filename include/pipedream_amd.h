@@ -135,6 +135,16 @@ int pd_adam_step(const pd_tensor_desc* descs, int n_tensors,
 int pd_gemm_f32(int trans_a, int trans_b, int M, int N, int K,
                 const float* A, int lda, const float* B, int ldb,
                 float beta, float* C, int ldc, const float* bias, int relu, void* stream);
+/* The same product split over k for problems with too few output tiles to fill the GPU (the
+ * recurrent LSTM products with M = batch, the VGG classifier layers with M = 64):
+ * partials[s][M][N] (dense) = op(A)[:, k in split s] op(B)[k in split s, :].  The caller sums the
+ * partials in index order (deterministic): pd_splitk_reduce_f32, or the LSTM cell kernels. */
+int pd_gemm_splitk_f32(int trans_a, int trans_b, int M, int N, int K,
+                       const float* A, int lda, const float* B, int ldb,
+                       float* partials, int splits, void* stream);
+/* C[M][ldc] = sum_s partials[s] (+ bias[N]) (+ beta*C) (ReLU); N and ldc multiples of 4. */
+int pd_splitk_reduce_f32(const float* partials, int splits, int M, int N, const float* bias, int relu,
+                         float beta, float* C, int ldc, void* stream);
 
 /* out[s][n] = sum over the s-th of `splits` row ranges of x[m][n]  (bias gradients).
  * With splits == 1 and beta != 0 the sum is added to beta*out. */
@@ -192,17 +202,19 @@ int pd_conv3x3_wgrad_nhwc_f32(const float* x, const float* dy, const float* relu
                               int N, int H, int W, int C, int K, void* stream);
 
 /* torch.nn.LSTM cell (gnmt_large/gpus=4/stage0.py:14-19), gate order i,f,g,o.
- * Forward, one time step: gates[B][4H] holds x W_ih^T + h_prev W_hh^T on entry (from
- * pd_gemm_f32) and the activated gates on exit; biases and c_prev may be NULL (= 0).
- * c = f*c_prev + i*g, h = o*tanh(c). */
-int pd_lstm_cell_fwd_f32(float* gates, const float* b_ih, const float* b_hh, const float* c_prev,
-                         float* c_out, float* h_out, int B, int H, void* stream);
-/* Backward of that step: dh = dy (+ dh_rec if not NULL); dc_io holds dL/dc_t from the next
- * step on entry (ignored when first_step != 0, i.e. for the last time step) and dL/dc_prev
- * on exit; dgates[B][4H] = gradients of the gate pre-activations. */
+ * Forward, one time step: gates[B][4H] holds x W_ih^T on entry, to which the n_rec split-k
+ * partial products rec[n_rec][B][4H] of h_prev W_hh^T (pd_gemm_splitk_f32; n_rec may be 0)
+ * and the biases are added; on exit it holds the activated gates.  Biases and c_prev may be
+ * NULL (= 0).  c = f*c_prev + i*g, h = o*tanh(c). */
+int pd_lstm_cell_fwd_f32(float* gates, const float* rec, int n_rec, const float* b_ih, const float* b_hh,
+                         const float* c_prev, float* c_out, float* h_out, int B, int H, void* stream);
+/* Backward of that step: dh = dy + sum of the n_rec partials dh_rec[n_rec][B][H] (dh_rec may be
+ * NULL); dc_io holds dL/dc_t from the next step on entry (ignored when first_step != 0, i.e.
+ * for the last time step) and dL/dc_prev on exit; dgates[B][4H] = gradients of the gate
+ * pre-activations. */
 int pd_lstm_cell_bwd_f32(const float* gates, const float* c_prev, const float* c, const float* dy,
-                         const float* dh_rec, float* dc_io, float* dgates, int B, int H, int first_step,
-                         void* stream);
+                         const float* dh_rec, int n_rec, float* dc_io, float* dgates, int B, int H,
+                         int first_step, void* stream);
 /* y = a + b: the residual connections `out13 = out13 + out10` (stage0.py:32, 36). */
 int pd_add_f32(const float* a, const float* b, float* y, uint64_t n, void* stream);
 /* torch.nn.Embedding (stage0.py:10): out[p][:] = weight[ids[p]][:].  Backward writes the

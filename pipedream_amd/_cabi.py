@@ -63,6 +63,8 @@ SIGNATURES = {
     "pd_sgd_step": (_i, [ctypes.POINTER(TensorDesc), _i, _d, _d, _d, _d, _i, _i, _d, _d, _vp], True),
     "pd_adam_step": (_i, [ctypes.POINTER(TensorDesc), _i, _d, _d, _d, _d, _d, _i64, _i, _d, _d, _vp], True),
     "pd_gemm_f32": (_i, [_i, _i, _i, _i, _i, _vp, _i, _vp, _i, _f, _vp, _i, _vp, _i, _vp], True),
+    "pd_gemm_splitk_f32": (_i, [_i, _i, _i, _i, _i, _vp, _i, _vp, _i, _vp, _i, _vp], True),
+    "pd_splitk_reduce_f32": (_i, [_vp, _i, _i, _i, _vp, _i, _f, _vp, _i, _vp], True),
     "pd_colsum_f32": (_i, [_vp, _vp, _u64, _i, _u64, _i, _f, _vp], True),
     "pd_relu_fwd_f32": (_i, [_vp, _vp, _u64, _vp], True),
     "pd_relu_bwd_f32": (_i, [_vp, _vp, _vp, _u64, _vp], True),
@@ -75,8 +77,8 @@ SIGNATURES = {
     "pd_conv3x3_wgrad_workspace_bytes": (_i, [_i, _i, _i, _i, _i, ctypes.POINTER(ctypes.c_uint64)], True),
     "pd_conv3x3_dgrad_nhwc_f32": (_i, [_vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _vp], True),
     "pd_conv3x3_wgrad_nhwc_f32": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _u64, _i, _i, _i, _i, _i, _vp], True),
-    "pd_lstm_cell_fwd_f32": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _vp], True),
-    "pd_lstm_cell_bwd_f32": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _vp], True),
+    "pd_lstm_cell_fwd_f32": (_i, [_vp, _vp, _i, _vp, _vp, _vp, _vp, _vp, _i, _i, _vp], True),
+    "pd_lstm_cell_bwd_f32": (_i, [_vp, _vp, _vp, _vp, _vp, _i, _vp, _vp, _i, _i, _i, _vp], True),
     "pd_add_f32": (_i, [_vp, _vp, _vp, _u64, _vp], True),
     "pd_embedding_fwd_f32": (_i, [_vp, _vp, _vp, _i, _i, _i64, _vp], True),
     "pd_embedding_bwd_f32": (_i, [_vp, _vp, _vp, _i, _i, _i64, _i64, _vp], True),

@@ -36,6 +36,8 @@ struct GemmArgs {
     float beta;         // C = acc + beta*C_old (0 -> overwrite, C_old not read)
     int relu;
     int a_vec, b_vec;   // 128-bit global loads allowed for A / B
+    int k_per_split;    // blockIdx.z owns k in [z*k_per_split, (z+1)*k_per_split) and writes C + z*c_split
+    long long c_split;  // elements between the partial results of consecutive splits
 };
 
 // Operand tile in LDS.  KC (k-contiguous): [ROWS][BK+4]; otherwise [BK][ROWS+4].
@@ -144,9 +146,12 @@ __global__ __launch_bounds__(GEMM_THREADS) void pd_gemm_f32_kernel(const GemmArg
             for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.f;
 
     float4_t ra[TA::VEC_PER_THREAD], rb[TB::VEC_PER_THREAD];
-    const int nk = (a.K + BK - 1) / BK;
-    TA::load(ra, a.A, a.lda, m0, 0, a.M, a.K, a.a_vec, tid);
-    TB::load(rb, a.B, a.ldb, n0, 0, a.N, a.K, a.b_vec, tid);
+    const int k_begin = blockIdx.z * a.k_per_split;
+    const int k_end = min(a.K, k_begin + a.k_per_split);
+    const int nk = (k_end - k_begin + BK - 1) / BK;
+    float* const C = a.C + blockIdx.z * a.c_split;
+    TA::load(ra, a.A, a.lda, m0, k_begin, a.M, k_end, a.a_vec, tid);
+    TB::load(rb, a.B, a.ldb, n0, k_begin, a.N, k_end, a.b_vec, tid);
     TA::store(lds_a[0], ra, tid);
     TB::store(lds_b[0], rb, tid);
     __syncthreads();
@@ -154,8 +159,8 @@ __global__ __launch_bounds__(GEMM_THREADS) void pd_gemm_f32_kernel(const GemmArg
     for (int kt = 0; kt < nk; ++kt) {
         const int cur = kt & 1;
         if (kt + 1 < nk) {  // prefetch the next chunk into registers while this one is multiplied
-            TA::load(ra, a.A, a.lda, m0, (kt + 1) * BK, a.M, a.K, a.a_vec, tid);
-            TB::load(rb, a.B, a.ldb, n0, (kt + 1) * BK, a.N, a.K, a.b_vec, tid);
+            TA::load(ra, a.A, a.lda, m0, k_begin + (kt + 1) * BK, a.M, k_end, a.a_vec, tid);
+            TB::load(rb, a.B, a.ldb, n0, k_begin + (kt + 1) * BK, a.N, k_end, a.b_vec, tid);
         }
 #pragma unroll
         for (int g = 0; g < BK / 8; ++g) {
@@ -191,7 +196,7 @@ __global__ __launch_bounds__(GEMM_THREADS) void pd_gemm_f32_kernel(const GemmArg
             for (int e = 0; e < 16; ++e) {
                 const int row = m0 + wm * (BM / 2) + i * 32 + 8 * (e / 4) + 4 * h + (e % 4);
                 if (row >= a.M) continue;
-                float* p = a.C + (size_t)row * a.ldc + col;
+                float* p = C + (size_t)row * a.ldc + col;
                 float v = acc[i][j][e] + bv;
                 if (a.beta != 0.f) v += a.beta * *p;
                 if (a.relu) v = v > 0.f ? v : 0.f;
@@ -201,8 +206,8 @@ __global__ __launch_bounds__(GEMM_THREADS) void pd_gemm_f32_kernel(const GemmArg
 }
 
 template <int BM, int BN>
-int launch_gemm(int trans_a, int trans_b, const GemmArgs& g, hipStream_t s) {
-    dim3 grid((g.N + BN - 1) / BN, (g.M + BM - 1) / BM);
+int launch_gemm(int trans_a, int trans_b, const GemmArgs& g, hipStream_t s, int splits = 1) {
+    dim3 grid((g.N + BN - 1) / BN, (g.M + BM - 1) / BM, splits);
     // A is k-contiguous when it is NOT transposed; B (stored [K][N]) is k-contiguous when it IS.
     if (!trans_a && trans_b) pd_gemm_f32_kernel<BM, BN, true, true><<<grid, GEMM_THREADS, 0, s>>>(g);
     else if (!trans_a && !trans_b) pd_gemm_f32_kernel<BM, BN, true, false><<<grid, GEMM_THREADS, 0, s>>>(g);
@@ -210,6 +215,26 @@ int launch_gemm(int trans_a, int trans_b, const GemmArgs& g, hipStream_t s) {
     else pd_gemm_f32_kernel<BM, BN, false, true><<<grid, GEMM_THREADS, 0, s>>>(g);
     PD_CHECK_LAUNCH("pd_gemm_f32");
     return PD_OK;
+}
+
+// out = (sum over splits of partials) (+ bias) (+ beta*out) (relu): 4 elements per thread
+__global__ __launch_bounds__(256) void splitk_reduce_kernel(const float* __restrict__ partials, int splits, int M, int N,
+                                                           const float* __restrict__ bias, int relu, float beta,
+                                                           float* __restrict__ C, int ldc) {
+    const int n4 = N / 4;
+    const long long id = (long long)blockIdx.x * 256 + threadIdx.x;
+    if (id >= (long long)M * n4) return;
+    const int row = (int)(id / n4), col = (int)(id % n4) * 4;
+    const size_t per = (size_t)M * N;
+    float4_t v = *(const float4_t*)(partials + (size_t)row * N + col);
+    for (int s = 1; s < splits; ++s) v += *(const float4_t*)(partials + s * per + (size_t)row * N + col);
+    if (bias) v += *(const float4_t*)(bias + col);
+    float* p = C + (size_t)row * ldc + col;
+    if (beta != 0.f) v += beta * *(const float4_t*)p;
+    if (relu)
+#pragma unroll
+        for (int j = 0; j < 4; ++j) v[j] = v[j] > 0.f ? v[j] : 0.f;
+    *(float4_t*)p = v;
 }
 
 }  // namespace
@@ -229,9 +254,46 @@ extern "C" int pd_gemm_f32(int trans_a, int trans_b, int M, int N, int K, const 
     g.relu = relu != 0;
     g.a_vec = pd_aligned(A, 16) && lda % 4 == 0;
     g.b_vec = pd_aligned(B, 16) && ldb % 4 == 0;
+    g.k_per_split = K;
+    g.c_split = 0;
     hipStream_t s = (hipStream_t)stream;
     // Small problems use 64x64 tiles so that more of the 256 CUs get a block.
     long tiles128 = (long)((M + 127) / 128) * ((N + 127) / 128);
     if (tiles128 >= 256) return launch_gemm<128, 128>(trans_a, trans_b, g, s);
     return launch_gemm<64, 64>(trans_a, trans_b, g, s);
+}
+
+extern "C" int pd_gemm_splitk_f32(int trans_a, int trans_b, int M, int N, int K, const float* A, int lda,
+                                  const float* B, int ldb, float* partials, int splits, void* stream) {
+    PD_REQUIRE(M > 0 && N > 0 && K > 0 && splits >= 1 && splits <= 1024, PD_ESHAPE, "pd_gemm_splitk_f32: bad dimensions");
+    PD_REQUIRE(A && B && partials, PD_EINVAL, "pd_gemm_splitk_f32: NULL operand");
+    PD_REQUIRE(lda >= (trans_a ? M : K) && ldb >= (trans_b ? K : N), PD_ESHAPE,
+               "pd_gemm_splitk_f32: leading dimension smaller than the row length");
+    GemmArgs g;
+    g.A = A; g.B = B; g.C = partials; g.bias = nullptr;
+    g.M = M; g.N = N; g.K = K;
+    g.lda = lda; g.ldb = ldb; g.ldc = N;
+    g.beta = 0.f;
+    g.relu = 0;
+    g.a_vec = pd_aligned(A, 16) && lda % 4 == 0;
+    g.b_vec = pd_aligned(B, 16) && ldb % 4 == 0;
+    // every split gets a whole number of 16-wide k chunks; trailing splits may be empty and then write zeros
+    g.k_per_split = (((K + splits - 1) / splits) + BK - 1) / BK * BK;
+    g.c_split = (long long)M * N;
+    hipStream_t s = (hipStream_t)stream;
+    if (M > 64 && N >= 128) return launch_gemm<128, 128>(trans_a, trans_b, g, s, splits);
+    return launch_gemm<64, 64>(trans_a, trans_b, g, s, splits);
+}
+
+extern "C" int pd_splitk_reduce_f32(const float* partials, int splits, int M, int N, const float* bias, int relu,
+                                    float beta, float* C, int ldc, void* stream) {
+    PD_REQUIRE(M > 0 && N > 0 && N % 4 == 0 && splits >= 1 && ldc >= N && ldc % 4 == 0, PD_ESHAPE,
+               "pd_splitk_reduce_f32: need N and ldc multiples of 4");
+    PD_REQUIRE(partials && C && pd_aligned(partials, 16) && pd_aligned(C, 16) && (!bias || pd_aligned(bias, 16)), PD_EINVAL,
+               "pd_splitk_reduce_f32: NULL or unaligned pointer");
+    const long long total = (long long)M * (N / 4);
+    splitk_reduce_kernel<<<dim3((unsigned)((total + 255) / 256)), dim3(256), 0, (hipStream_t)stream>>>(
+        partials, splits, M, N, bias, relu != 0, beta, C, ldc);
+    PD_CHECK_LAUNCH("pd_splitk_reduce_f32");
+    return PD_OK;
 }

@@ -23,6 +23,7 @@ __device__ __forceinline__ float sigmoidf_(float x) { return 1.0f / (1.0f + expf
 // gates: [B][4H] pre-activations (x W_ih^T + h W_hh^T), overwritten with the ACTIVATED
 // gates i,f,g,o which the backward pass needs.  One thread = 4 consecutive hidden units.
 __global__ __launch_bounds__(LSTM_THREADS) void lstm_cell_fwd_kernel(float* __restrict__ gates,
+                                                                     const float* __restrict__ rec, int n_rec,
                                                                      const float* __restrict__ b_ih,
                                                                      const float* __restrict__ b_hh,
                                                                      const float* __restrict__ c_prev,
@@ -37,6 +38,13 @@ __global__ __launch_bounds__(LSTM_THREADS) void lstm_cell_fwd_kernel(float* __re
     float4_t gf = *(const float4_t*)(g + H + j);
     float4_t gg = *(const float4_t*)(g + 2 * H + j);
     float4_t go = *(const float4_t*)(g + 3 * H + j);
+    for (int s = 0; s < n_rec; ++s) {   // split-k partial sums of h_{t-1} W_hh^T, added in a fixed order
+        const float* r = rec + ((size_t)s * B + b) * 4 * H;
+        gi += *(const float4_t*)(r + j);
+        gf += *(const float4_t*)(r + H + j);
+        gg += *(const float4_t*)(r + 2 * H + j);
+        go += *(const float4_t*)(r + 3 * H + j);
+    }
     if (b_ih) {
         gi += *(const float4_t*)(b_ih + j) + *(const float4_t*)(b_hh + j);
         gf += *(const float4_t*)(b_ih + H + j) + *(const float4_t*)(b_hh + H + j);
@@ -69,7 +77,7 @@ __global__ __launch_bounds__(LSTM_THREADS) void lstm_cell_bwd_kernel(const float
                                                                      const float* __restrict__ c_prev,
                                                                      const float* __restrict__ c,
                                                                      const float* __restrict__ dy,
-                                                                     const float* __restrict__ dh_rec,
+                                                                     const float* __restrict__ dh_rec, int n_rec,
                                                                      float* __restrict__ dc_io,
                                                                      float* __restrict__ dgates, int B, int H,
                                                                      int first_step) {
@@ -87,7 +95,8 @@ __global__ __launch_bounds__(LSTM_THREADS) void lstm_cell_bwd_kernel(const float
     if (c_prev) cp = *(const float4_t*)(c_prev + o);
     const float4_t ct = *(const float4_t*)(c + o);
     float4_t dh = *(const float4_t*)(dy + o);
-    if (dh_rec) dh += *(const float4_t*)(dh_rec + o);
+    if (dh_rec)
+        for (int s = 0; s < n_rec; ++s) dh += *(const float4_t*)(dh_rec + (size_t)s * B * H + o);
     float4_t dc = {0.f, 0.f, 0.f, 0.f};
     if (!first_step) dc = *(const float4_t*)(dc_io + o);
     float4_t di, df, dg, dO, dcp;
@@ -172,8 +181,10 @@ __global__ __launch_bounds__(LSTM_THREADS) void embedding_bwd_kernel(const int64
 
 }  // namespace
 
-extern "C" int pd_lstm_cell_fwd_f32(float* gates, const float* b_ih, const float* b_hh, const float* c_prev,
-                                    float* c_out, float* h_out, int B, int H, void* stream) {
+extern "C" int pd_lstm_cell_fwd_f32(float* gates, const float* rec, int n_rec, const float* b_ih, const float* b_hh,
+                                    const float* c_prev, float* c_out, float* h_out, int B, int H, void* stream) {
+    PD_REQUIRE(n_rec >= 0 && (n_rec == 0 || (rec && pd_aligned(rec, 16))), PD_EINVAL,
+               "pd_lstm_cell_fwd_f32: rec must be a 16-byte aligned pointer when n_rec > 0");
     PD_REQUIRE(B > 0 && H > 0 && H % 4 == 0, PD_ESHAPE, "pd_lstm_cell_fwd_f32: need B > 0 and H a positive multiple of 4");
     PD_REQUIRE(gates && c_out && h_out, PD_EINVAL, "pd_lstm_cell_fwd_f32: NULL pointer");
     PD_REQUIRE((b_ih == nullptr) == (b_hh == nullptr), PD_EINVAL, "pd_lstm_cell_fwd_f32: pass both biases or neither");
@@ -182,14 +193,15 @@ extern "C" int pd_lstm_cell_fwd_f32(float* gates, const float* b_ih, const float
                PD_EINVAL, "pd_lstm_cell_fwd_f32: pointers must be 16-byte aligned");
     const int total = B * (H / 4);
     lstm_cell_fwd_kernel<<<dim3((total + LSTM_THREADS - 1) / LSTM_THREADS), dim3(LSTM_THREADS), 0,
-                           (hipStream_t)stream>>>(gates, b_ih, b_hh, c_prev, c_out, h_out, B, H);
+                           (hipStream_t)stream>>>(gates, rec, n_rec, b_ih, b_hh, c_prev, c_out, h_out, B, H);
     PD_CHECK_LAUNCH("pd_lstm_cell_fwd_f32");
     return PD_OK;
 }
 
 extern "C" int pd_lstm_cell_bwd_f32(const float* gates, const float* c_prev, const float* c, const float* dy,
-                                    const float* dh_rec, float* dc_io, float* dgates, int B, int H, int first_step,
-                                    void* stream) {
+                                    const float* dh_rec, int n_rec, float* dc_io, float* dgates, int B, int H,
+                                    int first_step, void* stream) {
+    PD_REQUIRE(!dh_rec || n_rec >= 1, PD_EINVAL, "pd_lstm_cell_bwd_f32: dh_rec needs n_rec >= 1");
     PD_REQUIRE(B > 0 && H > 0 && H % 4 == 0, PD_ESHAPE, "pd_lstm_cell_bwd_f32: need B > 0 and H a positive multiple of 4");
     PD_REQUIRE(gates && c && dy && dc_io && dgates, PD_EINVAL, "pd_lstm_cell_bwd_f32: NULL pointer");
     PD_REQUIRE(pd_aligned(gates, 16) && pd_aligned(c, 16) && pd_aligned(dy, 16) && pd_aligned(dc_io, 16) &&
@@ -197,7 +209,7 @@ extern "C" int pd_lstm_cell_bwd_f32(const float* gates, const float* c_prev, con
                PD_EINVAL, "pd_lstm_cell_bwd_f32: pointers must be 16-byte aligned");
     const int total = B * (H / 4);
     lstm_cell_bwd_kernel<<<dim3((total + LSTM_THREADS - 1) / LSTM_THREADS), dim3(LSTM_THREADS), 0,
-                           (hipStream_t)stream>>>(gates, c_prev, c, dy, dh_rec, dc_io, dgates, B, H, first_step);
+                           (hipStream_t)stream>>>(gates, c_prev, c, dy, dh_rec, n_rec, dc_io, dgates, B, H, first_step);
     PD_CHECK_LAUNCH("pd_lstm_cell_bwd_f32");
     return PD_OK;
 }

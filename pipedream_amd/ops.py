@@ -81,9 +81,49 @@ def gemm(a, b, trans_a=False, trans_b=False, bias=None, relu=False, out=None, be
     lda = a.stride(0) if a.size(0) > 1 else a.size(1)
     ldb = b.stride(0) if b.size(0) > 1 else b.size(1)
     ldc = out.stride(0) if out.size(0) > 1 else out.size(1)
+    splits = splitk_factor(M, N, K)
+    if splits > 1 and N % 4 == 0 and ldc % 4 == 0 and out.data_ptr() % 16 == 0:
+        # too few output tiles for 256 CUs: split k over more blocks, then one fused reduce + epilogue
+        part = torch.empty((splits, M, N), dtype=torch.float32, device=a.device)
+        _cabi.lib().pd_gemm_splitk_f32(int(trans_a), int(trans_b), M, N, K, _ptr(a), lda, _ptr(b), ldb, _ptr(part),
+                                       splits, _cabi.stream_ptr())
+        _cabi.lib().pd_splitk_reduce_f32(_ptr(part), splits, M, N, _ptr(bias), int(relu), float(beta), _ptr(out), ldc,
+                                         _cabi.stream_ptr())
+        return out
     _cabi.lib().pd_gemm_f32(int(trans_a), int(trans_b), M, N, K, _ptr(a), lda, _ptr(b), ldb, float(beta),
                             _ptr(out), ldc, _ptr(bias), int(relu), _cabi.stream_ptr())
     return out
+
+
+SPLITK_TARGET_BLOCKS = 256     # one block per CU
+SPLITK_MIN_K = 128             # k per split is never smaller than this
+
+
+def splitk_factor(M, N, K):
+    """Number of k ranges a product is split into so that about one block per CU runs (1 = no split).
+    Mirrors the tile choice of pd_gemm_splitk_f32: 128 x 128 tiles when M > 64 and N >= 128, else 64 x 64."""
+    t = 128 if (M > 64 and N >= 128) else 64
+    tiles = -(-M // t) * -(-N // t)
+    if tiles * 2 > SPLITK_TARGET_BLOCKS or K < 2 * SPLITK_MIN_K:
+        return 1
+    return max(1, min(SPLITK_TARGET_BLOCKS // tiles, K // SPLITK_MIN_K, 64))
+
+
+def gemm_splitk(a, b, trans_a, trans_b, partials):
+    """partials[s] = op(a)[:, k range s] @ op(b)[k range s, :] for s < partials.size(0); the consumer sums them."""
+    _rowmajor2d(a, "a")
+    _rowmajor2d(b, "b")
+    M, K = (a.size(1), a.size(0)) if trans_a else (a.size(0), a.size(1))
+    Kb, N = (b.size(1), b.size(0)) if trans_b else (b.size(0), b.size(1))
+    if K != Kb or partials.dim() != 3 or tuple(partials.shape[1:]) != (M, N) or not partials.is_contiguous():
+        raise ValueError("gemm_splitk: shapes %s x %s -> %s do not fit" % (tuple(a.shape), tuple(b.shape),
+                                                                            tuple(partials.shape)))
+    _check(partials, "partials")
+    lda = a.stride(0) if a.size(0) > 1 else a.size(1)
+    ldb = b.stride(0) if b.size(0) > 1 else b.size(1)
+    _cabi.lib().pd_gemm_splitk_f32(int(trans_a), int(trans_b), M, N, K, _ptr(a), lda, _ptr(b), ldb, _ptr(partials),
+                                   partials.size(0), _cabi.stream_ptr())
+    return partials
 
 
 def colsum(x, out=None, beta=0.0):
@@ -328,11 +368,13 @@ def lstm_forward(x, w_ih, w_hh, b_ih, b_hh):
     gates = gemm(x2, w_ih, trans_b=True).view(T, B, 4 * H)
     y = torch.empty((T, B, H), dtype=torch.float32, device=x.device)
     c = torch.empty((T, B, H), dtype=torch.float32, device=x.device)
+    # the recurrent product h_{t-1} W_hh^T has only B rows: split over k, summed inside the cell kernel
+    rec = torch.empty((splitk_factor(B, 4 * H, H), B, 4 * H), dtype=torch.float32, device=x.device)
     for t in range(T):
         if t > 0:
-            gemm(y[t - 1], w_hh, trans_b=True, out=gates[t], beta=1.0)
-        lib.pd_lstm_cell_fwd_f32(_ptr(gates[t]), _ptr(b_ih), _ptr(b_hh), _ptr(c[t - 1]) if t > 0 else None,
-                                 _ptr(c[t]), _ptr(y[t]), B, H, s())
+            gemm_splitk(y[t - 1], w_hh, False, True, rec)
+        lib.pd_lstm_cell_fwd_f32(_ptr(gates[t]), _ptr(rec), rec.size(0) if t > 0 else 0, _ptr(b_ih), _ptr(b_hh),
+                                 _ptr(c[t - 1]) if t > 0 else None, _ptr(c[t]), _ptr(y[t]), B, H, s())
     return y, (gates, c)
 
 
@@ -344,12 +386,13 @@ def lstm_backward(dy, x, y, gates, c, w_ih, w_hh, need_dx=True):
     lib, s = _cabi.lib(), _cabi.stream_ptr
     dgates = torch.empty((T, B, 4 * H), dtype=torch.float32, device=x.device)
     dc = torch.empty((B, H), dtype=torch.float32, device=x.device)
-    dh_rec = None
+    dh_rec = torch.empty((splitk_factor(B, H, 4 * H), B, H), dtype=torch.float32, device=x.device)
     for t in range(T - 1, -1, -1):
         lib.pd_lstm_cell_bwd_f32(_ptr(gates[t]), _ptr(c[t - 1]) if t > 0 else None, _ptr(c[t]), _ptr(dy[t]),
-                                 _ptr(dh_rec), _ptr(dc), _ptr(dgates[t]), B, H, int(t == T - 1), s())
+                                 _ptr(dh_rec) if t < T - 1 else None, dh_rec.size(0), _ptr(dc), _ptr(dgates[t]), B, H,
+                                 int(t == T - 1), s())
         if t > 0:
-            dh_rec = gemm(dgates[t], w_hh)                      # [B,4H] @ [4H,H]
+            gemm_splitk(dgates[t], w_hh, False, False, dh_rec)      # [B,4H] @ [4H,H], split over 4H
     dg2 = dgates.view(T * B, 4 * H)
     x2 = x.contiguous().view(T * B, I)
     dw_ih = gemm(dg2, x2, trans_a=True)
