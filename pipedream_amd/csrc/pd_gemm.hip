@@ -217,6 +217,210 @@ int launch_gemm(int trans_a, int trans_b, const GemmArgs& g, hipStream_t s, int 
     return PD_OK;
 }
 
+// ---------------------------------------------------------------------------------------
+// Skinny split-k kernel: M <= 128 (the LSTM recurrent products with M = batch, the
+// classifier layers with M = 64), A k-contiguous.  A block owns all M rows x 128 columns
+// of one k range and is bound by fetching its operands, so they are streamed with 128-bit
+// direct-to-LDS loads (lane l's 16 bytes land at <base> + 16*l) through a ring of 8
+// stages of 16 k, 6 to 7 stages in flight, and multiplied as they arrive.
+// Because the LDS placement of such a load is fixed, the lanes fetch a permutation that
+// makes the fragment reads conflict-free: the 16-byte slot q of row r of a k-contiguous
+// stage holds k-group q ^ ((r >> 2) & 3); a row-contiguous stage ([k][128 columns]) has its
+// two 256-byte halves swapped for k % 8 >= 4.
+// The fragment reads are inline assembly: the compiler cannot tell which ring stage a
+// direct-to-LDS load writes and would wait for all loads in flight before any LDS read;
+// here the wait is an explicit vmcnt that leaves the younger stages in flight.  Stage
+// numbers past the end of the k range re-fetch the last stage (and are not multiplied), so
+// the number of loads in flight is the same in every iteration.
+typedef __attribute__((address_space(3))) void* lds_void_ptr;
+typedef __attribute__((address_space(1))) const void* global_void_ptr;
+
+constexpr int SK_COLS = 128;             // tile columns
+constexpr int SK_STAGES = 8;             // ring stages of BK = 16
+
+// WM = 2: up to 128 rows, waves 2 x 2, 64 x 64 each.  WM = 1: up to 64 rows, waves 1 x 4, 64 x 32 each.
+template <int WM, bool B_KC>
+struct Skinny {
+    static constexpr int BM = 64 * WM;
+    static constexpr int WN = 4 / WM;
+    static constexpr int TN = SK_COLS / (32 * WN);
+    static constexpr int A_STAGE = BM * BK * 4, B_STAGE = SK_COLS * BK * 4;
+    static constexpr int B_BASE = SK_STAGES * A_STAGE;
+    static constexpr int LDS_BYTES = SK_STAGES * (A_STAGE + B_STAGE);
+    static constexpr int A_PER_WAVE = BM / 16 / 4, B_PER_WAVE = SK_COLS / 16 / 4;
+    static constexpr int IPT = A_PER_WAVE + B_PER_WAVE;      // loads per lane and stage
+    static constexpr int IN_FLIGHT = SK_STAGES - 2;           // younger stages outstanding at the wait
+
+    size_t src_a[A_PER_WAVE], src_b[B_PER_WAVE];
+    uint32_t fa_addr[2][2], fb_addr[TN][2];       // [fragment][k-group g] LDS byte addresses, stage 0
+
+    __device__ __forceinline__ void init(const GemmArgs& a, int n0, int wave, int lane, uint32_t lds_base) {
+        const int wm = wave / WN, wn = wave % WN;
+        const int idx = lane % 32, h = lane / 32;
+#pragma unroll
+        for (int t = 0; t < A_PER_WAVE; ++t) {
+            const int row = (wave + 4 * t) * 16 + lane / 4;
+            const int kq = (lane % 4) ^ ((row >> 2) & 3);
+            src_a[t] = (size_t)min(row, a.M - 1) * a.lda + kq * 4;
+        }
+#pragma unroll
+        for (int t = 0; t < B_PER_WAVE; ++t) {
+            const int n = wave + 4 * t;
+            if (B_KC) {
+                const int row = n * 16 + lane / 4;
+                const int kq = (lane % 4) ^ ((row >> 2) & 3);
+                src_b[t] = (size_t)min(n0 + row, a.N - 1) * a.ldb + kq * 4;
+            } else {
+                const int k = 2 * n + lane / 32;
+                int col = ((lane % 32) ^ (((k >> 2) & 1) << 4)) * 4;
+                if (n0 + col >= a.N) col = 0;
+                src_b[t] = (size_t)k * a.ldb + n0 + col;
+            }
+        }
+#pragma unroll
+        for (int g = 0; g < 2; ++g) {
+#pragma unroll
+            for (int i = 0; i < 2; ++i) {
+                const int r = (wm * 2 + i) * 32 + idx;
+                fa_addr[i][g] = lds_base + r * 64 + (((2 * g + h) ^ ((r >> 2) & 3)) * 16);
+            }
+#pragma unroll
+            for (int j = 0; j < TN; ++j) {
+                const int r = (wn * TN + j) * 32 + idx;
+                if (B_KC) fb_addr[j][g] = lds_base + B_BASE + r * 64 + (((2 * g + h) ^ ((r >> 2) & 3)) * 16);
+                else fb_addr[j][g] = lds_base + B_BASE + ((8 * g + 4 * h) * SK_COLS + (r ^ (h << 6))) * 4;
+            }
+        }
+    }
+
+    template <int ST>
+    __device__ __forceinline__ void issue(const GemmArgs& a, char* lds, int k, int wave) const {
+#pragma unroll
+        for (int t = 0; t < A_PER_WAVE; ++t)
+            __builtin_amdgcn_global_load_lds((global_void_ptr)(a.A + src_a[t] + k),
+                                             (lds_void_ptr)(lds + ST * A_STAGE + (wave + 4 * t) * 1024), 16, 0, 0);
+#pragma unroll
+        for (int t = 0; t < B_PER_WAVE; ++t)
+            __builtin_amdgcn_global_load_lds((global_void_ptr)(a.B + src_b[t] + (B_KC ? (size_t)k : (size_t)k * a.ldb)),
+                                             (lds_void_ptr)(lds + B_BASE + ST * B_STAGE + (wave + 4 * t) * 1024), 16, 0, 0);
+    }
+
+    // fragments of ring stage ST: fa[i][g], fb[j][g] (4 consecutive k-steps each)
+    template <int ST>
+    __device__ __forceinline__ void read(float4_t (&fa)[2][2], float4_t (&fb)[TN][2]) const {
+#pragma unroll
+        for (int g = 0; g < 2; ++g) {
+#pragma unroll
+            for (int i = 0; i < 2; ++i)
+                asm volatile("ds_read_b128 %0, %1 offset:%2" : "=v"(fa[i][g]) : "v"(fa_addr[i][g]), "n"(ST * A_STAGE) : "memory");
+#pragma unroll
+            for (int j = 0; j < TN; ++j) {
+                if (B_KC) {
+                    asm volatile("ds_read_b128 %0, %1 offset:%2" : "=v"(fb[j][g]) : "v"(fb_addr[j][g]), "n"(ST * B_STAGE) : "memory");
+                } else {
+                    float q0, q1, q2, q3;
+                    asm volatile("ds_read_b32 %0, %1 offset:%2" : "=v"(q0) : "v"(fb_addr[j][g]), "n"(ST * B_STAGE) : "memory");
+                    asm volatile("ds_read_b32 %0, %1 offset:%2" : "=v"(q1) : "v"(fb_addr[j][g]), "n"(ST * B_STAGE + SK_COLS * 4) : "memory");
+                    asm volatile("ds_read_b32 %0, %1 offset:%2" : "=v"(q2) : "v"(fb_addr[j][g]), "n"(ST * B_STAGE + 2 * SK_COLS * 4) : "memory");
+                    asm volatile("ds_read_b32 %0, %1 offset:%2" : "=v"(q3) : "v"(fb_addr[j][g]), "n"(ST * B_STAGE + 3 * SK_COLS * 4) : "memory");
+                    asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(q0), "+v"(q1), "+v"(q2), "+v"(q3));
+                    fb[j][g] = float4_t{q0, q1, q2, q3};
+                }
+            }
+        }
+        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+#pragma unroll
+        for (int g = 0; g < 2; ++g) {
+#pragma unroll
+            for (int i = 0; i < 2; ++i) asm volatile("" : "+v"(fa[i][g]));
+#pragma unroll
+            for (int j = 0; j < TN; ++j) asm volatile("" : "+v"(fb[j][g]));
+        }
+    }
+};
+
+template <int N>
+__device__ __forceinline__ void sk_wait_vmcnt() {
+    // vmcnt is split over bits [3:0] and [15:14]; expcnt and lgkmcnt left unconstrained
+    __builtin_amdgcn_s_waitcnt((N & 15) | ((N >> 4) << 14) | (7 << 4) | (15 << 8));
+}
+
+template <int WM, bool B_KC>
+__global__ __launch_bounds__(GEMM_THREADS) void pd_gemm_skinny_kernel(const GemmArgs a) {
+    using S = Skinny<WM, B_KC>;
+    constexpr int TN = S::TN;
+    __shared__ __attribute__((aligned(1024))) char lds[S::LDS_BYTES];
+    const int lane = threadIdx.x % 64;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / 64);
+    const int wm = wave / S::WN, wn = wave % S::WN;
+    const int idx = lane % 32, h = lane / 32;
+    const int n0 = blockIdx.x * SK_COLS;
+    const int k_begin = blockIdx.z * a.k_per_split;
+    const int k_end = min(a.K, k_begin + a.k_per_split);
+    const int total = k_end > k_begin ? (k_end - k_begin) / BK : 0;      // stages to multiply
+    float* const C = a.C + blockIdx.z * a.c_split;
+
+    float16_t acc[2][TN];
+#pragma unroll
+    for (int i = 0; i < 2; ++i)
+#pragma unroll
+        for (int j = 0; j < TN; ++j)
+#pragma unroll
+            for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.f;
+
+    if (total > 0) {
+        S sk;
+        sk.init(a, n0, wave, lane, (uint32_t)(size_t)(lds_void_ptr)lds);
+        // k of stage number i, clamped to the last stage of the range
+#define SK_K(i) (k_begin + min((i), total - 1) * BK)
+        sk.template issue<0>(a, lds, SK_K(0), wave);
+        sk.template issue<1>(a, lds, SK_K(1), wave);
+        sk.template issue<2>(a, lds, SK_K(2), wave);
+        sk.template issue<3>(a, lds, SK_K(3), wave);
+        sk.template issue<4>(a, lds, SK_K(4), wave);
+        sk.template issue<5>(a, lds, SK_K(5), wave);
+        sk.template issue<6>(a, lds, SK_K(6), wave);
+        static_assert(SK_STAGES == 8, "the ring fill and the unrolled loop are written for 8 stages");
+        // Stage i (ring slot ST): wait until it has landed everywhere; every wave is then also past
+        // its reads of stage i-1, so that slot is refilled with stage i+7; then read and multiply.
+#define SK_STAGE(ST)                                                                                      \
+        {                                                                                                     \
+            const int i = i0 + ST;                                                                            \
+            sk_wait_vmcnt<S::IN_FLIGHT * S::IPT>();                                                          \
+            __builtin_amdgcn_s_barrier();                                                                     \
+            sk.template issue<(ST + 7) % 8>(a, lds, SK_K(i + 7), wave);                                      \
+            if (i < total) {                                                                                  \
+                float4_t fa[2][2], fb[TN][2];                                                                 \
+                sk.template read<ST>(fa, fb);                                                                 \
+                _Pragma("unroll") for (int g = 0; g < 2; ++g)                                                 \
+                _Pragma("unroll") for (int q = 0; q < 4; ++q)                                                 \
+                _Pragma("unroll") for (int ii = 0; ii < 2; ++ii)                                              \
+                _Pragma("unroll") for (int jj = 0; jj < TN; ++jj)                                             \
+                    acc[ii][jj] = __builtin_amdgcn_mfma_f32_32x32x2f32(fa[ii][g][q], fb[jj][g][q], acc[ii][jj], 0, 0, 0); \
+            }                                                                                                 \
+        }
+        for (int i0 = 0; i0 < total; i0 += SK_STAGES) {
+            SK_STAGE(0) SK_STAGE(1) SK_STAGE(2) SK_STAGE(3) SK_STAGE(4) SK_STAGE(5) SK_STAGE(6) SK_STAGE(7)
+        }
+#undef SK_STAGE
+#undef SK_K
+        sk_wait_vmcnt<0>();     // the trailing re-fetches must not outlive the block's LDS allocation
+    }
+
+#pragma unroll
+    for (int i = 0; i < 2; ++i)
+#pragma unroll
+        for (int j = 0; j < TN; ++j) {
+            const int col = n0 + (wn * TN + j) * 32 + idx;
+            if (col >= a.N) continue;
+#pragma unroll
+            for (int e = 0; e < 16; ++e) {
+                const int row = (wm * 2 + i) * 32 + 8 * (e / 4) + 4 * h + (e % 4);
+                if (row < a.M) C[(size_t)row * a.ldc + col] = acc[i][j][e];
+            }
+        }
+}
+
 // out = (sum over splits of partials) (+ bias) (+ beta*out) (relu): 4 elements per thread
 __global__ __launch_bounds__(256) void splitk_reduce_kernel(const float* __restrict__ partials, int splits, int M, int N,
                                                            const float* __restrict__ bias, int relu, float beta,
@@ -281,6 +485,19 @@ extern "C" int pd_gemm_splitk_f32(int trans_a, int trans_b, int M, int N, int K,
     g.k_per_split = (((K + splits - 1) / splits) + BK - 1) / BK * BK;
     g.c_split = (long long)M * N;
     hipStream_t s = (hipStream_t)stream;
+    if (!trans_a && M <= 128 && N % 4 == 0 && g.a_vec && g.b_vec && g.k_per_split % BK == 0 && K % BK == 0 &&
+        (size_t)128 * (lda > ldb ? lda : ldb) * 4 < (1ull << 31)) {
+        const dim3 grid((N + SK_COLS - 1) / SK_COLS, 1, splits);
+        if (M <= 64) {
+            if (trans_b) pd_gemm_skinny_kernel<1, true><<<grid, GEMM_THREADS, 0, s>>>(g);
+            else pd_gemm_skinny_kernel<1, false><<<grid, GEMM_THREADS, 0, s>>>(g);
+        } else {
+            if (trans_b) pd_gemm_skinny_kernel<2, true><<<grid, GEMM_THREADS, 0, s>>>(g);
+            else pd_gemm_skinny_kernel<2, false><<<grid, GEMM_THREADS, 0, s>>>(g);
+        }
+        PD_CHECK_LAUNCH("pd_gemm_splitk_f32");
+        return PD_OK;
+    }
     if (M > 64 && N >= 128) return launch_gemm<128, 128>(trans_a, trans_b, g, s, splits);
     return launch_gemm<64, 64>(trans_a, trans_b, g, s, splits);
 }

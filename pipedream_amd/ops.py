@@ -81,8 +81,10 @@ def gemm(a, b, trans_a=False, trans_b=False, bias=None, relu=False, out=None, be
     lda = a.stride(0) if a.size(0) > 1 else a.size(1)
     ldb = b.stride(0) if b.size(0) > 1 else b.size(1)
     ldc = out.stride(0) if out.size(0) > 1 else out.size(1)
-    splits = splitk_factor(M, N, K)
-    if splits > 1 and N % 4 == 0 and ldc % 4 == 0 and out.data_ptr() % 16 == 0:
+    splits = splitk_factor(M, N, K, trans_a)
+    # M <= 128: the streaming kernel behind pd_gemm_splitk_f32 also wins without a split (one partial)
+    skinny = not trans_a and M <= 128 and K % 16 == 0 and K >= 256 and N >= 128
+    if (splits > 1 or skinny) and N % 4 == 0 and ldc % 4 == 0 and out.data_ptr() % 16 == 0:
         # too few output tiles for 256 CUs: split k over more blocks, then one fused reduce + epilogue
         part = torch.empty((splits, M, N), dtype=torch.float32, device=a.device)
         _cabi.lib().pd_gemm_splitk_f32(int(trans_a), int(trans_b), M, N, K, _ptr(a), lda, _ptr(b), ldb, _ptr(part),
@@ -99,11 +101,16 @@ SPLITK_TARGET_BLOCKS = 256     # one block per CU
 SPLITK_MIN_K = 128             # k per split is never smaller than this
 
 
-def splitk_factor(M, N, K):
+def splitk_factor(M, N, K, trans_a=False):
     """Number of k ranges a product is split into so that about one block per CU runs (1 = no split).
-    Mirrors the tile choice of pd_gemm_splitk_f32: 128 x 128 tiles when M > 64 and N >= 128, else 64 x 64."""
-    t = 128 if (M > 64 and N >= 128) else 64
-    tiles = -(-M // t) * -(-N // t)
+    Mirrors the tile choice of pd_gemm_splitk_f32: its streaming kernel for M <= 128 (A not transposed,
+    K a multiple of 16) owns all rows x 128 columns per block; otherwise tiles are 128 x 128 when M > 64
+    and N >= 128, else 64 x 64."""
+    if not trans_a and M <= 128 and K % 16 == 0:
+        tiles = -(-N // 128)
+    else:
+        t = 128 if (M > 64 and N >= 128) else 64
+        tiles = -(-M // t) * -(-N // t)
     if tiles * 2 > SPLITK_TARGET_BLOCKS or K < 2 * SPLITK_MIN_K:
         return 1
     return max(1, min(SPLITK_TARGET_BLOCKS // tiles, K // SPLITK_MIN_K, 64))

@@ -51,6 +51,32 @@ def test_gemm_epilogues():
     _gemm_case(300, 300, 300, False, False, bias=True, relu=True, beta=0.5)
 
 
+@pytest.mark.parametrize("M,N,K,ta,tb", [
+    (128, 4096, 1024, False, True),     # LSTM recurrent forward: direct-to-LDS skinny kernel, k-contiguous B
+    (128, 1024, 4096, False, False),    # LSTM recurrent backward: row-contiguous B
+    (64, 1000, 4096, False, True),      # classifier: N not a multiple of the 128-column tile
+    (5, 260, 2048, False, False),       # few rows, ragged columns
+    (100, 132, 1040, False, True),      # K a multiple of 16 but not of 128: a short last round
+    (64, 256, 1030, False, True),       # K not a multiple of 16: general split kernel
+    (96, 512, 2048, True, False),       # transposed A: general split kernel
+])
+def test_gemm_split_k_paths(M, N, K, ta, tb):
+    """Products with too few output tiles are split over k (ops.splitk_factor > 1); partial
+    sums are added in a fixed order, so the result is reproducible bit for bit."""
+    assert ops.splitk_factor(M, N, K, ta) > 1
+    _gemm_case(M, N, K, ta, tb)
+    _gemm_case(M, N, K, ta, tb, bias=True, relu=True, beta=0.5)
+    g = torch.Generator().manual_seed(1)
+    a = torch.randn((K, M) if ta else (M, K), generator=g).cuda()
+    b = torch.randn((N, K) if tb else (K, N), generator=g).cuda()
+    assert torch.equal(ops.gemm(a, b, trans_a=ta, trans_b=tb), ops.gemm(a, b, trans_a=ta, trans_b=tb))
+    # explicit partials: more splits than k chunks leaves trailing partials at zero
+    part = torch.full((70, M, N), float("nan")).cuda()
+    ops.gemm_splitk(a, b, ta, tb, part)
+    want = (a.double().t() if ta else a.double()) @ (b.double().t() if tb else b.double())
+    torch.testing.assert_close(part.double().sum(0), want, rtol=1e-5, atol=2e-6 * math.sqrt(K) * 9.0)
+
+
 def test_gemm_strided_views_and_identity():
     # leading dimension larger than the row; unaligned base (scalar load path)
     big = torch.randn(70, 90).cuda()
