@@ -247,8 +247,17 @@ __global__ __launch_bounds__(PW_THREADS) void colsum_kernel(const float* __restr
     const uint64_t r0 = blockIdx.y * rows_per;
     const uint64_t r1 = (r0 + rows_per < M) ? r0 + rows_per : M;
     float s = 0.f;
-    if (col < N)
-        for (uint64_t r = r0 + w; r < r1; r += 4) s += x[r * ld + col];
+    if (col < N) {
+        // 8 independent loads in flight per lane (a chain of dependent adds would be latency-bound);
+        // the order of the additions is fixed, so the result is reproducible
+        float t[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+        uint64_t r = r0 + w;
+        for (; r + 28 < r1; r += 32)
+#pragma unroll
+            for (int u = 0; u < 8; ++u) t[u] += x[(r + 4 * u) * ld + col];
+        for (; r < r1; r += 4) t[0] += x[r * ld + col];
+        s = ((t[0] + t[1]) + (t[2] + t[3])) + ((t[4] + t[5]) + (t[6] + t[7]));
+    }
     part[w][threadIdx.x % 64] = s;
     __syncthreads();
     if (w == 0 && col < N) {

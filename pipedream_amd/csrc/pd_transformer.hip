@@ -114,7 +114,7 @@ __global__ __launch_bounds__(TR_THREADS) void layernorm_fwd_kernel(const uint16_
 
 // dx for each row; per-block partial sums of dgamma / dbeta over the block's rows.
 // A block handles ROWS_PER_BLOCK rows, each wave every 4th of them.
-constexpr int LN_ROWS_PER_BLOCK = 32;
+constexpr int LN_ROWS_PER_BLOCK = 8;
 
 __global__ __launch_bounds__(TR_THREADS) void layernorm_bwd_kernel(const uint16_t* __restrict__ dy,
                                                                    const uint16_t* __restrict__ x,
@@ -203,18 +203,23 @@ __global__ __launch_bounds__(TR_THREADS) void softmax_fwd_kernel(const uint16_t*
     float m = -INFINITY;
 #pragma unroll
     for (int v = 0; v < MAX_VEC; ++v)
+        if (v < r.nvec) {            // wave-uniform: rows shorter than 2048 skip the unused vectors
 #pragma unroll
-        for (int k = 0; k < 8; ++k)
-            if ((v * 64 + lane) * 8 + k < n) m = fmaxf(m, r.x[v][k]);
+            for (int k = 0; k < 8; ++k)
+                if ((v * 64 + lane) * 8 + k < n) m = fmaxf(m, r.x[v][k]);
+        }
     m = wave_max(m);
     float s = 0.f;
 #pragma unroll
     for (int v = 0; v < MAX_VEC; ++v)
+        if (v < r.nvec) {
 #pragma unroll
-        for (int k = 0; k < 8; ++k) {
-            const bool in = (v * 64 + lane) * 8 + k < n;
-            r.x[v][k] = in ? expf(r.x[v][k] - m) : 0.f;
-            s += r.x[v][k];
+            for (int k = 0; k < 8; ++k) {
+                const bool in = (v * 64 + lane) * 8 + k < n;
+                // e^(x-m) = 2^((x-m) log2 e) on the hardware exp2 (about 1 ulp; the result is rounded to bf16)
+                r.x[v][k] = in ? __builtin_amdgcn_exp2f((r.x[v][k] - m) * 1.44269504088896340736f) : 0.f;
+                s += r.x[v][k];
+            }
         }
     const float inv = 1.0f / wave_sum(s);
 #pragma unroll
@@ -241,8 +246,10 @@ __global__ __launch_bounds__(TR_THREADS) void softmax_bwd_kernel(const uint16_t*
     float s = 0.f;
 #pragma unroll
     for (int v = 0; v < MAX_VEC; ++v)
+        if (v < ry.nvec) {
 #pragma unroll
-        for (int k = 0; k < 8; ++k) s += ry.x[v][k] * rd.x[v][k];
+            for (int k = 0; k < 8; ++k) s += ry.x[v][k] * rd.x[v][k];
+        }
     s = wave_sum(s);
 #pragma unroll
     for (int v = 0; v < MAX_VEC; ++v) {
@@ -307,24 +314,40 @@ __global__ __launch_bounds__(TR_THREADS) void cast_bf16_f32_kernel(const uint16_
     for (uint64_t k = i; k < n && k < i + 4; ++k) y[k] = bf2f(x[k]);
 }
 
-// Column sums of a bf16 [M][N] matrix into fp32 partials out[split][N].
+// Column sums of a bf16 [M][N] matrix into fp32 partials out[split][N].  A lane owns 8
+// adjacent columns (one 16-byte load per row), a block 512 columns; its 4 waves take every
+// 4th row of the split and are combined through LDS in a fixed order.
 __global__ __launch_bounds__(TR_THREADS) void colsum_bf16_kernel(const uint16_t* __restrict__ x,
                                                                  float* __restrict__ out, uint64_t M, int N,
-                                                                 uint64_t ld) {
-    __shared__ float part[4][64];
-    const int col = blockIdx.x * 64 + threadIdx.x % 64;
-    const int w = threadIdx.x / 64;
+                                                                 uint64_t ld, int vec) {
+    __shared__ float part[4][512];
+    const int lane = threadIdx.x % 64, w = threadIdx.x / 64;
+    const int col = blockIdx.x * 512 + lane * 8;
     const uint64_t rows_per = (M + gridDim.y - 1) / gridDim.y;
     const uint64_t r0 = blockIdx.y * rows_per;
     const uint64_t r1 = (r0 + rows_per < M) ? r0 + rows_per : M;
-    float s = 0.f;
-    if (col < N)
-        for (uint64_t r = r0 + w; r < r1; r += 4) s += bf2f(x[r * ld + col]);
-    part[w][threadIdx.x % 64] = s;
+    float s[8];
+#pragma unroll
+    for (int k = 0; k < 8; ++k) s[k] = 0.f;
+    if (vec && col + 8 <= N) {
+        for (uint64_t r = r0 + w; r < r1; r += 4) {
+            const u16x8 v = *(const u16x8*)(x + r * ld + col);
+#pragma unroll
+            for (int k = 0; k < 8; ++k) s[k] += bf2f(v[k]);
+        }
+    } else {
+        for (uint64_t r = r0 + w; r < r1; r += 4)
+#pragma unroll
+            for (int k = 0; k < 8; ++k)
+                if (col + k < N) s[k] += bf2f(x[r * ld + col + k]);
+    }
+#pragma unroll
+    for (int k = 0; k < 8; ++k) part[w][lane * 8 + k] = s[k];
     __syncthreads();
-    if (w == 0 && col < N)
-        out[(uint64_t)blockIdx.y * N + col] =
-            (part[0][threadIdx.x] + part[1][threadIdx.x]) + (part[2][threadIdx.x] + part[3][threadIdx.x]);
+    for (int c = threadIdx.x; c < 512; c += TR_THREADS) {
+        const int gc = blockIdx.x * 512 + c;
+        if (gc < N) out[(uint64_t)blockIdx.y * N + gc] = (part[0][c] + part[1][c]) + (part[2][c] + part[3][c]);
+    }
 }
 
 int row_args_ok(const char* who, long long rows, int n) {
@@ -446,7 +469,8 @@ extern "C" int pd_colsum_bf16(const uint16_t* x, float* out, uint64_t M, int N, 
     if (N == 0) return PD_OK;
     PD_REQUIRE(x && out, PD_EINVAL, "pd_colsum_bf16: NULL operand");
     PD_REQUIRE(ld >= (uint64_t)N, PD_ESHAPE, "pd_colsum_bf16: ld < N");
-    colsum_bf16_kernel<<<dim3((N + 63) / 64, splits), dim3(TR_THREADS), 0, (hipStream_t)stream>>>(x, out, M, N, ld);
+    const int vec = pd_aligned(x, 16) && ld % 8 == 0;
+    colsum_bf16_kernel<<<dim3((N + 511) / 512, splits), dim3(TR_THREADS), 0, (hipStream_t)stream>>>(x, out, M, N, ld, vec);
     PD_CHECK_LAUNCH("pd_colsum_bf16");
     return PD_OK;
 }

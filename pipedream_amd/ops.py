@@ -617,7 +617,8 @@ def colsum_bf16(x, acc=None):
     """fp32 column sums of a bf16 matrix; added to ``acc`` when given."""
     M, N = x.shape
     lib = _cabi.lib()
-    splits = min(256, max(1, M // 256))
+    # about two blocks per CU (a block covers 512 columns), at least 16 rows per split
+    splits = max(1, min(512 // -(-N // 512), M // 16, 1024))
     part = torch.empty((splits, N), dtype=torch.float32, device=x.device)
     lib.pd_colsum_bf16(_ptr(x), _ptr(part), M, N, x.stride(0), splits, _cabi.stream_ptr())
     if acc is None:
