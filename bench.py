@@ -214,12 +214,118 @@ def cpu_baseline(timed_steps=2):
             "sample": "%d steady-state steps at batch 64 after 1 warm-up step (%.1f s/step)" % (timed_steps, sec)}
 
 
+# ---- other configurations (not the default line): one stage each, same step definition ----------
+
+def _run_steps(step, steps, warmup):
+    """Throughput over `steps` un-instrumented steps, then a short instrumented pass for the per-kernel
+    figures (an event pair around each of the thousands of launches of these stages would slow the
+    timed region itself)."""
+    import torch
+    from pipedream_amd import ops
+    for _ in range(warmup):
+        step()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        step()
+    torch.cuda.synchronize()
+    elapsed = time.perf_counter() - t0
+    ops.kernel_timer = {}
+    for _ in range(min(steps, 4)):
+        step()
+    torch.cuda.synchronize()
+    timer, ops.kernel_timer = ops.kernel_timer, None
+    stats = {}
+    for name, recs in timer.items():
+        ms = sum(s.elapsed_time(e) for s, e, _ in recs)
+        stats[name] = {"launches": len(recs), "avg_us": round(1e3 * ms / len(recs), 1),
+                       "TFLOP/s": round(sum(w for _, _, w in recs) / (ms * 1e-3) / 1e12, 2)}
+    return elapsed, stats
+
+
+def gnmt_run(steps, warmup):
+    """Embedding (32320 x 1024) + 4 LSTM layers (hidden 1024, residuals), T = 50, batch 128, fp32,
+    AdamWithWeightStashing with stash depth 3 (2 forwards in flight)."""
+    import torch
+    from pipedream_amd import adam
+    from pipedream_amd.stages import gnmt
+    torch.manual_seed(0)
+    m = gnmt.Stage0(dropout=0.0).cuda()
+    opt = adam.AdamWithWeightStashing([m], list(m.parameters()), None, 1.0, 3, lr=1e-3, betas=(0.9, 0.999))
+    ids = torch.randint(0, 32320, (50, 128)).cuda()
+    dy = (torch.randn(50, 128, 1024) * 1e-2).cuda()
+    pend = [m(ids) for _ in range(2)]
+
+    def step():
+        pend.append(m(ids))
+        opt.zero_grad()
+        opt.load_old_params()
+        pend.pop(0).backward(dy)
+        opt.load_new_params()
+        opt.step()
+
+    elapsed, stats = _run_steps(step, steps, warmup)
+    return elapsed, stats, 128, "f32", ("GNMT-style stage: embedding 32320x1024 + 4 LSTM layers hidden 1024 with residuals, "
+                                         "seq 50, batch 128, fp32, Adam, stash depth 3")
+
+
+def transformer_run(steps, warmup):
+    """6 pre-LN transformer layers (hidden 1024, 16 heads, FFN 4096), micro-batch 8 x 512 tokens,
+    bf16 compute, fp32 master weights + Adam every 4 micro-batches, 2 weight versions.  One step =
+    one micro-batch forward + backward (+ the update on every 4th)."""
+    import torch
+    from pipedream_amd import adam
+    from pipedream_amd.stages import transformer
+    torch.manual_seed(0)
+    m = transformer.Stage0().cuda()
+    opt = adam.AdamWithWeightStashing([m], list(m.parameters()), None, 1.0, 2, update_interval=4, bf16_image=True,
+                                      lr=1e-3, betas=(0.9, 0.999))
+    x = torch.randn(8, 512, 1024).cuda()
+    dy = (torch.randn(8, 512, 1024) * 0.05).bfloat16().cuda()
+    pend = [m(x)]
+
+    def step():
+        pend.append(m(x))
+        opt.zero_grad()
+        opt.load_old_params()
+        pend.pop(0).backward(dy)
+        opt.load_new_params()
+        opt.step()
+
+    elapsed, stats = _run_steps(step, steps, warmup)
+    return elapsed, stats, 8, "bf16", ("PipeDream-2BW stage: 6 transformer layers (hidden 1024, 16 heads, FFN 4096, GELU, "
+                                        "pre-LN), seq 512, micro-batch 8, 4-micro-batch accumulation, 2 weight versions, "
+                                        "bf16 compute, fp32 master Adam")
+
+
+def secondary(args):
+    run, kernel, peak = {"gnmt": (gnmt_run, "gemm_f32", PEAK_FP32_MFMA_TFLOPS),
+                         "transformer": (transformer_run, "gemm_bf16", 2500.0)}[args.workload]
+    elapsed, stats, batch, dtype, desc = run(args.steps, args.warmup)
+    k = stats[kernel]
+    out = {
+        "metric": "samples/sec per stage (fwd+bwd+stashed update)", "value": batch * args.steps / elapsed,
+        "unit": "samples/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": 1e3 * elapsed / args.steps, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": dtype, "data": "synthetic", "config": {"workload": desc, "global_batch": batch,
+                                                        "parallelism": "1 stage on 1 GPU"},
+        "roofline": {"bound": "mfma", "achieved": k["TFLOP/s"], "peak": peak, "unit": "TFLOP/s",
+                     "frac": k["TFLOP/s"] / peak, "traffic": None, "kernel": kernel, "launches": k["launches"],
+                     "avg_us": k["avg_us"]},
+        "kernels": stats,
+    }
+    print(json.dumps(out))
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--workload", default="vgg16_front", choices=["vgg16_front", "gnmt", "transformer"],
+                    help="vgg16_front (default) is the headline configuration; the others print the same kind of "
+                         "line for the LSTM and transformer stages (no CPU baseline)")
     ap.add_argument("--pmc-probe", action="store_true",
                     help="run the counter-calibration copy and two benchmark steps, print no JSON")
     ap.add_argument("--traffic-bytes", type=float, default=None,
@@ -234,6 +340,9 @@ def main():
 
     if args.pmc_probe:
         pmc_probe()
+        return
+    if args.workload != "vgg16_front":
+        secondary(args)
         return
     elapsed, stats, _ = gpu_run(args.steps, args.warmup)
     conv = stats["conv3x3_fwd_kernel"]

@@ -87,13 +87,15 @@ def gemm(a, b, trans_a=False, trans_b=False, bias=None, relu=False, out=None, be
     if (splits > 1 or skinny) and N % 4 == 0 and ldc % 4 == 0 and out.data_ptr() % 16 == 0:
         # too few output tiles for 256 CUs: split k over more blocks, then one fused reduce + epilogue
         part = torch.empty((splits, M, N), dtype=torch.float32, device=a.device)
-        _cabi.lib().pd_gemm_splitk_f32(int(trans_a), int(trans_b), M, N, K, _ptr(a), lda, _ptr(b), ldb, _ptr(part),
-                                       splits, _cabi.stream_ptr())
+        with _timed("gemm_f32_splitk", 2.0 * M * N * K):
+            _cabi.lib().pd_gemm_splitk_f32(int(trans_a), int(trans_b), M, N, K, _ptr(a), lda, _ptr(b), ldb, _ptr(part),
+                                           splits, _cabi.stream_ptr())
         _cabi.lib().pd_splitk_reduce_f32(_ptr(part), splits, M, N, _ptr(bias), int(relu), float(beta), _ptr(out), ldc,
                                          _cabi.stream_ptr())
         return out
-    _cabi.lib().pd_gemm_f32(int(trans_a), int(trans_b), M, N, K, _ptr(a), lda, _ptr(b), ldb, float(beta),
-                            _ptr(out), ldc, _ptr(bias), int(relu), _cabi.stream_ptr())
+    with _timed("gemm_f32", 2.0 * M * N * K):
+        _cabi.lib().pd_gemm_f32(int(trans_a), int(trans_b), M, N, K, _ptr(a), lda, _ptr(b), ldb, float(beta),
+                                _ptr(out), ldc, _ptr(bias), int(relu), _cabi.stream_ptr())
     return out
 
 
@@ -128,8 +130,9 @@ def gemm_splitk(a, b, trans_a, trans_b, partials):
     _check(partials, "partials")
     lda = a.stride(0) if a.size(0) > 1 else a.size(1)
     ldb = b.stride(0) if b.size(0) > 1 else b.size(1)
-    _cabi.lib().pd_gemm_splitk_f32(int(trans_a), int(trans_b), M, N, K, _ptr(a), lda, _ptr(b), ldb, _ptr(partials),
-                                   partials.size(0), _cabi.stream_ptr())
+    with _timed("gemm_f32_splitk", 2.0 * M * N * K):
+        _cabi.lib().pd_gemm_splitk_f32(int(trans_a), int(trans_b), M, N, K, _ptr(a), lda, _ptr(b), ldb, _ptr(partials),
+                                       partials.size(0), _cabi.stream_ptr())
     return partials
 
 
@@ -496,19 +499,21 @@ def gemm_bf16(a, b, trans_a=False, trans_b=False, out=None, out_f32=False, alpha
             raise ValueError("gemm_bf16: residual shape")
     if bias is not None:
         _check(bias, "bias")
-    _cabi.lib().pd_gemm_bf16(int(trans_a), int(trans_b), M, N, K, _ptr(a), a.stride(0), _ptr(b), b.stride(0),
-                             _ptr(out), out.stride(0), int(out_f32), float(alpha), float(beta), _ptr(bias),
-                             _ptr(residual), residual.stride(0) if residual is not None else 0, 1, 1, None,
-                             _cabi.stream_ptr())
+    with _timed("gemm_bf16", 2.0 * M * N * K):
+        _cabi.lib().pd_gemm_bf16(int(trans_a), int(trans_b), M, N, K, _ptr(a), a.stride(0), _ptr(b), b.stride(0),
+                                 _ptr(out), out.stride(0), int(out_f32), float(alpha), float(beta), _ptr(bias),
+                                 _ptr(residual), residual.stride(0) if residual is not None else 0, 1, 1, None,
+                                 _cabi.stream_ptr())
     return out
 
 
 def _batched(ta, tb, M, N, K, A, a_off, lda, B, b_off, ldb, C, c_off, ldc, alpha, bo, bi, strides):
     arr = (ctypes.c_int64 * 6)(*strides)
     es = 2
-    _cabi.lib().pd_gemm_bf16(int(ta), int(tb), M, N, K, _vp(A.data_ptr() + a_off * es), lda,
-                             _vp(B.data_ptr() + b_off * es), ldb, _vp(C.data_ptr() + c_off * es), ldc, 0,
-                             float(alpha), 0.0, None, None, 0, bo, bi, arr, _cabi.stream_ptr())
+    with _timed("gemm_bf16_batched", 2.0 * M * N * K * bo * bi):
+        _cabi.lib().pd_gemm_bf16(int(ta), int(tb), M, N, K, _vp(A.data_ptr() + a_off * es), lda,
+                                 _vp(B.data_ptr() + b_off * es), ldb, _vp(C.data_ptr() + c_off * es), ldc, 0,
+                                 float(alpha), 0.0, None, None, 0, bo, bi, arr, _cabi.stream_ptr())
 
 
 def attention_forward(qkv, batch, seq, heads):
