@@ -223,6 +223,16 @@ __global__ __launch_bounds__(CONV_THREADS, 2) void conv3x3_fwd_kernel(const Conv
 #pragma unroll
                     for (int j = 0; j < 2; ++j)
                         acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(fa[i][s], fb[j][s], acc[i][j], 0, 0, 0);
+            // Instruction order for the scheduler: the four fragment reads of the NEXT step are spread
+            // over the first twelve MFMAs of this one (3 MFMAs, 1 LDS read, ...), so their latency is
+            // covered by this wave's own MFMAs instead of stalling it at the top of every step.
+            if (step == 0) __builtin_amdgcn_sched_group_barrier(0x100, 4, 0);
+#pragma unroll
+            for (int q = 0; q < 4; ++q) {
+                __builtin_amdgcn_sched_group_barrier(0x008, 3, 0);
+                __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+            }
+            __builtin_amdgcn_sched_group_barrier(0x008, 4, 0);
         }
     }
 
@@ -253,7 +263,8 @@ __global__ __launch_bounds__(CONV_THREADS, 2) void conv3x3_fwd_kernel(const Conv
             const int q = id / (BN / 4), k4 = (id % (BN / 4)) * 4;
             const int gy = y0 + q / TW, gx = x0 + q % TW;
             if (gy < a.H && gx < a.W && k0 + k4 < a.K)
-                *(float4_t*)(yn + ((size_t)gy * a.W + gx) * a.K + k0 + k4) = *(const float4_t*)(lds + q * OP + k4);
+                __builtin_nontemporal_store(*(const float4_t*)(lds + q * OP + k4),
+                                            (float4_t*)(yn + ((size_t)gy * a.W + gx) * a.K + k0 + k4));
         }
     } else {
 #pragma unroll
