@@ -571,6 +571,160 @@ __global__ __launch_bounds__(CONV_THREADS, 2) void conv3x3_wgrad_kernel(const Wg
     }
 }
 
+// Weight gradient, pipelined variant (C and K multiples of 4, 16-byte aligned tensors): one block
+// of 8 waves per CU.  A tile's global loads (dY, the ReLU mask, the X halo: 14 128-bit loads per
+// thread) stay in registers while the previous tile is multiplied, and both LDS tiles are
+// double-buffered: the registers are written to the other buffer in the middle of the multiply
+// phase, leaving one barrier per tile and no phase in which the matrix pipe waits for memory.
+// The zero fill and the mask are applied when the registers go to LDS.  Waves 0-3 reduce the
+// first half of a tile's pixels, waves 4-7 the second half (two waves per SIMD: a single wave
+// cannot issue MFMAs back to back at the full rate), each into its own partial sum.
+constexpr int WGP_THREADS = 512;
+
+template <int TH, int TW, bool MASKED>
+struct WgradStage {
+    static constexpr int PIX = TH * TW, HW_ = TW + 2, HALO = (TH + 2) * (TW + 2), CS = 64;
+    static constexpr int DY_ITERS = (PIX * (CS / 4) + WGP_THREADS - 1) / WGP_THREADS;
+    static constexpr int X_ITERS = (HALO * (CS / 4) + WGP_THREADS - 1) / WGP_THREADS;
+    float4_t rdy[DY_ITERS], rm[MASKED ? DY_ITERS : 1], rx[X_ITERS];
+    uint32_t ok_dy, ok_x;
+
+    __device__ __forceinline__ void load(const WgradArgs& a, int tile, int k0, int c0, int tid) {
+        int b = tile;
+        const int tx = b % a.tiles_x;
+        b /= a.tiles_x;
+        const int ty = b % a.tiles_y;
+        const int n = b / a.tiles_y;
+        const int y0 = ty * TH, x0 = tx * TW;
+        const float* xn = a.x + (size_t)n * a.H * a.W * a.C;
+        const float* dyn = a.dy + (size_t)n * a.H * a.W * a.K;
+        const float* mn = MASKED ? a.mask + (size_t)n * a.H * a.W * a.K : dyn;
+        ok_dy = ok_x = 0;
+#pragma unroll
+        for (int it = 0; it < DY_ITERS; ++it) {
+            const int id = tid + it * WGP_THREADS;
+            const int p = id / (CS / 4), q4 = (id % (CS / 4)) * 4;
+            const int gy = y0 + p / TW, gx = x0 + p % TW;
+            const int k = k0 + q4;
+            const bool ok = id < PIX * (CS / 4) && gy < a.H && gx < a.W && k < a.K;
+            const size_t off = ok ? ((size_t)gy * a.W + gx) * a.K + k : 0;
+            rdy[it] = *(const float4_t*)(dyn + off);
+            if (MASKED) rm[it] = *(const float4_t*)(mn + off);
+            ok_dy |= (ok ? 1u : 0u) << it;
+        }
+#pragma unroll
+        for (int it = 0; it < X_ITERS; ++it) {
+            const int id = tid + it * WGP_THREADS;
+            const int p = id / (CS / 4), q4 = (id % (CS / 4)) * 4;
+            const int gy = y0 + p / HW_ - 1, gx = x0 + p % HW_ - 1;
+            const int c = c0 + q4;
+            const bool ok = id < HALO * (CS / 4) && gy >= 0 && gy < a.H && gx >= 0 && gx < a.W && c < a.C;
+            const size_t off = ok ? ((size_t)gy * a.W + gx) * a.C + c : 0;     // a select, not a branch
+            rx[it] = *(const float4_t*)(xn + off);
+            ok_x |= (ok ? 1u : 0u) << it;
+        }
+    }
+
+    __device__ __forceinline__ void store(float* dy_tile, float* x_tile, int tid) const {
+        const float4_t zero = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int it = 0; it < DY_ITERS; ++it) {
+            const int id = tid + it * WGP_THREADS;
+            float4_t v = rdy[it];
+            if (MASKED)
+#pragma unroll
+                for (int j = 0; j < 4; ++j) v[j] = rm[it][j] > 0.f ? v[j] : 0.f;
+            if (id < PIX * (CS / 4))
+                *(float4_t*)(dy_tile + (id / (CS / 4)) * CS + (id % (CS / 4)) * 4) = ((ok_dy >> it) & 1u) ? v : zero;
+        }
+#pragma unroll
+        for (int it = 0; it < X_ITERS; ++it) {
+            const int id = tid + it * WGP_THREADS;
+            if (id < HALO * (CS / 4))
+                *(float4_t*)(x_tile + (id / (CS / 4)) * CS + (id % (CS / 4)) * 4) = ((ok_x >> it) & 1u) ? rx[it] : zero;
+        }
+    }
+};
+
+template <int TH, int TW, bool MASKED>
+__global__ __launch_bounds__(WGP_THREADS, 1) void conv3x3_wgrad_pipe_kernel(const WgradArgs a) {
+    using Stage = WgradStage<TH, TW, MASKED>;
+    constexpr int PIX = Stage::PIX, HW_ = Stage::HW_, HALO = Stage::HALO, CS = Stage::CS;
+    constexpr int BUF = PIX * CS + HALO * CS;       // floats per buffer: dY tile, then X halo tile
+    __shared__ __attribute__((aligned(16))) float lds[2 * BUF];
+
+    const int tid = threadIdx.x;
+    const int wave = tid / 64, lane = tid % 64;
+    const int idx = lane % 32, h = lane / 32;
+    const int half = wave / 4;                     // which half of the tile's pixel pairs
+    const int kt = (wave % 4) / 2, ct = wave % 2;
+    const int k0 = blockIdx.y * 64, c0 = blockIdx.z * 64;
+    const bool wave_active = (c0 + ct * 32) < a.C && (k0 + kt * 32) < a.K;
+
+    float16_t acc[9];
+#pragma unroll
+    for (int t = 0; t < 9; ++t)
+#pragma unroll
+        for (int e = 0; e < 16; ++e) acc[t][e] = 0.f;
+    float bsum = 0.f;
+
+    // reduction over pixel pairs [pp0, pp1) of the tile in `buf`: lane-half h takes pixel 2*pp + h
+    auto multiply = [&](const float* buf, int pp0, int pp1) {
+        const float* dy_tile = buf + kt * 32 + idx;
+        const float* x_tile = buf + PIX * CS + ct * 32 + idx;
+#pragma unroll 2
+        for (int pp = pp0; pp < pp1; ++pp) {
+            const int p = 2 * pp + h;
+            const float av = dy_tile[p * CS];
+            bsum += av;
+            const int xb = ((p / TW) * HW_ + (p % TW)) * CS;
+#pragma unroll
+            for (int t = 0; t < 9; ++t) {
+                const float bv = x_tile[xb + ((t / 3) * HW_ + (t % 3)) * CS];
+                acc[t] = __builtin_amdgcn_mfma_f32_32x32x2f32(av, bv, acc[t], 0, 0, 0);
+            }
+        }
+    };
+
+    Stage st;
+    int tile = blockIdx.x;
+    int cur = 0;
+    if (tile < a.n_tiles) {
+        st.load(a, tile, k0, c0, tid);
+        st.store(lds, lds + PIX * CS, tid);
+    }
+    __syncthreads();
+    for (; tile < a.n_tiles; tile += gridDim.x) {
+        const int next = tile + gridDim.x;
+        const float* buf = lds + cur * BUF;
+        float* other = lds + (cur ^ 1) * BUF;
+        if (next < a.n_tiles) st.load(a, next, k0, c0, tid);
+        const int pp0 = half * (PIX / 4);
+        if (wave_active) multiply(buf, pp0, pp0 + PIX / 8);
+        if (next < a.n_tiles) st.store(other, other + PIX * CS, tid);
+        if (wave_active) multiply(buf, pp0 + PIX / 8, pp0 + PIX / 4);
+        __syncthreads();    // `buf` may be overwritten, `other` is complete
+        cur ^= 1;
+    }
+
+    float* pw = a.part_w + (size_t)(blockIdx.x * 2 + half) * a.K * 9 * a.C;
+    const int c = c0 + ct * 32 + idx;
+    if (wave_active && c < a.C) {
+#pragma unroll
+        for (int t = 0; t < 9; ++t)
+#pragma unroll
+            for (int e = 0; e < 16; ++e) {
+                const int k = k0 + kt * 32 + 8 * (e / 4) + 4 * h + (e % 4);
+                if (k < a.K) pw[((size_t)k * 9 + t) * a.C + c] = acc[t][e];
+            }
+    }
+    if (a.part_b && blockIdx.z == 0 && ct == 0) {
+        const float other = __shfl_xor(bsum, 32, 64);
+        const int k = k0 + kt * 32 + idx;
+        if (h == 0 && k < a.K) a.part_b[(size_t)(blockIdx.x * 2 + half) * a.K + k] = bsum + other;
+    }
+}
+
 // Weight gradient for very few input channels (9*C <= 32, i.e. the first VGG layer with
 // C = 3): all 9*C (tap, channel) pairs fit the 32 columns of ONE MFMA tile, so a pixel pair
 // costs 2 MFMAs (two 32-row out-channel tiles) instead of 18.  The kernel is then bound by
@@ -745,9 +899,14 @@ TileShape pick_tile(int H, int W) {
 constexpr int WGRAD_TH = 8, WGRAD_TW = 16;
 constexpr int WGRAD_MAX_BLOCKS = 512;
 
-int wgrad_blocks(int N, int H, int W) {
+// Number of pixel-range blocks (= partial sums to reduce): with the (K/64) x (C/64) channel blocks
+// about WGRAD_MAX_BLOCKS workgroups in total, i.e. two rounds of one block per CU.
+int wgrad_blocks(int N, int H, int W, int C, int K) {
     const long tiles = (long)N * ((H + WGRAD_TH - 1) / WGRAD_TH) * ((W + WGRAD_TW - 1) / WGRAD_TW);
-    return (int)(tiles < WGRAD_MAX_BLOCKS ? tiles : WGRAD_MAX_BLOCKS);
+    const long pairs = 9 * C <= 32 ? (K + 63) / 64 : (long)((K + 63) / 64) * ((C + 63) / 64);
+    long nb = WGRAD_MAX_BLOCKS / pairs;
+    if (nb < 1) nb = 1;
+    return (int)(tiles < nb ? tiles : nb);
 }
 
 int check_dims(const char* who, int N, int H, int W, int C, int K) {
@@ -825,7 +984,8 @@ extern "C" int pd_conv3x3_wgrad_workspace_bytes(int N, int H, int W, int C, int 
     if (rc != PD_OK) return rc;
     PD_REQUIRE(bytes != nullptr, PD_EINVAL, "pd_conv3x3_wgrad_workspace_bytes: NULL pointer");
     // the few-channel kernel writes one partial per wave (4 per block)
-    const uint64_t nb = (uint64_t)wgrad_blocks(N, H, W) * (9 * C <= 32 ? 4 : 1);
+    // partial sums per pixel-range block: 4 in the few-channel kernel (one per wave), 2 in the pipelined one
+    const uint64_t nb = (uint64_t)wgrad_blocks(N, H, W, C, K) * (9 * C <= 32 ? 4 : 2);
     *bytes = nb * ((uint64_t)K * 9 * C + (uint64_t)K) * sizeof(float);
     return PD_OK;
 }
@@ -848,8 +1008,9 @@ extern "C" int pd_conv3x3_wgrad_nhwc_f32(const float* x, const float* dy, const 
     a.tiles_y = (H + WGRAD_TH - 1) / WGRAD_TH;
     a.n_tiles = N * a.tiles_x * a.tiles_y;
     const bool small_c = 9 * C <= 32;
-    const int nblk = wgrad_blocks(N, H, W);
-    const int nb = nblk * (small_c ? 4 : 1);     // number of partial sums
+    const int nblk = wgrad_blocks(N, H, W, C, K);
+    const bool vec = (C % 4 == 0) && pd_aligned(x, 16) && (K % 4 == 0) && pd_aligned(dy, 16) && (!relu_out || pd_aligned(relu_out, 16));
+    const int nb = nblk * (small_c ? 4 : (vec ? 2 : 1));     // number of partial sums
     a.part_w = (float*)workspace;
     a.part_b = dbias ? a.part_w + (size_t)nb * K * 9 * C : nullptr;
     a.c_vec = (C % 4 == 0) && pd_aligned(x, 16);
@@ -860,7 +1021,9 @@ extern "C" int pd_conv3x3_wgrad_nhwc_f32(const float* x, const float* dy, const 
         conv3x3_wgrad_smallc_kernel<WGRAD_TH, WGRAD_TW><<<grid, CONV_THREADS, 0, s>>>(a);
     } else {
         dim3 grid(nblk, (K + 63) / 64, (C + 63) / 64);
-        conv3x3_wgrad_kernel<WGRAD_TH, WGRAD_TW><<<grid, CONV_THREADS, 0, s>>>(a);
+        if (a.c_vec && a.k_vec && relu_out) conv3x3_wgrad_pipe_kernel<WGRAD_TH, WGRAD_TW, true><<<grid, WGP_THREADS, 0, s>>>(a);
+        else if (a.c_vec && a.k_vec) conv3x3_wgrad_pipe_kernel<WGRAD_TH, WGRAD_TW, false><<<grid, WGP_THREADS, 0, s>>>(a);
+        else conv3x3_wgrad_kernel<WGRAD_TH, WGRAD_TW><<<grid, CONV_THREADS, 0, s>>>(a);
     }
     PD_CHECK_LAUNCH("pd_conv3x3_wgrad_nhwc_f32");
     const int nw = K * 9 * C;
