@@ -699,9 +699,12 @@ extern "C" int pd_gemm_bf16(int trans_a, int trans_b, int M, int N, int K, const
     const long tiles128 = (long)((M + 127) / 128) * ((N + 127) / 128) * batch;
     // direct-to-LDS kernel: whole ring rounds of k, and per-lane byte offsets that fit 32 bits
     const bool dma_ok = K % (DK * NS) == 0 && (long long)256 * (lda > ldb ? lda : ldb) * 2 < (1ll << 31);
-    if (dma_ok && tiles256 >= 256) return launch_gemm_bf16_dma<256, 256>(trans_a, trans_b, g, batch, s);
+    const bool wide = M >= 256 && N >= 256;       // a 256 x 256 tile is mostly inside the matrix
+    if (dma_ok && wide && tiles256 >= 256) return launch_gemm_bf16_dma<256, 256>(trans_a, trans_b, g, batch, s);
     if (dma_ok && M >= 128 && N >= 128) return launch_gemm_bf16_dma<128, 128>(trans_a, trans_b, g, batch, s);
-    if (tiles256 >= 192) return launch_gemm_bf16<256, 256, 2, 4>(trans_a, trans_b, g, batch, s);
-    if (tiles128 >= 128) return launch_gemm_bf16<128, 128, 2, 2>(trans_a, trans_b, g, batch, s);
+    if (wide && tiles256 >= 192) return launch_gemm_bf16<256, 256, 2, 4>(trans_a, trans_b, g, batch, s);
+    // narrow outputs (attention: N = head dimension): tall tiles, all waves stacked along M
+    if (N <= 64 && M >= 256) return launch_gemm_bf16<256, 64, 4, 1>(trans_a, trans_b, g, batch, s);
+    if (M >= 128 && N >= 128 && tiles128 >= 128) return launch_gemm_bf16<128, 128, 2, 2>(trans_a, trans_b, g, batch, s);
     return launch_gemm_bf16<64, 64, 2, 2>(trans_a, trans_b, g, batch, s);
 }
