@@ -256,6 +256,14 @@ int pd_layernorm_bwd_bf16(const uint16_t* dy, const uint16_t* x, const float* ga
                           const float* rstd, uint16_t* dx, float* part_dgamma, float* part_dbeta,
                           int M, int H, void* stream);
 
+/* Fused attention forward of one transformer layer: qkv [batch*seq][3H] (Q | K | V, the heads
+ * contiguous inside each, H = heads*head_dim) -> P = softmax(Q K^T / sqrt(head_dim)) written as
+ * probs [batch][heads][seq][seq] (the backward pass reads it) and ctx = P V as [batch*seq][H].
+ * The scores stay in registers (fp32).  Supported shapes: pd_attention_fwd_supported() != 0
+ * (head_dim 64, seq 128 / 256 / 512); other shapes use pd_gemm_bf16 + pd_softmax_fwd_bf16. */
+int pd_attention_fwd_supported(int seq, int head_dim);
+int pd_attention_fwd_bf16(const uint16_t* qkv, uint16_t* ctx, uint16_t* probs, int batch, int seq, int heads,
+                          int head_dim, void* stream);
 /* Row softmax (row length multiple of 8, <= 2048) and its backward dx = y*(dy - sum(dy*y)). */
 int pd_softmax_fwd_bf16(const uint16_t* x, uint16_t* y, int64_t rows, int n, void* stream);
 int pd_softmax_bwd_bf16(const uint16_t* y, const uint16_t* dy, uint16_t* dx, int64_t rows, int n, void* stream);

@@ -528,6 +528,11 @@ def attention_forward(qkv, batch, seq, heads):
     dev = qkv.device
     probs = torch.empty((batch, heads, seq, seq), dtype=BF16, device=dev)
     ctx = torch.empty((batch * seq, H), dtype=BF16, device=dev)
+    if _cabi.lib().pd_attention_fwd_supported(seq, d):
+        with _timed("attention_fwd", 4.0 * batch * heads * seq * seq * d):
+            _cabi.lib().pd_attention_fwd_bf16(_ptr(qkv), _ptr(ctx), _ptr(probs), batch, seq, heads, d,
+                                              _cabi.stream_ptr())
+        return ctx, probs
     scale = 1.0 / (d ** 0.5)
     ld = 3 * H
     # scores = scale * Q K^T

@@ -105,6 +105,26 @@ def test_gemm_bf16_large_tile_epilogues():
     assert torch.equal(shifted, ops.gemm_bf16(a, b, trans_b=True))
 
 
+@pytest.mark.parametrize("batch,seq,heads", [(2, 128, 3), (1, 256, 2), (2, 512, 4)])
+def test_fused_attention_forward(batch, seq, heads):
+    """The fused kernel (head dimension 64) against attention evaluated in fp64 from the same bf16
+    q, k, v; probabilities and context are bf16, so one bf16 ulp (2^-8 relative) per element plus
+    the rounding of P inside the second product bounds the difference."""
+    from pipedream_amd import ops
+    d, H = 64, 64 * heads
+    g = torch.Generator().manual_seed(seq + heads)
+    qkv = (torch.randn(batch * seq, 3 * H, generator=g) * 1.5).to(BF)
+    ctx, probs = ops.attention_forward(qkv.cuda(), batch, seq, heads)
+    q, k, v = [t.reshape(batch, seq, heads, d).transpose(1, 2).double() for t in qkv.split(H, dim=-1)]
+    p = torch.softmax(q @ k.transpose(-1, -2) / math.sqrt(d), dim=-1)
+    want = (p @ v).transpose(1, 2).reshape(batch * seq, H)
+    assert tuple(probs.shape) == (batch, heads, seq, seq)
+    torch.testing.assert_close(probs.float().cpu().double(), p, rtol=2 ** -7, atol=1e-6)
+    assert float((probs.float().sum(-1) - 1).abs().max()) < 2e-2
+    assert _rel(ctx, want.float()) < 4e-3
+    torch.testing.assert_close(ctx.float().cpu().double(), want, rtol=2e-2, atol=2e-2)
+
+
 def test_layernorm_softmax_gelu_vs_torch():
     from pipedream_amd import ops
     g = torch.Generator().manual_seed(1)
