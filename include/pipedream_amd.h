@@ -264,6 +264,12 @@ int pd_layernorm_bwd_bf16(const uint16_t* dy, const uint16_t* x, const float* ga
 int pd_attention_fwd_supported(int seq, int head_dim);
 int pd_attention_fwd_bf16(const uint16_t* qkv, uint16_t* ctx, uint16_t* probs, int batch, int seq, int heads,
                           int head_dim, void* stream);
+/* Query side of its backward pass (same shape support): with dctx = dL/dctx and the ctx and probs
+ * of the forward pass, ds [batch][heads][seq][seq] = P o (dctx V^T - delta) / sqrt(head_dim),
+ * delta_q = sum_d dctx[q][d] ctx[q][d], and the Q third of dqkv [batch*seq][3H] = ds K.  The K and
+ * V thirds are the caller's two products over queries: dK = ds^T Q, dV = P^T dctx (pd_gemm_bf16). */
+int pd_attention_bwd_bf16(const uint16_t* qkv, const uint16_t* probs, const uint16_t* ctx, const uint16_t* dctx,
+                          uint16_t* ds, uint16_t* dqkv, int batch, int seq, int heads, int head_dim, void* stream);
 /* Row softmax (row length multiple of 8, <= 2048) and its backward dx = y*(dy - sum(dy*y)). */
 int pd_softmax_fwd_bf16(const uint16_t* x, uint16_t* y, int64_t rows, int n, void* stream);
 int pd_softmax_bwd_bf16(const uint16_t* y, const uint16_t* dy, uint16_t* dx, int64_t rows, int n, void* stream);

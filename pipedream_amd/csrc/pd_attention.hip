@@ -150,6 +150,97 @@ __global__ __launch_bounds__(AT_THREADS) void attention_fwd_kernel(const uint16_
             u16x4{at_f2bf(oacc[dt][0]), at_f2bf(oacc[dt][1]), at_f2bf(oacc[dt][2]), at_f2bf(oacc[dt][3])};
 }
 
+// Backward, query side: dP = dO V^T, dS = scale * P o (dP - delta) with delta_q = sum_d dO[q][d] O[q][d]
+// (= sum_k dP[q][k] P[q][k]), dQ = dS K.  Same block shape and the same transposed formulation as
+// the forward kernel with the roles V -> A operand of the first product, K -> transposed operand of
+// the second: dP^T = V dO^T lands in the layout of the stored P, and the packed dS^T accumulators are
+// the B operand of dQ^T = K^T dS^T.  dS (bf16, scale folded in) is written out for the two products
+// that reduce over queries (dK = dS^T Q, dV = P^T dO), which stay strided-batched GEMMs.
+template <int S>
+__global__ __launch_bounds__(AT_THREADS) void attention_bwd_kernel(const uint16_t* __restrict__ qkv,
+                                                                  const uint16_t* __restrict__ probs,
+                                                                  const uint16_t* __restrict__ ctx,
+                                                                  const uint16_t* __restrict__ dctx,
+                                                                  uint16_t* __restrict__ ds_out,
+                                                                  uint16_t* __restrict__ dqkv, int heads, float scale) {
+    constexpr int NT = S / 16;
+    __shared__ __attribute__((aligned(16))) uint16_t v_lds[S * AT_KP];     // fragment reads along d
+    __shared__ __attribute__((aligned(16))) uint16_t k_lds[S * AT_VP];     // transposing reads
+
+    const int tid = threadIdx.x, wave = tid / 64, lane = tid % 64;
+    const int li = lane % 16, g = lane / 16;
+    const int bh = blockIdx.y, b = bh / heads, h = bh % heads;
+    const int H = heads * AT_D, ld = 3 * H;
+    const uint16_t* base = qkv + (size_t)b * S * ld + h * AT_D;
+
+    for (int id = tid; id < S * (AT_D / 8); id += AT_THREADS) {
+        const int row = id / (AT_D / 8), c8 = (id % (AT_D / 8)) * 8;
+        const u16x8 kv = *(const u16x8*)(base + (size_t)row * ld + H + c8);
+        const u16x8 vv = *(const u16x8*)(base + (size_t)row * ld + 2 * H + c8);
+        *(u16x8*)(k_lds + row * AT_VP + c8) = kv;
+        *(u16x8*)(v_lds + row * AT_KP + c8) = vv;
+    }
+
+    const int q = blockIdx.x * AT_QB + wave * 16 + li;
+    const size_t orow = ((size_t)b * S + q) * H + h * AT_D;
+    bf16x8 dof[2];
+    float delta = 0.f;
+#pragma unroll
+    for (int s = 0; s < 2; ++s) {
+        const u16x8 d8 = *(const u16x8*)(dctx + orow + 32 * s + 8 * g);
+        const u16x8 o8 = *(const u16x8*)(ctx + orow + 32 * s + 8 * g);
+        dof[s] = __builtin_bit_cast(bf16x8, d8);
+#pragma unroll
+        for (int j = 0; j < 8; ++j)
+            delta += __uint_as_float((uint32_t)d8[j] << 16) * __uint_as_float((uint32_t)o8[j] << 16);
+    }
+    delta += __shfl_xor(delta, 16, 64);
+    delta += __shfl_xor(delta, 32, 64);
+    __syncthreads();
+
+    const uint16_t* prow = probs + ((size_t)bh * S + q) * S + 4 * g;
+    uint16_t* dsrow = ds_out + ((size_t)bh * S + q) * S + 4 * g;
+    float4_t qacc[4];
+#pragma unroll
+    for (int dt = 0; dt < 4; ++dt) qacc[dt] = float4_t{0.f, 0.f, 0.f, 0.f};
+    typedef __attribute__((address_space(3))) short4_t* lds_ptr;
+#pragma unroll 2
+    for (int u = 0; u < NT / 2; ++u) {
+        u16x8 dsp;
+#pragma unroll
+        for (int half = 0; half < 2; ++half) {
+            const int t = 2 * u + half;
+            float4_t acc = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+            for (int s = 0; s < 2; ++s) {
+                const bf16x8 vf = __builtin_bit_cast(bf16x8, *(const u16x8*)(v_lds + (16 * t + li) * AT_KP + 32 * s + 8 * g));
+                acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf, dof[s], acc, 0, 0, 0);
+            }
+            const u16x4 p4 = *(const u16x4*)(prow + 16 * t);
+#pragma unroll
+            for (int e = 0; e < 4; ++e)
+                dsp[4 * half + e] = at_f2bf(scale * __uint_as_float((uint32_t)p4[e] << 16) * (acc[e] - delta));
+        }
+        *(u16x4*)(dsrow + 32 * u) = u16x4{dsp[0], dsp[1], dsp[2], dsp[3]};
+        *(u16x4*)(dsrow + 32 * u + 16) = u16x4{dsp[4], dsp[5], dsp[6], dsp[7]};
+        const bf16x8 dsf = __builtin_bit_cast(bf16x8, dsp);
+        const uint16_t* kb = k_lds + (32 * u + 4 * g + li / 4) * AT_VP + 4 * (li % 4);
+#pragma unroll
+        for (int dt = 0; dt < 4; ++dt) {
+            const short4_t lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_ptr)(kb + 16 * dt));
+            const short4_t hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_ptr)(kb + 16 * AT_VP + 16 * dt));
+            const short8_t k8 = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+            qacc[dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, k8), dsf, qacc[dt], 0, 0, 0);
+        }
+    }
+
+    uint16_t* qrow = dqkv + ((size_t)b * S + q) * ld + h * AT_D + 4 * g;     // the Q third of dqkv
+#pragma unroll
+    for (int dt = 0; dt < 4; ++dt)
+        *(u16x4*)(qrow + 16 * dt) =
+            u16x4{at_f2bf(qacc[dt][0]), at_f2bf(qacc[dt][1]), at_f2bf(qacc[dt][2]), at_f2bf(qacc[dt][3])};
+}
+
 }  // namespace
 
 extern "C" int pd_attention_fwd_supported(int seq, int head_dim) {
@@ -172,5 +263,26 @@ extern "C" int pd_attention_fwd_bf16(const uint16_t* qkv, uint16_t* ctx, uint16_
     else if (seq == 256) attention_fwd_kernel<256><<<grid, AT_THREADS, 0, s>>>(qkv, ctx, probs, heads, scale_log2e);
     else attention_fwd_kernel<128><<<grid, AT_THREADS, 0, s>>>(qkv, ctx, probs, heads, scale_log2e);
     PD_CHECK_LAUNCH("pd_attention_fwd_bf16");
+    return PD_OK;
+}
+
+extern "C" int pd_attention_bwd_bf16(const uint16_t* qkv, const uint16_t* probs, const uint16_t* ctx,
+                                     const uint16_t* dctx, uint16_t* ds, uint16_t* dqkv, int batch, int seq, int heads,
+                                     int head_dim, void* stream) {
+    PD_REQUIRE(batch > 0 && heads > 0, PD_ESHAPE, "pd_attention_bwd_bf16: batch and heads must be positive");
+    PD_REQUIRE(pd_attention_fwd_supported(seq, head_dim), PD_ESHAPE,
+               "pd_attention_bwd_bf16: needs head_dim 64 and seq 128, 256 or 512 (got %d, %d)", head_dim, seq);
+    PD_REQUIRE(qkv && probs && ctx && dctx && ds && dqkv, PD_EINVAL, "pd_attention_bwd_bf16: NULL pointer");
+    PD_REQUIRE(pd_aligned(qkv, 16) && pd_aligned(ctx, 16) && pd_aligned(dctx, 16) && pd_aligned(probs, 8) &&
+                   pd_aligned(ds, 8) && pd_aligned(dqkv, 8),
+               PD_EINVAL, "pd_attention_bwd_bf16: qkv, ctx, dctx must be 16-byte, probs, ds, dqkv 8-byte aligned");
+    PD_REQUIRE((long long)batch * heads <= 65535, PD_ESHAPE, "pd_attention_bwd_bf16: too many (batch, head) pairs");
+    const float scale = 1.0f / sqrtf((float)head_dim);
+    const dim3 grid(seq / AT_QB, batch * heads);
+    hipStream_t s = (hipStream_t)stream;
+    if (seq == 512) attention_bwd_kernel<512><<<grid, AT_THREADS, 0, s>>>(qkv, probs, ctx, dctx, ds, dqkv, heads, scale);
+    else if (seq == 256) attention_bwd_kernel<256><<<grid, AT_THREADS, 0, s>>>(qkv, probs, ctx, dctx, ds, dqkv, heads, scale);
+    else attention_bwd_kernel<128><<<grid, AT_THREADS, 0, s>>>(qkv, probs, ctx, dctx, ds, dqkv, heads, scale);
+    PD_CHECK_LAUNCH("pd_attention_bwd_bf16");
     return PD_OK;
 }

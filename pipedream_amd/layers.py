@@ -391,7 +391,7 @@ class _TransformerLayerFn(torch.autograd.Function):
         dx2 = ops.add_bf16(layernorm_backward(dh2, x2, ln2_w, ln2_b, mean2, rstd2), dy2)
         # x2 = o(attn(qkv(LN1(x)))) + x
         datt = linear_backward(dx2, att, o_w, o_b)
-        dqkv = ops.attention_backward(datt, qkv, probs, B, S, heads)
+        dqkv = ops.attention_backward(datt, qkv, probs, B, S, heads, ctx=att)
         dh1 = linear_backward(dqkv, h1, qkv_w, qkv_b)
         dx = ops.add_bf16(layernorm_backward(dh1, x2d, ln1_w, ln1_b, mean1, rstd1), dx2)
         return (dx.view(B, S, H), None, None) + (None,) * 12

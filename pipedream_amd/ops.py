@@ -545,8 +545,8 @@ def attention_forward(qkv, batch, seq, heads):
     return ctx, probs
 
 
-def attention_backward(dctx, qkv, probs, batch, seq, heads):
-    """Gradient with respect to qkv."""
+def attention_backward(dctx, qkv, probs, batch, seq, heads, ctx=None):
+    """Gradient with respect to qkv.  `ctx` (the forward output) selects the fused query-side kernel."""
     _mat_bf16(dctx, "dctx")
     H = qkv.size(1) // 3
     d = H // heads
@@ -557,6 +557,19 @@ def attention_backward(dctx, qkv, probs, batch, seq, heads):
     dqkv = torch.empty_like(qkv)
     dP = torch.empty_like(probs)
     sP = (heads * seq * seq, seq * seq)
+    if ctx is not None and _cabi.lib().pd_attention_fwd_supported(seq, d):
+        _mat_bf16(ctx, "ctx")
+        if tuple(ctx.shape) != (batch * seq, H) or not ctx.is_contiguous():
+            raise ValueError("attention_backward: ctx must be a contiguous [batch*seq, H] matrix")
+        # dS (scaled) and dQ in one kernel; dV = P^T dctx and dK = dS^T Q reduce over queries
+        with _timed("attention_bwd", 4.0 * batch * heads * seq * seq * d):
+            _cabi.lib().pd_attention_bwd_bf16(_ptr(qkv), _ptr(probs), _ptr(ctx), _ptr(dctx), _ptr(dP), _ptr(dqkv),
+                                              batch, seq, heads, d, _cabi.stream_ptr())
+        _batched(1, 0, seq, d, seq, probs, 0, seq, dctx, 0, H, dqkv, 2 * H, ld, 1.0, batch, heads,
+                 sP + (seq * H, d, seq * ld, d))
+        _batched(1, 0, seq, d, seq, dP, 0, seq, qkv, 0, ld, dqkv, H, ld, 1.0, batch, heads,
+                 sP + (seq * ld, d, seq * ld, d))
+        return dqkv
     # dP = dctx V^T
     _batched(0, 1, seq, seq, d, dctx, 0, H, qkv, 2 * H, ld, dP, 0, seq, 1.0, batch, heads,
              (seq * H, d, seq * ld, d) + sP)

@@ -125,6 +125,29 @@ def test_fused_attention_forward(batch, seq, heads):
     torch.testing.assert_close(ctx.float().cpu().double(), want, rtol=2e-2, atol=2e-2)
 
 
+@pytest.mark.parametrize("batch,seq,heads", [(2, 128, 3), (1, 512, 2)])
+def test_fused_attention_backward(batch, seq, heads):
+    """dqkv of the fused path (query-side kernel + the two products over queries) against autograd
+    in fp64 through softmax(q k^T / sqrt(d)) v on the same bf16 inputs, and against the unfused
+    HIP path (batched products + softmax backward)."""
+    from pipedream_amd import ops
+    d, H = 64, 64 * heads
+    g = torch.Generator().manual_seed(7 * seq + heads)
+    qkv = (torch.randn(batch * seq, 3 * H, generator=g)).to(BF)
+    dctx = (torch.randn(batch * seq, H, generator=g) * 0.1).to(BF)
+    ref = qkv.double().requires_grad_()
+    q, k, v = [t.reshape(batch, seq, heads, d).transpose(1, 2) for t in ref.split(H, dim=-1)]
+    out = (torch.softmax(q @ k.transpose(-1, -2) / math.sqrt(d), dim=-1) @ v).transpose(1, 2).reshape(batch * seq, H)
+    out.backward(dctx.double())
+    ctx, probs = ops.attention_forward(qkv.cuda(), batch, seq, heads)
+    fused = ops.attention_backward(dctx.cuda(), qkv.cuda(), probs, batch, seq, heads, ctx=ctx)
+    plain = ops.attention_backward(dctx.cuda(), qkv.cuda(), probs, batch, seq, heads)
+    for name, lo in (("dq", 0), ("dk", H), ("dv", 2 * H)):
+        want = ref.grad[:, lo:lo + H].float()
+        assert _rel(fused[:, lo:lo + H], want) < 2e-2, (name, _rel(fused[:, lo:lo + H], want))
+        assert _rel(fused[:, lo:lo + H], plain[:, lo:lo + H].float().cpu()) < 2e-2, name
+
+
 def test_layernorm_softmax_gelu_vs_torch():
     from pipedream_amd import ops
     g = torch.Generator().manual_seed(1)
