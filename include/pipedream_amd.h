@@ -256,20 +256,22 @@ int pd_layernorm_bwd_bf16(const uint16_t* dy, const uint16_t* x, const float* ga
                           const float* rstd, uint16_t* dx, float* part_dgamma, float* part_dbeta,
                           int M, int H, void* stream);
 
-/* Fused attention forward of one transformer layer: qkv [batch*seq][3H] (Q | K | V, the heads
- * contiguous inside each, H = heads*head_dim) -> P = softmax(Q K^T / sqrt(head_dim)) written as
- * probs [batch][heads][seq][seq] (the backward pass reads it) and ctx = P V as [batch*seq][H].
- * The scores stay in registers (fp32).  Supported shapes: pd_attention_fwd_supported() != 0
- * (head_dim 64, seq 128 / 256 / 512); other shapes use pd_gemm_bf16 + pd_softmax_fwd_bf16. */
+/* Fused attention of one transformer layer.  qkv is [batch*seq][3H] (Q | K | V, the heads contiguous
+ * inside each, H = heads*head_dim).  Forward: ctx [batch*seq][H] = softmax(Q K^T / sqrt(head_dim)) V; the
+ * scores stay in registers (fp32).  Optional outputs (NULL to skip): probs [batch][heads][seq][seq], the
+ * bf16 probabilities, and lse2 [batch][heads][seq] (fp32), log2 of the softmax denominator in the scaled
+ * base-2 domain, from which the backward pass recomputes the probabilities:
+ * P[q][k] = 2^(s_qk log2(e) / sqrt(head_dim) - lse2[q]).
+ * Supported shapes: pd_attention_fwd_supported() != 0 (head_dim 64, seq 128 / 256 / 512); other shapes
+ * use pd_gemm_bf16 + pd_softmax_fwd_bf16 / pd_softmax_bwd_bf16. */
 int pd_attention_fwd_supported(int seq, int head_dim);
-int pd_attention_fwd_bf16(const uint16_t* qkv, uint16_t* ctx, uint16_t* probs, int batch, int seq, int heads,
-                          int head_dim, void* stream);
-/* Query side of its backward pass (same shape support): with dctx = dL/dctx and the ctx and probs
- * of the forward pass, ds [batch][heads][seq][seq] = P o (dctx V^T - delta) / sqrt(head_dim),
- * delta_q = sum_d dctx[q][d] ctx[q][d], and the Q third of dqkv [batch*seq][3H] = ds K.  The K and
- * V thirds are the caller's two products over queries: dK = ds^T Q, dV = P^T dctx (pd_gemm_bf16). */
-int pd_attention_bwd_bf16(const uint16_t* qkv, const uint16_t* probs, const uint16_t* ctx, const uint16_t* dctx,
-                          uint16_t* ds, uint16_t* dqkv, int batch, int seq, int heads, int head_dim, void* stream);
+int pd_attention_fwd_bf16(const uint16_t* qkv, uint16_t* ctx, uint16_t* probs, float* lse2, int batch, int seq,
+                          int heads, int head_dim, void* stream);
+/* Backward: dqkv [batch*seq][3H] from dctx = dL/dctx, the forward's ctx and lse2.  Two kernels: the
+ * query side (dQ; also writes delta [batch][heads][seq] = sum_d dctx*ctx, workspace owned by the
+ * caller) and the key side (dK, dV).  Neither reads or writes a [seq][seq] tensor. */
+int pd_attention_bwd_bf16(const uint16_t* qkv, const uint16_t* ctx, const uint16_t* dctx, const float* lse2,
+                          float* delta, uint16_t* dqkv, int batch, int seq, int heads, int head_dim, void* stream);
 /* Row softmax (row length multiple of 8, <= 2048) and its backward dx = y*(dy - sum(dy*y)). */
 int pd_softmax_fwd_bf16(const uint16_t* x, uint16_t* y, int64_t rows, int n, void* stream);
 int pd_softmax_bwd_bf16(const uint16_t* y, const uint16_t* dy, uint16_t* dx, int64_t rows, int n, void* stream);

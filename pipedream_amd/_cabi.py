@@ -88,7 +88,7 @@ SIGNATURES = {
     "pd_layernorm_bwd_partials": (_i, [_i], False),
     "pd_layernorm_bwd_bf16": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _vp], True),
     "pd_attention_fwd_supported": (_i, [_i, _i], False),
-    "pd_attention_fwd_bf16": (_i, [_vp, _vp, _vp, _i, _i, _i, _i, _vp], True),
+    "pd_attention_fwd_bf16": (_i, [_vp, _vp, _vp, _vp, _i, _i, _i, _i, _vp], True),
     "pd_attention_bwd_bf16": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _vp], True),
     "pd_softmax_fwd_bf16": (_i, [_vp, _vp, _i64, _i, _vp], True),
     "pd_softmax_bwd_bf16": (_i, [_vp, _vp, _vp, _i64, _i, _vp], True),

@@ -349,7 +349,7 @@ class _TransformerLayerFn(torch.autograd.Function):
         bw = ops.bf16_weight
         h1, mean1, rstd1 = ops.layernorm_forward(x2d, ln1_w, ln1_b, eps)
         qkv = ops.gemm_bf16(h1, bw(qkv_w), trans_b=True, bias=qkv_b)
-        att, probs = ops.attention_forward(qkv, B, S, heads)
+        att, att_aux = ops.attention_forward(qkv, B, S, heads)
         x2 = ops.gemm_bf16(att, bw(o_w), trans_b=True, bias=o_b, residual=x2d)
         h2, mean2, rstd2 = ops.layernorm_forward(x2, ln2_w, ln2_b, eps)
         f = ops.gemm_bf16(h2, bw(fc1_w), trans_b=True, bias=fc1_b)
@@ -357,13 +357,13 @@ class _TransformerLayerFn(torch.autograd.Function):
         y = ops.gemm_bf16(g, bw(fc2_w), trans_b=True, bias=fc2_b, residual=x2)
         ctx.dims = (B, S, H, heads)
         ctx.params = (ln1_w, ln1_b, qkv_w, qkv_b, o_w, o_b, ln2_w, ln2_b, fc1_w, fc1_b, fc2_w, fc2_b)
-        ctx.save_for_backward(x2d, h1, mean1, rstd1, qkv, probs, att, x2, h2, mean2, rstd2, f, g)
+        ctx.save_for_backward(x2d, h1, mean1, rstd1, qkv, att_aux, att, x2, h2, mean2, rstd2, f, g)
         return y.view(B, S, H)
 
     @staticmethod
     def backward(ctx, dy):
         B, S, H, heads = ctx.dims
-        x2d, h1, mean1, rstd1, qkv, probs, att, x2, h2, mean2, rstd2, f, g = ctx.saved_tensors
+        x2d, h1, mean1, rstd1, qkv, att_aux, att, x2, h2, mean2, rstd2, f, g = ctx.saved_tensors
         ln1_w, ln1_b, qkv_w, qkv_b, o_w, o_b, ln2_w, ln2_b, fc1_w, fc1_b, fc2_w, fc2_b = ctx.params
         bw = ops.bf16_weight
         dy2 = dy.contiguous().view(B * S, H)
@@ -391,7 +391,7 @@ class _TransformerLayerFn(torch.autograd.Function):
         dx2 = ops.add_bf16(layernorm_backward(dh2, x2, ln2_w, ln2_b, mean2, rstd2), dy2)
         # x2 = o(attn(qkv(LN1(x)))) + x
         datt = linear_backward(dx2, att, o_w, o_b)
-        dqkv = ops.attention_backward(datt, qkv, probs, B, S, heads, ctx=att)
+        dqkv = ops.attention_backward(datt, qkv, att_aux, B, S, heads, ctx=att)
         dh1 = linear_backward(dqkv, h1, qkv_w, qkv_b)
         dx = ops.add_bf16(layernorm_backward(dh1, x2d, ln1_w, ln1_b, mean1, rstd1), dx2)
         return (dx.view(B, S, H), None, None) + (None,) * 12

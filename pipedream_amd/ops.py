@@ -516,9 +516,11 @@ def _batched(ta, tb, M, N, K, A, a_off, lda, B, b_off, ldb, C, c_off, ldc, alpha
                                  float(alpha), 0.0, None, None, 0, bo, bi, arr, _cabi.stream_ptr())
 
 
-def attention_forward(qkv, batch, seq, heads):
-    """qkv: [batch*seq, 3H] bf16 (Q | K | V, heads contiguous inside each).  Returns
-    (ctx [batch*seq, H], probs [batch, heads, seq, seq])."""
+def attention_forward(qkv, batch, seq, heads, need_probs=False):
+    """qkv: [batch*seq, 3H] bf16 (Q | K | V, heads contiguous inside each).  Returns (ctx [batch*seq, H],
+    aux) where aux is what attention_backward needs: on the fused path (head dimension 64, seq 128 / 256 /
+    512) the fp32 vector lse2 [batch, heads, seq], otherwise -- or with need_probs -- the bf16
+    probabilities [batch, heads, seq, seq]."""
     _mat_bf16(qkv, "qkv")
     H = qkv.size(1) // 3
     d = H // heads
@@ -526,13 +528,15 @@ def attention_forward(qkv, batch, seq, heads):
         raise ValueError("attention: qkv shape %s does not fit batch %d seq %d heads %d"
                          % (tuple(qkv.shape), batch, seq, heads))
     dev = qkv.device
-    probs = torch.empty((batch, heads, seq, seq), dtype=BF16, device=dev)
     ctx = torch.empty((batch * seq, H), dtype=BF16, device=dev)
     if _cabi.lib().pd_attention_fwd_supported(seq, d):
+        probs = torch.empty((batch, heads, seq, seq), dtype=BF16, device=dev) if need_probs else None
+        lse2 = None if need_probs else torch.empty((batch, heads, seq), dtype=torch.float32, device=dev)
         with _timed("attention_fwd", 4.0 * batch * heads * seq * seq * d):
-            _cabi.lib().pd_attention_fwd_bf16(_ptr(qkv), _ptr(ctx), _ptr(probs), batch, seq, heads, d,
+            _cabi.lib().pd_attention_fwd_bf16(_ptr(qkv), _ptr(ctx), _ptr(probs), _ptr(lse2), batch, seq, heads, d,
                                               _cabi.stream_ptr())
-        return ctx, probs
+        return ctx, (probs if need_probs else lse2)
+    probs = torch.empty((batch, heads, seq, seq), dtype=BF16, device=dev)
     scale = 1.0 / (d ** 0.5)
     ld = 3 * H
     # scores = scale * Q K^T
@@ -545,8 +549,9 @@ def attention_forward(qkv, batch, seq, heads):
     return ctx, probs
 
 
-def attention_backward(dctx, qkv, probs, batch, seq, heads, ctx=None):
-    """Gradient with respect to qkv.  `ctx` (the forward output) selects the fused query-side kernel."""
+def attention_backward(dctx, qkv, aux, batch, seq, heads, ctx=None):
+    """Gradient with respect to qkv; `aux` is the second result of attention_forward (lse2 needs `ctx`,
+    the forward output, as well)."""
     _mat_bf16(dctx, "dctx")
     H = qkv.size(1) // 3
     d = H // heads
@@ -555,21 +560,20 @@ def attention_backward(dctx, qkv, probs, batch, seq, heads, ctx=None):
     ld = 3 * H
     scale = 1.0 / (d ** 0.5)
     dqkv = torch.empty_like(qkv)
+    if aux.dtype == torch.float32:
+        if ctx is None:
+            raise ValueError("attention_backward: the fused path needs ctx")
+        _mat_bf16(ctx, "ctx")
+        if tuple(ctx.shape) != (batch * seq, H) or not ctx.is_contiguous() or tuple(aux.shape) != (batch, heads, seq):
+            raise ValueError("attention_backward: ctx must be a contiguous [batch*seq, H] matrix, lse2 [batch, heads, seq]")
+        delta = torch.empty_like(aux)
+        with _timed("attention_bwd", 10.0 * batch * heads * seq * seq * d):
+            _cabi.lib().pd_attention_bwd_bf16(_ptr(qkv), _ptr(ctx), _ptr(dctx), _ptr(aux), _ptr(delta), _ptr(dqkv),
+                                              batch, seq, heads, d, _cabi.stream_ptr())
+        return dqkv
+    probs = aux
     dP = torch.empty_like(probs)
     sP = (heads * seq * seq, seq * seq)
-    if ctx is not None and _cabi.lib().pd_attention_fwd_supported(seq, d):
-        _mat_bf16(ctx, "ctx")
-        if tuple(ctx.shape) != (batch * seq, H) or not ctx.is_contiguous():
-            raise ValueError("attention_backward: ctx must be a contiguous [batch*seq, H] matrix")
-        # dS (scaled) and dQ in one kernel; dV = P^T dctx and dK = dS^T Q reduce over queries
-        with _timed("attention_bwd", 4.0 * batch * heads * seq * seq * d):
-            _cabi.lib().pd_attention_bwd_bf16(_ptr(qkv), _ptr(probs), _ptr(ctx), _ptr(dctx), _ptr(dP), _ptr(dqkv),
-                                              batch, seq, heads, d, _cabi.stream_ptr())
-        _batched(1, 0, seq, d, seq, probs, 0, seq, dctx, 0, H, dqkv, 2 * H, ld, 1.0, batch, heads,
-                 sP + (seq * H, d, seq * ld, d))
-        _batched(1, 0, seq, d, seq, dP, 0, seq, qkv, 0, ld, dqkv, H, ld, 1.0, batch, heads,
-                 sP + (seq * ld, d, seq * ld, d))
-        return dqkv
     # dP = dctx V^T
     _batched(0, 1, seq, seq, d, dctx, 0, H, qkv, 2 * H, ld, dP, 0, seq, 1.0, batch, heads,
              (seq * H, d, seq * ld, d) + sP)

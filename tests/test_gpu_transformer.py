@@ -114,7 +114,9 @@ def test_fused_attention_forward(batch, seq, heads):
     d, H = 64, 64 * heads
     g = torch.Generator().manual_seed(seq + heads)
     qkv = (torch.randn(batch * seq, 3 * H, generator=g) * 1.5).to(BF)
-    ctx, probs = ops.attention_forward(qkv.cuda(), batch, seq, heads)
+    ctx, probs = ops.attention_forward(qkv.cuda(), batch, seq, heads, need_probs=True)
+    ctx2, lse2 = ops.attention_forward(qkv.cuda(), batch, seq, heads)
+    assert torch.equal(ctx, ctx2) and lse2.dtype == torch.float32 and tuple(lse2.shape) == (batch, heads, seq)
     q, k, v = [t.reshape(batch, seq, heads, d).transpose(1, 2).double() for t in qkv.split(H, dim=-1)]
     p = torch.softmax(q @ k.transpose(-1, -2) / math.sqrt(d), dim=-1)
     want = (p @ v).transpose(1, 2).reshape(batch * seq, H)
@@ -123,11 +125,14 @@ def test_fused_attention_forward(batch, seq, heads):
     assert float((probs.float().sum(-1) - 1).abs().max()) < 2e-2
     assert _rel(ctx, want.float()) < 4e-3
     torch.testing.assert_close(ctx.float().cpu().double(), want, rtol=2e-2, atol=2e-2)
+    # lse2 = log2 sum_k exp(s_k / sqrt(d)): the probabilities are recomputed from it in the backward pass
+    want_lse = torch.logsumexp(q @ k.transpose(-1, -2) / math.sqrt(d), dim=-1) / math.log(2.0)
+    torch.testing.assert_close(lse2.cpu().double(), want_lse, rtol=1e-5, atol=1e-4)
 
 
 @pytest.mark.parametrize("batch,seq,heads", [(2, 128, 3), (1, 512, 2)])
 def test_fused_attention_backward(batch, seq, heads):
-    """dqkv of the fused path (query-side kernel + the two products over queries) against autograd
+    """dqkv of the fused path (query-side and key-side kernels, probabilities recomputed) against autograd
     in fp64 through softmax(q k^T / sqrt(d)) v on the same bf16 inputs, and against the unfused
     HIP path (batched products + softmax backward)."""
     from pipedream_amd import ops
@@ -139,8 +144,9 @@ def test_fused_attention_backward(batch, seq, heads):
     q, k, v = [t.reshape(batch, seq, heads, d).transpose(1, 2) for t in ref.split(H, dim=-1)]
     out = (torch.softmax(q @ k.transpose(-1, -2) / math.sqrt(d), dim=-1) @ v).transpose(1, 2).reshape(batch * seq, H)
     out.backward(dctx.double())
-    ctx, probs = ops.attention_forward(qkv.cuda(), batch, seq, heads)
-    fused = ops.attention_backward(dctx.cuda(), qkv.cuda(), probs, batch, seq, heads, ctx=ctx)
+    ctx, lse2 = ops.attention_forward(qkv.cuda(), batch, seq, heads)
+    _, probs = ops.attention_forward(qkv.cuda(), batch, seq, heads, need_probs=True)
+    fused = ops.attention_backward(dctx.cuda(), qkv.cuda(), lse2, batch, seq, heads, ctx=ctx)
     plain = ops.attention_backward(dctx.cuda(), qkv.cuda(), probs, batch, seq, heads)
     for name, lo in (("dq", 0), ("dk", H), ("dv", 2 * H)):
         want = ref.grad[:, lo:lo + H].float()
