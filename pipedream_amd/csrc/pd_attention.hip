@@ -46,20 +46,24 @@ constexpr int AT_QB = 128;             // queries (keys) per block
 constexpr int AT_P = AT_D + 8;         // LDS row pitch (bf16)
 constexpr float AT_LOG2E = 1.44269504088896340736f;
 
-__device__ __forceinline__ uint16_t at_f2bf(float f) {
-    uint32_t u = __float_as_uint(f);
-    if ((u & 0x7fffffffu) > 0x7f800000u) return (uint16_t)((u >> 16) | 0x0040u);
-    u += 0x7fffu + ((u >> 16) & 1u);
-    return (uint16_t)(u >> 16);
-}
+__device__ __forceinline__ uint16_t at_f2bf(float f) { return pd_f2bf(f); }
 __device__ __forceinline__ float at_bf2f(uint16_t h) { return __uint_as_float((uint32_t)h << 16); }
 
 // rows [0, S) x 64 columns of a [.][ld] bf16 matrix -> LDS with pitch AT_P
 template <int S>
 __device__ __forceinline__ void at_stage(uint16_t* lds, const uint16_t* __restrict__ g, int ld, int tid) {
-    for (int id = tid; id < S * (AT_D / 8); id += AT_THREADS) {
-        const int row = id / (AT_D / 8), c8 = (id % (AT_D / 8)) * 8;
-        *(u16x8*)(lds + row * AT_P + c8) = *(const u16x8*)(g + (size_t)row * ld + c8);
+    constexpr int ITERS = S * (AT_D / 8) / AT_THREADS;
+    static_assert(S * (AT_D / 8) % AT_THREADS == 0, "rows divide over the block");
+    u16x8 r[ITERS];
+#pragma unroll
+    for (int it = 0; it < ITERS; ++it) {         // all loads in flight before the first LDS store
+        const int id = tid + it * AT_THREADS;
+        r[it] = *(const u16x8*)(g + (size_t)(id / (AT_D / 8)) * ld + (id % (AT_D / 8)) * 8);
+    }
+#pragma unroll
+    for (int it = 0; it < ITERS; ++it) {
+        const int id = tid + it * AT_THREADS;
+        *(u16x8*)(lds + (id / (AT_D / 8)) * AT_P + (id % (AT_D / 8)) * 8) = r[it];
     }
 }
 

@@ -64,12 +64,7 @@ struct GemmBf16Args {
     int vec_store;              // C (and residual) can be written with 16-byte vectors
 };
 
-__device__ __forceinline__ uint16_t f2bf(float f) {
-    uint32_t u = __float_as_uint(f);
-    if ((u & 0x7fffffffu) > 0x7f800000u) return (uint16_t)((u >> 16) | 0x0040u);
-    u += 0x7fffu + ((u >> 16) & 1u);
-    return (uint16_t)(u >> 16);
-}
+__device__ __forceinline__ uint16_t f2bf(float f) { return pd_f2bf(f); }
 __device__ __forceinline__ float bf2f(uint16_t h) { return __uint_as_float((uint32_t)h << 16); }
 
 // Epilogue of one wave: its (32*TM) x (32*TN) accumulator tile -> C.

@@ -44,3 +44,9 @@ static inline bool pd_aligned(const void* p, size_t a) { return ((uintptr_t)p & 
 
 // 64-lane wavefronts on gfx950.
 #define PD_WAVE 64
+
+#if defined(__HIPCC__)
+// fp32 -> bf16, round to nearest even: the gfx950 conversion instruction (v_cvt_pk_bf16_f32; the
+// compiler pairs two adjacent conversions into one instruction).
+__device__ __forceinline__ uint16_t pd_f2bf(float f) { return __builtin_bit_cast(uint16_t, (__bf16)f); }
+#endif

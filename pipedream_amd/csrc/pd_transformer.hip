@@ -19,12 +19,7 @@ constexpr int TR_THREADS = 256;
 constexpr int MAX_VEC = 4;   // rows up to 64 lanes * 8 elements * MAX_VEC = 2048 elements
 
 __device__ __forceinline__ float bf2f(uint16_t h) { return __uint_as_float((uint32_t)h << 16); }
-__device__ __forceinline__ uint16_t f2bf(float f) {
-    uint32_t u = __float_as_uint(f);
-    if ((u & 0x7fffffffu) > 0x7f800000u) return (uint16_t)((u >> 16) | 0x0040u);
-    u += 0x7fffu + ((u >> 16) & 1u);
-    return (uint16_t)(u >> 16);
-}
+__device__ __forceinline__ uint16_t f2bf(float f) { return pd_f2bf(f); }
 __device__ __forceinline__ float wave_sum(float v) {
 #pragma unroll
     for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o, 64);
