@@ -81,12 +81,14 @@ class Linear(torch.nn.Module):
 # --------------------------------------------------------------------------------------
 class _Conv3x3Fn(torch.autograd.Function):
     @staticmethod
-    def forward(ctx, x, weight, bias, relu):
+    def forward(ctx, x, weight, bias, relu, grad_premasked=False):
         x = ops.to_nhwc(x)
         y = ops.conv3x3_forward(x, weight, bias, relu)
         ctx.relu = relu
         ctx.has_bias = bias is not None
-        ctx.save_for_backward(x, weight, y if relu else None)
+        # with grad_premasked the consumer's backward (a pooling layer with relu=True) has already
+        # zeroed dy wherever y == 0, so the gradient kernels need not read y at all
+        ctx.save_for_backward(x, weight, y if (relu and not grad_premasked) else None)
         return y
 
     @staticmethod
@@ -100,16 +102,22 @@ class _Conv3x3Fn(torch.autograd.Function):
             dx = ops.conv3x3_input_grad(dy, weight, relu_out=y)
         if ctx.needs_input_grad[1] or (ctx.has_bias and ctx.needs_input_grad[2]):
             dw, db = ops.conv3x3_weight_grad(x, dy, with_bias=ctx.has_bias, relu_out=y)
-        return dx, dw, db, None
+        return dx, dw, db, None, None
 
 
 class Conv2d(torch.nn.Module):
     """``torch.nn.Conv2d(in, out, kernel_size=3, stride=1, padding=1)`` (the only
     convolution shape in the reference's VGG16 stages), optionally with the following
     ReLU fused into the epilogue.  The weight has torch's logical shape [out, in, 3, 3]
-    and channels_last memory order; activations are kept in NHWC order."""
+    and channels_last memory order; activations are kept in NHWC order.
 
-    def __init__(self, in_channels, out_channels, kernel_size=3, stride=1, padding=1, bias=True, relu=False):
+    ``grad_premasked=True`` (only with ``relu=True``) declares that the layer's output goes only to a
+    layer whose backward already drops the gradient where this output is zero -- ``MaxPool2d(relu=True)``,
+    which is the identity on an already rectified input in the forward pass -- so the ReLU backward need
+    not be applied (and the output not be read) again here.  Results are identical either way."""
+
+    def __init__(self, in_channels, out_channels, kernel_size=3, stride=1, padding=1, bias=True, relu=False,
+                 grad_premasked=False):
         super(Conv2d, self).__init__()
         norm = lambda v: tuple(v) if isinstance(v, (tuple, list)) else (v, v)
         if norm(kernel_size) != (3, 3) or norm(stride) != (1, 1) or norm(padding) != (1, 1):
@@ -117,6 +125,9 @@ class Conv2d(torch.nn.Module):
         self.in_channels = in_channels
         self.out_channels = out_channels
         self.relu = relu
+        if grad_premasked and not relu:
+            raise ValueError("grad_premasked only makes sense with relu=True")
+        self.grad_premasked = grad_premasked
         w = torch.empty(out_channels, in_channels, 3, 3)
         torch.nn.init.kaiming_uniform_(w, a=math.sqrt(5))
         self.weight = torch.nn.Parameter(w.contiguous(memory_format=torch.channels_last))
@@ -127,7 +138,7 @@ class Conv2d(torch.nn.Module):
             self.bias = None
 
     def forward(self, x):
-        return _Conv3x3Fn.apply(x, self.weight, self.bias, self.relu)
+        return _Conv3x3Fn.apply(x, self.weight, self.bias, self.relu, self.grad_premasked)
 
     def extra_repr(self):
         return "{}, {}, kernel_size=(3, 3), stride=(1, 1), padding=(1, 1), relu={}".format(

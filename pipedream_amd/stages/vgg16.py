@@ -40,11 +40,14 @@ class FrontStage(torch.nn.Module):
     def __init__(self):
         super(FrontStage, self).__init__()
         self.layer2 = layers.Conv2d(3, 64, relu=True)
-        self.layer4 = layers.Conv2d(64, 64, relu=True)
-        self.layer6 = layers.MaxPool2d(2, 2)
+        # a pooling layer with relu=True is the identity on the rectified output of the convolution
+        # before it and masks the gradient in its backward kernel, so that convolution's gradient
+        # kernels read no mask (grad_premasked)
+        self.layer4 = layers.Conv2d(64, 64, relu=True, grad_premasked=True)
+        self.layer6 = layers.MaxPool2d(2, 2, relu=True)
         self.layer7 = layers.Conv2d(64, 128, relu=True)
-        self.layer9 = layers.Conv2d(128, 128, relu=True)
-        self.layer11 = layers.MaxPool2d(2, 2)
+        self.layer9 = layers.Conv2d(128, 128, relu=True, grad_premasked=True)
+        self.layer11 = layers.MaxPool2d(2, 2, relu=True)
         _initialize_weights(self)
 
     def forward(self, input0):
@@ -70,8 +73,8 @@ class Stage1(torch.nn.Module):
         super(Stage1, self).__init__()
         self.layer2 = layers.MaxPool2d(2, 2, relu=True)    # layer1 ReLU + layer2 MaxPool
         self.layer3 = layers.Conv2d(64, 128, relu=True)    # + layer4
-        self.layer5 = layers.Conv2d(128, 128, relu=True)   # + layer6
-        self.layer7 = layers.MaxPool2d(2, 2)
+        self.layer5 = layers.Conv2d(128, 128, relu=True, grad_premasked=True)   # + layer6; masked by layer7
+        self.layer7 = layers.MaxPool2d(2, 2, relu=True)
         self.layer8 = layers.Conv2d(128, 256, relu=True)   # + layer9
         _initialize_weights(self)
 
@@ -85,8 +88,8 @@ class Stage2(torch.nn.Module):
     def __init__(self):
         super(Stage2, self).__init__()
         self.layer1 = layers.Conv2d(256, 256, relu=True)   # + layer2
-        self.layer3 = layers.Conv2d(256, 256, relu=True)   # + layer4
-        self.layer5 = layers.MaxPool2d(2, 2)
+        self.layer3 = layers.Conv2d(256, 256, relu=True, grad_premasked=True)   # + layer4; masked by layer5
+        self.layer5 = layers.MaxPool2d(2, 2, relu=True)
         self.layer6 = layers.Conv2d(256, 512, relu=True)   # + layer7
         self.layer8 = layers.Conv2d(512, 512, relu=True)   # + layer9
         self.layer10 = layers.Conv2d(512, 512, relu=True)  # + layer11
@@ -104,8 +107,8 @@ class Stage3(torch.nn.Module):
         self.layer1 = layers.MaxPool2d(2, 2)
         self.layer2 = layers.Conv2d(512, 512, relu=True)   # + layer3
         self.layer4 = layers.Conv2d(512, 512, relu=True)   # + layer5
-        self.layer6 = layers.Conv2d(512, 512, relu=True)   # + layer7
-        self.layer8 = layers.MaxPool2d(2, 2)
+        self.layer6 = layers.Conv2d(512, 512, relu=True, grad_premasked=True)   # + layer7; masked by layer8
+        self.layer8 = layers.MaxPool2d(2, 2, relu=True)
         self.flatten = layers.Flatten()
         self.layer11 = layers.Linear(25088, 4096, relu=True)   # + layer12
         self.layer13 = layers.Dropout(p=dropout)
