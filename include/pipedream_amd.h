@@ -189,8 +189,13 @@ int pd_conv3x3_fwd_nhwc_f32(const float* x, const float* w, const float* bias, f
 int pd_conv3x3_filter_rot180_f32(const float* w, float* out, int K, int C, void* stream);
 /* Input gradient dx[N,H,W,C] = conv3x3(dy[N,H,W,K], w_rot[C][3][3][K]).  If relu_out is not
  * NULL it is the forward output of the fused conv+ReLU layer and dy is taken as 0 where
- * relu_out <= 0 (the ReLU backward applied while the tile is loaded). */
-int pd_conv3x3_dgrad_nhwc_f32(const float* dy, const float* w_rot, const float* relu_out, float* dx,
+ * relu_out <= 0 (the ReLU backward applied while the tile is loaded).  If x_rectified is not
+ * NULL it is this layer's own input [N,H,W,C], itself the output of a ReLU, and dx is written
+ * as 0 where x_rectified <= 0: the ReLU backward of the PRODUCING layer applied in this
+ * kernel's epilogue, so that layer's gradient kernels need no mask (torch.nn.ReLU(inplace=True)
+ * between two convolutions, vgg16/gpus=4_straight/stage0.py:13-15). */
+int pd_conv3x3_dgrad_nhwc_f32(const float* dy, const float* w_rot, const float* relu_out,
+                              const float* x_rectified, float* dx,
                               int N, int H, int W, int K, int C, void* stream);
 /* Weight and (optional, dbias may be NULL) bias gradient of the same convolution:
  * dw[k][r][s][c] = sum_{n,y,x} dy[n,y,x,k] * x[n,y+r-1,x+s-1,c].  Deterministic two-pass

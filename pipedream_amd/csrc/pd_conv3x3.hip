@@ -43,6 +43,8 @@ struct ConvArgs {
     const float* bias;  // [K] or null
     const float* mask;  // [N,H,W,C] or null: x is taken as 0 where mask <= 0 (fused ReLU backward)
     float* y;           // [N,H,W,K]
+    const float* out_mask;  // [N,H,W,K] or null: y is written as 0 where out_mask <= 0 (the ReLU
+                            // backward of the layer that produced this convolution's input)
     int N, H, W, C, K;
     int relu;
     int tiles_x, tiles_y;
@@ -241,6 +243,21 @@ __global__ __launch_bounds__(CONV_THREADS, 2) void conv3x3_fwd_kernel(const Conv
     //      covers whole 256-byte pixel rows of the NHWC output -------------------------------
     float* yn = a.y + (size_t)n * a.H * a.W * a.K;
     if (a.y_vec) {
+        // the output mask (if any) is fetched before the transpose, so its latency is covered by
+        // the LDS traffic and the barriers below
+        constexpr int NV = 256 * (BN / 4) / CONV_THREADS;
+        float4_t mk[NV];
+        if (a.out_mask) {
+            const float* mn = a.out_mask + (size_t)n * a.H * a.W * a.K;
+#pragma unroll
+            for (int it = 0; it < NV; ++it) {
+                const int id = tid + it * CONV_THREADS;
+                const int q = id / (BN / 4), k4 = (id % (BN / 4)) * 4;
+                const int gy = y0 + q / TW, gx = x0 + q % TW;
+                if (gy < a.H && gx < a.W && k0 + k4 < a.K)
+                    mk[it] = __builtin_nontemporal_load((const float4_t*)(mn + ((size_t)gy * a.W + gx) * a.K + k0 + k4));
+            }
+        }
         __syncthreads();  // all waves are done reading the operand tiles
 #pragma unroll
         for (int j = 0; j < 2; ++j) {
@@ -258,13 +275,18 @@ __global__ __launch_bounds__(CONV_THREADS, 2) void conv3x3_fwd_kernel(const Conv
         }
         __syncthreads();
 #pragma unroll
-        for (int it = 0; it < 256 * (BN / 4) / CONV_THREADS; ++it) {
+        for (int it = 0; it < NV; ++it) {
             const int id = tid + it * CONV_THREADS;
             const int q = id / (BN / 4), k4 = (id % (BN / 4)) * 4;
             const int gy = y0 + q / TW, gx = x0 + q % TW;
-            if (gy < a.H && gx < a.W && k0 + k4 < a.K)
-                __builtin_nontemporal_store(*(const float4_t*)(lds + q * OP + k4),
-                                            (float4_t*)(yn + ((size_t)gy * a.W + gx) * a.K + k0 + k4));
+            if (gy < a.H && gx < a.W && k0 + k4 < a.K) {
+                float4_t v = *(const float4_t*)(lds + q * OP + k4);
+                if (a.out_mask) {
+#pragma unroll
+                    for (int c = 0; c < 4; ++c) v[c] = mk[it][c] > 0.f ? v[c] : 0.f;
+                }
+                __builtin_nontemporal_store(v, (float4_t*)(yn + ((size_t)gy * a.W + gx) * a.K + k0 + k4));
+            }
         }
     } else {
 #pragma unroll
@@ -279,9 +301,11 @@ __global__ __launch_bounds__(CONV_THREADS, 2) void conv3x3_fwd_kernel(const Conv
                     const int q = (wave * 2 + i) * 32 + 8 * (e / 4) + 4 * h + (e % 4);
                     const int gy = y0 + q / TW, gx = x0 + q % TW;
                     if (gy < a.H && gx < a.W) {
+                        const size_t o = ((size_t)gy * a.W + gx) * a.K + k;
                         float v = acc[i][j][e] + bv;
                         if (a.relu) v = v > 0.f ? v : 0.f;
-                        yn[((size_t)gy * a.W + gx) * a.K + k] = v;
+                        if (a.out_mask && !(a.out_mask[(size_t)n * a.H * a.W * a.K + o] > 0.f)) v = 0.f;
+                        yn[o] = v;
                     }
                 }
         }
@@ -917,17 +941,18 @@ int check_dims(const char* who, int N, int H, int W, int C, int K) {
 
 }  // namespace
 
-static int conv3x3_fwd_launch(const float* x, const float* w, const float* bias, const float* mask, float* y, int N,
-                              int H, int W, int C, int K, int relu, void* stream) {
+static int conv3x3_fwd_launch(const float* x, const float* w, const float* bias, const float* mask,
+                              const float* out_mask, float* y, int N, int H, int W, int C, int K, int relu,
+                              void* stream) {
     int rc = check_dims("pd_conv3x3_fwd_nhwc_f32", N, H, W, C, K);
     if (rc != PD_OK) return rc;
     PD_REQUIRE(x && w && y, PD_EINVAL, "pd_conv3x3_fwd_nhwc_f32: NULL pointer");
     ConvArgs a;
-    a.x = x; a.w = w; a.bias = bias; a.mask = mask; a.y = y;
+    a.x = x; a.w = w; a.bias = bias; a.mask = mask; a.y = y; a.out_mask = out_mask;
     a.N = N; a.H = H; a.W = W; a.C = C; a.K = K;
     a.relu = relu != 0;
     a.c_vec = (C % 4 == 0) && pd_aligned(x, 16) && pd_aligned(w, 16) && (!mask || pd_aligned(mask, 16));
-    a.y_vec = (K % 4 == 0) && pd_aligned(y, 16);
+    a.y_vec = (K % 4 == 0) && pd_aligned(y, 16) && (!out_mask || pd_aligned(out_mask, 16));
     const TileShape t = pick_tile(H, W);
     a.tiles_x = (W + t.tw - 1) / t.tw;
     a.tiles_y = (H + t.th - 1) / t.th;
@@ -942,7 +967,7 @@ static int conv3x3_fwd_launch(const float* x, const float* w, const float* bias,
     const bool small_c = C <= 8;
 #define PD_LAUNCH_FWD(TH_, TW_)                                                                        \
     do {                                                                                               \
-        if (9 * C <= 32 && !mask) conv3x3_fwd_smallc_kernel<TH_, TW_><<<grid, CONV_THREADS, 0, s>>>(a); \
+        if (9 * C <= 32 && !mask && !out_mask) conv3x3_fwd_smallc_kernel<TH_, TW_><<<grid, CONV_THREADS, 0, s>>>(a); \
         else if (!a.c_vec && mask) conv3x3_fwd_kernel<TH_, TW_, 8, true, false><<<grid, CONV_THREADS, 0, s>>>(a); \
         else if (!a.c_vec) conv3x3_fwd_kernel<TH_, TW_, 8, false, false><<<grid, CONV_THREADS, 0, s>>>(a);  \
         else if (small_c && mask) conv3x3_fwd_kernel<TH_, TW_, 8, true, true><<<grid, CONV_THREADS, 0, s>>>(a); \
@@ -960,14 +985,15 @@ static int conv3x3_fwd_launch(const float* x, const float* w, const float* bias,
 
 extern "C" int pd_conv3x3_fwd_nhwc_f32(const float* x, const float* w, const float* bias, float* y, int N, int H,
                                        int W, int C, int K, int relu, void* stream) {
-    return conv3x3_fwd_launch(x, w, bias, nullptr, y, N, H, W, C, K, relu, stream);
+    return conv3x3_fwd_launch(x, w, bias, nullptr, nullptr, y, N, H, W, C, K, relu, stream);
 }
 
-extern "C" int pd_conv3x3_dgrad_nhwc_f32(const float* dy, const float* w_rot, const float* relu_out, float* dx, int N,
-                                         int H, int W, int K, int C, void* stream) {
+extern "C" int pd_conv3x3_dgrad_nhwc_f32(const float* dy, const float* w_rot, const float* relu_out,
+                                         const float* x_rectified, float* dx, int N, int H, int W, int K, int C,
+                                         void* stream) {
     // the forward kernel with the roles of the channel counts swapped: input = dy (K channels),
     // filter = rot180(w) [C][3][3][K], output = dx (C channels)
-    return conv3x3_fwd_launch(dy, w_rot, nullptr, relu_out, dx, N, H, W, K, C, 0, stream);
+    return conv3x3_fwd_launch(dy, w_rot, nullptr, relu_out, x_rectified, dx, N, H, W, K, C, 0, stream);
 }
 
 extern "C" int pd_conv3x3_filter_rot180_f32(const float* w, float* out, int K, int C, void* stream) {

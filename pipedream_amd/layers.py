@@ -81,8 +81,9 @@ class Linear(torch.nn.Module):
 # --------------------------------------------------------------------------------------
 class _Conv3x3Fn(torch.autograd.Function):
     @staticmethod
-    def forward(ctx, x, weight, bias, relu, grad_premasked=False):
+    def forward(ctx, x, weight, bias, relu, grad_premasked=False, input_rectified=False):
         x = ops.to_nhwc(x)
+        ctx.input_rectified = input_rectified
         y = ops.conv3x3_forward(x, weight, bias, relu)
         ctx.relu = relu
         ctx.has_bias = bias is not None
@@ -99,10 +100,10 @@ class _Conv3x3Fn(torch.autograd.Function):
         # load dy, so no masked copy of dy is ever written
         dx = dw = db = None
         if ctx.needs_input_grad[0]:
-            dx = ops.conv3x3_input_grad(dy, weight, relu_out=y)
+            dx = ops.conv3x3_input_grad(dy, weight, relu_out=y, x_rectified=x if ctx.input_rectified else None)
         if ctx.needs_input_grad[1] or (ctx.has_bias and ctx.needs_input_grad[2]):
             dw, db = ops.conv3x3_weight_grad(x, dy, with_bias=ctx.has_bias, relu_out=y)
-        return dx, dw, db, None, None
+        return dx, dw, db, None, None, None
 
 
 class Conv2d(torch.nn.Module):
@@ -114,10 +115,13 @@ class Conv2d(torch.nn.Module):
     ``grad_premasked=True`` (only with ``relu=True``) declares that the layer's output goes only to a
     layer whose backward already drops the gradient where this output is zero -- ``MaxPool2d(relu=True)``,
     which is the identity on an already rectified input in the forward pass -- so the ReLU backward need
-    not be applied (and the output not be read) again here.  Results are identical either way."""
+    not be applied (and the output not be read) again here.  ``input_rectified=True`` makes this layer
+    such a consumer: it declares that the layer's input is the output of a ReLU (a preceding
+    ``Conv2d(relu=True, grad_premasked=True)``) and zeroes the input gradient where the input is zero
+    as it is stored.  Results are identical either way."""
 
     def __init__(self, in_channels, out_channels, kernel_size=3, stride=1, padding=1, bias=True, relu=False,
-                 grad_premasked=False):
+                 grad_premasked=False, input_rectified=False):
         super(Conv2d, self).__init__()
         norm = lambda v: tuple(v) if isinstance(v, (tuple, list)) else (v, v)
         if norm(kernel_size) != (3, 3) or norm(stride) != (1, 1) or norm(padding) != (1, 1):
@@ -128,6 +132,7 @@ class Conv2d(torch.nn.Module):
         if grad_premasked and not relu:
             raise ValueError("grad_premasked only makes sense with relu=True")
         self.grad_premasked = grad_premasked
+        self.input_rectified = input_rectified
         w = torch.empty(out_channels, in_channels, 3, 3)
         torch.nn.init.kaiming_uniform_(w, a=math.sqrt(5))
         self.weight = torch.nn.Parameter(w.contiguous(memory_format=torch.channels_last))
@@ -138,7 +143,7 @@ class Conv2d(torch.nn.Module):
             self.bias = None
 
     def forward(self, x):
-        return _Conv3x3Fn.apply(x, self.weight, self.bias, self.relu, self.grad_premasked)
+        return _Conv3x3Fn.apply(x, self.weight, self.bias, self.relu, self.grad_premasked, self.input_rectified)
 
     def extra_repr(self):
         return "{}, {}, kernel_size=(3, 3), stride=(1, 1), padding=(1, 1), relu={}".format(

@@ -298,12 +298,20 @@ def conv3x3_forward(x, w, bias=None, relu=False):
     return y
 
 
-def conv3x3_input_grad(dy, w, relu_out=None):
+def conv3x3_input_grad(dy, w, relu_out=None, x_rectified=None):
     """dx of conv3x3_forward: the forward kernel on dy with the 180-degree-rotated filter.
-    ``relu_out`` (the layer's fused-ReLU output) masks dy while it is loaded."""
+    ``relu_out`` (the layer's fused-ReLU output) masks dy while it is loaded.  ``x_rectified``
+    (the layer's input, when that input is the output of a ReLU) zeroes dx where the input is
+    not positive: the producing layer's ReLU backward, applied as dx is stored."""
     _check(dy, "dy")
     if relu_out is not None and not _dense_same_order(relu_out, dy):
         raise ValueError("conv3x3_input_grad: relu_out must have dy's shape and memory order")
+    if x_rectified is not None:
+        _check(x_rectified, "x_rectified")
+        if (x_rectified.dim() != 4 or x_rectified.shape[0] != dy.shape[0] or x_rectified.shape[2:] != dy.shape[2:]
+                or x_rectified.shape[1] != w.shape[1]
+                or not x_rectified.is_contiguous(memory_format=torch.channels_last)):
+            raise ValueError("conv3x3_input_grad: x_rectified must be the layer's channels_last input")
     n, h, wd, k = _nhwc_dims(dy)
     kw, c = _filter_dims(w)
     if kw != k:
@@ -314,7 +322,7 @@ def conv3x3_input_grad(dy, w, relu_out=None):
     lib.pd_conv3x3_filter_rot180_f32(_ptr(w), _ptr(wr), k, c, _cabi.stream_ptr())
     dx = torch.empty((n, c, h, wd), dtype=torch.float32, device=dy.device, memory_format=torch.channels_last)
     with _timed("conv3x3_fwd_kernel" if k > 8 else "conv3x3_fwd_kernel_smallc", 18.0 * c * k * n * h * wd):
-        lib.pd_conv3x3_dgrad_nhwc_f32(_ptr(dy), _ptr(wr), _ptr(relu_out), _ptr(dx), n, h, wd, k, c,
+        lib.pd_conv3x3_dgrad_nhwc_f32(_ptr(dy), _ptr(wr), _ptr(relu_out), _ptr(x_rectified), _ptr(dx), n, h, wd, k, c,
                                       _cabi.stream_ptr())
     return dx
 

@@ -39,14 +39,16 @@ class FrontStage(torch.nn.Module):
 
     def __init__(self):
         super(FrontStage, self).__init__()
-        self.layer2 = layers.Conv2d(3, 64, relu=True)
+        # a convolution with input_rectified=True masks its input gradient where its (rectified) input
+        # is zero, so the convolution before it reads no mask either
+        self.layer2 = layers.Conv2d(3, 64, relu=True, grad_premasked=True)
         # a pooling layer with relu=True is the identity on the rectified output of the convolution
         # before it and masks the gradient in its backward kernel, so that convolution's gradient
         # kernels read no mask (grad_premasked)
-        self.layer4 = layers.Conv2d(64, 64, relu=True, grad_premasked=True)
+        self.layer4 = layers.Conv2d(64, 64, relu=True, grad_premasked=True, input_rectified=True)
         self.layer6 = layers.MaxPool2d(2, 2, relu=True)
-        self.layer7 = layers.Conv2d(64, 128, relu=True)
-        self.layer9 = layers.Conv2d(128, 128, relu=True, grad_premasked=True)
+        self.layer7 = layers.Conv2d(64, 128, relu=True, grad_premasked=True)
+        self.layer9 = layers.Conv2d(128, 128, relu=True, grad_premasked=True, input_rectified=True)
         self.layer11 = layers.MaxPool2d(2, 2, relu=True)
         _initialize_weights(self)
 
@@ -60,8 +62,8 @@ class FrontStage(torch.nn.Module):
 class Stage0(torch.nn.Module):
     def __init__(self):
         super(Stage0, self).__init__()
-        self.layer2 = layers.Conv2d(3, 64, relu=True)      # + layer3 ReLU
-        self.layer4 = layers.Conv2d(64, 64)
+        self.layer2 = layers.Conv2d(3, 64, relu=True, grad_premasked=True)      # + layer3 ReLU; masked by layer4
+        self.layer4 = layers.Conv2d(64, 64, input_rectified=True)
         _initialize_weights(self)
 
     def forward(self, input0):
@@ -72,8 +74,8 @@ class Stage1(torch.nn.Module):
     def __init__(self):
         super(Stage1, self).__init__()
         self.layer2 = layers.MaxPool2d(2, 2, relu=True)    # layer1 ReLU + layer2 MaxPool
-        self.layer3 = layers.Conv2d(64, 128, relu=True)    # + layer4
-        self.layer5 = layers.Conv2d(128, 128, relu=True, grad_premasked=True)   # + layer6; masked by layer7
+        self.layer3 = layers.Conv2d(64, 128, relu=True, grad_premasked=True)    # + layer4; masked by layer5
+        self.layer5 = layers.Conv2d(128, 128, relu=True, grad_premasked=True, input_rectified=True)   # + layer6; masked by layer7
         self.layer7 = layers.MaxPool2d(2, 2, relu=True)
         self.layer8 = layers.Conv2d(128, 256, relu=True)   # + layer9
         _initialize_weights(self)
@@ -87,12 +89,12 @@ class Stage1(torch.nn.Module):
 class Stage2(torch.nn.Module):
     def __init__(self):
         super(Stage2, self).__init__()
-        self.layer1 = layers.Conv2d(256, 256, relu=True)   # + layer2
-        self.layer3 = layers.Conv2d(256, 256, relu=True, grad_premasked=True)   # + layer4; masked by layer5
+        self.layer1 = layers.Conv2d(256, 256, relu=True, grad_premasked=True)   # + layer2; masked by layer3
+        self.layer3 = layers.Conv2d(256, 256, relu=True, grad_premasked=True, input_rectified=True)   # + layer4; masked by layer5
         self.layer5 = layers.MaxPool2d(2, 2, relu=True)
-        self.layer6 = layers.Conv2d(256, 512, relu=True)   # + layer7
-        self.layer8 = layers.Conv2d(512, 512, relu=True)   # + layer9
-        self.layer10 = layers.Conv2d(512, 512, relu=True)  # + layer11
+        self.layer6 = layers.Conv2d(256, 512, relu=True, grad_premasked=True)   # + layer7; masked by layer8
+        self.layer8 = layers.Conv2d(512, 512, relu=True, grad_premasked=True, input_rectified=True)   # + layer9
+        self.layer10 = layers.Conv2d(512, 512, relu=True, input_rectified=True)  # + layer11
         _initialize_weights(self)
 
     def forward(self, input0):
@@ -105,9 +107,9 @@ class Stage3(torch.nn.Module):
     def __init__(self, dropout=0.5, num_classes=1000):
         super(Stage3, self).__init__()
         self.layer1 = layers.MaxPool2d(2, 2)
-        self.layer2 = layers.Conv2d(512, 512, relu=True)   # + layer3
-        self.layer4 = layers.Conv2d(512, 512, relu=True)   # + layer5
-        self.layer6 = layers.Conv2d(512, 512, relu=True, grad_premasked=True)   # + layer7; masked by layer8
+        self.layer2 = layers.Conv2d(512, 512, relu=True, grad_premasked=True)   # + layer3; masked by layer4
+        self.layer4 = layers.Conv2d(512, 512, relu=True, grad_premasked=True, input_rectified=True)   # + layer5
+        self.layer6 = layers.Conv2d(512, 512, relu=True, grad_premasked=True, input_rectified=True)   # + layer7; masked by layer8
         self.layer8 = layers.MaxPool2d(2, 2, relu=True)
         self.flatten = layers.Flatten()
         self.layer11 = layers.Linear(25088, 4096, relu=True)   # + layer12

@@ -113,6 +113,43 @@ def test_fused_relu_mask_in_gradient_kernels():
     assert torch.equal(dx, dx_ref) and torch.equal(dw, dw_ref) and torch.equal(db, db_ref)
 
 
+@pytest.mark.parametrize("C,K,H,W", [(24, 40, 20, 28), (6, 10, 9, 11), (64, 64, 32, 32)])
+def test_input_gradient_masked_by_rectified_input(C, K, H, W):
+    # x_rectified zeroes dx where the layer's input is zero, as the producing layer's ReLU backward would
+    g = torch.Generator().manual_seed(9)
+    x = _nhwc(torch.randn(2, C, H, W, generator=g).clamp_min(0))
+    w = _nhwc(torch.randn(K, C, 3, 3, generator=g) / 15)
+    dy = _nhwc(torch.randn(2, K, H, W, generator=g))
+    y = ops.conv3x3_forward(x, w, None, relu=True)
+    dx_ref = ops.relu_backward(ops.conv3x3_input_grad(dy, w, relu_out=y), x)
+    dx = ops.conv3x3_input_grad(dy, w, relu_out=y, x_rectified=x)
+    assert torch.equal(dx, dx_ref)
+    assert (dx[x <= 0] == 0).all() and (dx != 0).any()
+    with pytest.raises(ValueError):
+        ops.conv3x3_input_grad(dy, w, x_rectified=dy if C != K else x[:1])
+
+
+def test_premasked_layer_chain_matches_unfused_chain():
+    # conv+ReLU -> conv+ReLU -> pool, with the ReLU backward moved into the consumers' kernels
+    torch.manual_seed(12)
+    plain = torch.nn.Sequential(layers.Conv2d(8, 16, relu=True), layers.Conv2d(16, 16, relu=True),
+                                layers.MaxPool2d(2, 2)).cuda()
+    fused = torch.nn.Sequential(layers.Conv2d(8, 16, relu=True, grad_premasked=True),
+                                layers.Conv2d(16, 16, relu=True, grad_premasked=True, input_rectified=True),
+                                layers.MaxPool2d(2, 2, relu=True)).cuda()
+    fused.load_state_dict(plain.state_dict())
+    x = torch.randn(2, 8, 12, 12).cuda()
+    xa, xb = x.clone().requires_grad_(True), x.clone().requires_grad_(True)
+    ya, yb = plain(xa), fused(xb)
+    assert torch.equal(ya, yb)
+    dy = torch.randn_like(ya)
+    ya.backward(dy)
+    yb.backward(dy)
+    assert torch.equal(xa.grad, xb.grad)
+    for pa, pb in zip(plain.parameters(), fused.parameters()):
+        assert torch.equal(pa.grad, pb.grad)
+
+
 def test_identity_filter_is_exact():
     # a centre-tap identity filter must reproduce the input bit for bit
     x = torch.randn(2, 32, 20, 20)
