@@ -9,9 +9,11 @@ plays its downstream neighbour (consumes the sent activation, queues a synthetic
 gradient ~ N(0,1)*1e-3).  All inputs are resident in HBM before the timed region.
 
 Prints ONE JSON line (see the keys below).  `roofline` covers the dominant kernel, the
-MFMA fp32 3x3 convolution (`conv3x3_fwd_kernel<.,.,16>`, used for forward and input
-gradient): algorithmic flop of its launches in the timed region / their summed duration,
-both measured with HIP events around every launch on the launch stream.
+MFMA fp32 3x3 convolution by Winograd F(2x2, 3x3) (`winograd_fwd_kernel`, used for forward
+and input gradient): algorithmic flop of its launches in the timed region (those of the
+direct convolution, 2*9*C*K per output pixel) / their summed duration, both measured with
+HIP events around every launch on the launch stream.  The kernel issues 16/36 of those
+multiplications to the MFMA units; `executed` is the rate it actually executes.
 `cpu_baseline` times the CPU oracle (torch.nn on the host cores) on a bounded sample of
 the same workload.
 """
@@ -345,7 +347,8 @@ def main():
         secondary(args)
         return
     elapsed, stats, _ = gpu_run(args.steps, args.warmup)
-    conv = stats["conv3x3_fwd_kernel"]
+    wino = "conv3x3_winograd_kernel" in stats
+    conv = stats["conv3x3_winograd_kernel" if wino else "conv3x3_fwd_kernel"]
     achieved = conv["rate"] / 1e12
     out = {
         "metric": "samples/sec per stage (fwd+bwd+stashed update), VGG16 bs64; optimizer HBM GB/s",
@@ -366,9 +369,13 @@ def main():
         "roofline": {"bound": "mfma", "achieved": achieved, "peak": PEAK_FP32_MFMA_TFLOPS, "unit": "TFLOP/s",
                      "frac": achieved / PEAK_FP32_MFMA_TFLOPS,
                      "traffic": args.traffic_bytes if args.traffic_bytes is not None else MEASURED_TRAFFIC_BYTES,
-                     "kernel": "conv3x3_fwd_kernel<.,.,16> (forward + input gradient)",
+                     "kernel": ("winograd_fwd_kernel (F(2x2,3x3); forward + input gradient)" if wino
+                                else "conv3x3_fwd_kernel<.,.,16> (forward + input gradient)"),
                      "launches": conv["launches"], "avg_us": conv["avg_us"],
-                     "flop_per_launch": conv["work_per_launch"]},
+                     "flop_per_launch": conv["work_per_launch"],
+                     # what the MFMA units execute: 16 multiplies per 2x2 outputs instead of 36
+                     "executed": achieved * (16.0 / 36.0 if wino else 1.0),
+                     "executed_frac": achieved * (16.0 / 36.0 if wino else 1.0) / PEAK_FP32_MFMA_TFLOPS},
         "kernels": {k: {"launches": v["launches"], "avg_us": round(v["avg_us"], 1),
                         "TFLOP/s": round(v["rate"] / 1e12, 2)} for k, v in stats.items()},
         "optimizer_hbm": optimizer_bandwidth(),

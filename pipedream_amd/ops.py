@@ -280,6 +280,41 @@ def _filter_dims(w):
     return w.shape[0], w.shape[1]
 
 
+# Which kernel computes 3x3 convolutions and their input gradients: "auto" takes the Winograd
+# F(2x2, 3x3) kernel where it applies and pays (8 | C, C >= 16, K >= 32), "direct" always the
+# direct kernel, "winograd" the Winograd kernel wherever it applies.
+_CONV_ALGO = "auto"
+
+
+def set_conv_algorithm(name):
+    global _CONV_ALGO
+    if name not in ("auto", "direct", "winograd"):
+        raise ValueError("conv algorithm must be 'auto', 'direct' or 'winograd'")
+    _CONV_ALGO = name
+
+
+def _use_winograd(c, k):
+    if _CONV_ALGO == "direct" or not _cabi.lib().pd_conv3x3_winograd_supported(c, k):
+        return False
+    return _CONV_ALGO == "winograd" or (c >= 16 and k >= 32)
+
+
+def _winograd_conv(x, w, bias, in_mask, out_mask, n, h, wd, c, k, relu, rot180):
+    """The convolution with c input and k output channels through the Winograd kernels; ``w`` is its
+    own [k,c,3,3] filter, or with ``rot180`` the [c,k,3,3] filter of the layer whose input gradient
+    this is."""
+    lib = _cabi.lib()
+    nbytes = ctypes.c_uint64()
+    lib.pd_conv3x3_winograd_filter_bytes(c, k, ctypes.byref(nbytes))
+    u = torch.empty(nbytes.value // 4, dtype=torch.float32, device=x.device)
+    lib.pd_conv3x3_winograd_filter_f32(_ptr(w), _ptr(u), c, k, int(rot180), _cabi.stream_ptr())
+    y = torch.empty((n, k, h, wd), dtype=torch.float32, device=x.device, memory_format=torch.channels_last)
+    with _timed("conv3x3_winograd_kernel", 18.0 * c * k * n * h * wd):
+        lib.pd_conv3x3_winograd_fwd_nhwc_f32(_ptr(x), _ptr(u), _ptr(bias), _ptr(in_mask), _ptr(out_mask), _ptr(y),
+                                             n, h, wd, c, k, int(relu), _cabi.stream_ptr())
+    return y
+
+
 def conv3x3_forward(x, w, bias=None, relu=False):
     """y = conv2d(x, w, bias, stride 1, padding 1) (+ReLU).  x: NHWC-ordered [N,C,H,W]."""
     _check(x, "x")
@@ -291,6 +326,8 @@ def conv3x3_forward(x, w, bias=None, relu=False):
         _check(bias, "bias")
         if bias.numel() != k or not bias.is_contiguous():
             raise ValueError("conv3x3: bias must be a contiguous vector of K=%d" % k)
+    if _use_winograd(c, k):
+        return _winograd_conv(x, w, bias, None, None, n, h, wd, c, k, relu, False)
     y = torch.empty((n, k, h, wd), dtype=torch.float32, device=x.device, memory_format=torch.channels_last)
     with _timed("conv3x3_fwd_kernel" if c > 8 else "conv3x3_fwd_kernel_smallc", 18.0 * c * k * n * h * wd):
         _cabi.lib().pd_conv3x3_fwd_nhwc_f32(_ptr(x), _ptr(w), _ptr(bias), _ptr(y), n, h, wd, c, k, int(relu),
@@ -316,6 +353,8 @@ def conv3x3_input_grad(dy, w, relu_out=None, x_rectified=None):
     kw, c = _filter_dims(w)
     if kw != k:
         raise ValueError("conv3x3_input_grad: dy has %d channels, filter has %d outputs" % (k, kw))
+    if _use_winograd(k, c):
+        return _winograd_conv(dy, w, None, relu_out, x_rectified, n, h, wd, k, c, False, True)
     lib = _cabi.lib()
     # rotated filter: logical [C, K, 3, 3] in channels_last order = memory [C][3][3][K]
     wr = torch.empty((c, k, 3, 3), dtype=torch.float32, device=w.device, memory_format=torch.channels_last)

@@ -3,6 +3,11 @@ ABI against the torch CPU library (the third-party routine the reference's Conv2
 call) in fp64, plus a brute-force direct convolution on a tiny case that pins the index
 conventions (tap order, padding, which operand is flipped).
 
+Every test runs under both convolution algorithms: "direct" and "winograd" (F(2x2, 3x3), taken
+where its shape conditions hold, the direct kernel elsewhere).  The Winograd kernel is pinned by the
+same library results at the same tolerance, by the brute-force case below through a filter that is
+not symmetric under any flip, and by an impulse response that must reproduce each filter tap.
+
 Tolerance: fp32 accumulation over R terms against an fp64 result: rtol 1e-5 plus
 atol = 4e-7 * sqrt(R) * (typical |term| sum scale) as set per test."""
 import math
@@ -15,6 +20,13 @@ import torch.nn.functional as F
 from pipedream_amd import layers, ops
 
 pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(autouse=True, params=["direct", "winograd"])
+def conv_algorithm(request):
+    ops.set_conv_algorithm(request.param)
+    yield request.param
+    ops.set_conv_algorithm("auto")
 
 
 def _nhwc(t):
@@ -150,7 +162,38 @@ def test_premasked_layer_chain_matches_unfused_chain():
         assert torch.equal(pa.grad, pb.grad)
 
 
-def test_identity_filter_is_exact():
+def test_winograd_impulse_response_and_brute_force():
+    # the Winograd path on shapes it accepts: (a) brute-force direct convolution of a small case with
+    # random (asymmetric) filters; (b) a unit impulse must return the flipped filter taps around it
+    ops.set_conv_algorithm("winograd")
+    rng = np.random.RandomState(1)
+    x = rng.randn(1, 8, 6, 7)
+    w = rng.randn(4, 8, 3, 3)
+    b = rng.randn(4)
+    got = ops.conv3x3_forward(_nhwc(torch.tensor(x, dtype=torch.float32)), _nhwc(torch.tensor(w, dtype=torch.float32)),
+                              torch.tensor(b, dtype=torch.float32).cuda())
+    np.testing.assert_allclose(got.cpu().numpy(), _direct_conv(x, w, b), rtol=1e-5, atol=2e-5)
+    x = torch.zeros(1, 16, 20, 37)
+    x[0, 5, 9, 30] = 1.0
+    w = torch.randn(32, 16, 3, 3)
+    y = ops.conv3x3_forward(_nhwc(x), _nhwc(w)).cpu()
+    for r in range(3):
+        for s_ in range(3):
+            # y[k, 9 - (r-1), 30 - (s-1)] = w[k, 5, r, s]
+            torch.testing.assert_close(y[0, :, 10 - r, 31 - s_], w[:, 5, r, s_], rtol=1e-5, atol=1e-5)
+    y[0, :, 8:11, 29:32] = 0
+    assert y.abs().max() < 1e-5
+    # input gradient = correlation with the unflipped taps
+    dy = torch.zeros(1, 32, 20, 37)
+    dy[0, 7, 0, 36] = 1.0                        # a corner: padding on two sides
+    dx = ops.conv3x3_input_grad(_nhwc(dy), _nhwc(w)).cpu()
+    torch.testing.assert_close(dx[0, :, 0, 36], w[7, :, 1, 1], rtol=1e-5, atol=1e-5)
+    torch.testing.assert_close(dx[0, :, 1, 35], w[7, :, 2, 0], rtol=1e-5, atol=1e-5)
+
+
+def test_identity_filter_is_exact(conv_algorithm):
+    if conv_algorithm != "direct":
+        pytest.skip("bit-exact pass-through is a property of the direct kernel only")
     # a centre-tap identity filter must reproduce the input bit for bit
     x = torch.randn(2, 32, 20, 20)
     w = torch.zeros(32, 32, 3, 3)
