@@ -32,7 +32,7 @@ SGD_KW = dict(lr=0.01, momentum=0.9, weight_decay=5e-4)
 PEAK_FP32_MFMA_TFLOPS = 157.3
 # HBM bytes per launch of the dominant kernel, from the rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE
 # runs summarised under profiles/ (None until measured for the current kernel).
-MEASURED_TRAFFIC_BYTES = 1.446e9
+MEASURED_TRAFFIC_BYTES = 1.253e9
 
 
 def build_stage():
@@ -144,7 +144,7 @@ def pmc_probe():
     """Workload for `rocprofv3 --pmc FETCH_SIZE` / `--pmc WRITE_SIZE` runs: a plain copy of
     known size (calibrates the counters: pd_copy_kernel moves 1 GiB in and 1 GiB out per
     launch) followed by two steady-state steps of the benchmark stage, so the per-dispatch
-    counter values of conv3x3_fwd_kernel cover exactly the launch mix of the timed region."""
+    counter values of the convolution kernels cover exactly the launch mix of the timed region."""
     import ctypes
     import torch
     from pipedream_amd import _cabi
