@@ -213,6 +213,18 @@ int pd_conv3x3_winograd_filter_f32(const float* w, float* u, int C, int K, int r
 int pd_conv3x3_winograd_fwd_nhwc_f32(const float* x, const float* u, const float* bias,
                                      const float* in_mask, const float* out_mask, float* y,
                                      int N, int H, int W, int C, int K, int relu, void* stream);
+/* Weight (and optional bias) gradient of the same convolution in the Winograd domain: sums
+ * dU = sum over 2x2 output tiles of (A dY A^T) (B^T d B) in persistent blocks, adds the blocks' partial
+ * sums in fixed order and applies G^T . G.  Deterministic; agrees with pd_conv3x3_wgrad_nhwc_f32 to
+ * fp32 rounding.  Needs C and K multiples of 64 with (C/64)*(K/64) a power of two <= 32
+ * (pd_conv3x3_winograd_wgrad_supported() returns 1) and a workspace of
+ * pd_conv3x3_winograd_wgrad_workspace_bytes() bytes.  dw is [K][3][3][C]; dbias may be NULL.
+ * (Backward of torch.nn.Conv2d, vgg16/gpus=4_straight/stage0.py:12-14.) */
+int pd_conv3x3_winograd_wgrad_supported(int C, int K);
+int pd_conv3x3_winograd_wgrad_workspace_bytes(int C, int K, uint64_t* bytes);
+int pd_conv3x3_winograd_wgrad_nhwc_f32(const float* x, const float* dy, float* dw, float* dbias,
+                                       void* workspace, uint64_t workspace_bytes,
+                                       int N, int H, int W, int C, int K, void* stream);
 /* Weight and (optional, dbias may be NULL) bias gradient of the same convolution:
  * dw[k][r][s][c] = sum_{n,y,x} dy[n,y,x,k] * x[n,y+r-1,x+s-1,c].  Deterministic two-pass
  * reduction through a caller-provided workspace of pd_conv3x3_wgrad_workspace_bytes().

@@ -520,3 +520,427 @@ extern "C" int pd_conv3x3_winograd_fwd_nhwc_f32(const float* x, const float* u, 
     PD_CHECK_LAUNCH(who);
     return PD_OK;
 }
+
+// =====================================================================================================
+// Weight gradient in the Winograd domain.
+//
+//   dU[g][k][c] = sum over tiles of  dM[g][tile][k] * V[g][tile][c],   dM = A dY A^T,  V = B^T d B,
+//   dw[k][.][.][c] = G^T dU[.][k][c] G
+//
+// (the derivative of Y = A^T [U .* V] A with U = G g G^T): 16 GEMMs [K x tiles] * [tiles x C] whose
+// reduction runs over all 2 x 2 output tiles of the batch, again 16 multiplies where the direct
+// algorithm needs 36.  A persistent 512-thread block owns one (64 out-channel, 64 in-channel) block pair
+// and a contiguous range of strips (1 x 8 tiles = 2 x 16 output pixels), keeps all 16 x 64 x 64 sums in
+// its accumulators (8 GEMMs x 32 x 32 per wave) and writes them once at the end; two small kernels add
+// the blocks' partial sums in fixed order and apply G^T . G (deterministic, no atomics).
+//
+// Per strip (= one pipeline step, 32 MFMAs per wave):
+//   * x: the 4 x 18 pixel x 64 channel patch goes global -> registers (a step in flight) -> LDS; every
+//     thread then forms one row of B^T d for one (tile, 4 channels), applies . B and writes V[g][tile][c]
+//     (the two 32-channel halves of odd tiles are swapped, so the B-fragment reads below, which take an
+//     even tile in lanes 0-31 and an odd one in lanes 32-63, hit different banks);
+//   * dY never touches LDS: the MFMA A operand of lane (k, h) is dM[g][tile 2j+h][k], so each lane loads
+//     the 4 x 4 dY values of its own k for its four tiles (128-byte runs across a half wave), a step
+//     ahead, and forms the dM values it needs with a few additions right before the MFMAs.  The signs of
+//     A's last row/column are left out here and applied in the final transform.
+//   * dbias[k] is the sum of dM[1][1] (= the sum of a tile's four dY values) over all tiles.
+// =====================================================================================================
+namespace {
+
+constexpr int WW_THREADS = 512;
+constexpr int WW_TILES = 8;                          // tiles per strip
+constexpr int WW_PATCH_W = 2 * WW_TILES + 2;         // input columns of a strip's patch
+constexpr int WW_ROW_PIECES = 320;                   // 16-byte pieces per patch row, padded from 18*16 to 5 waves
+constexpr int WW_V_STAGE = WG_G * WW_TILES * 64;     // floats: [g][tile][c]
+constexpr int WW_RAW_STAGE = 4 * WW_PATCH_W * 64;    // floats: [row][pixel][c]
+constexpr int WW_RAW_OFF = 2 * WW_V_STAGE;
+constexpr int WW_LDS_FLOATS = WW_RAW_OFF + 2 * WW_RAW_STAGE;
+constexpr int WW_BLOCKS = 256;                       // persistent blocks: 8 dies x 32
+constexpr int WW_PART_FLOATS = WG_G * 64 * 64;       // one block's partial dU
+
+struct WinoWgradArgs {
+    const float* x;      // [N,H,W,C]
+    const float* dy;     // [N,H,W,K]
+    float* part;         // [pair][rank][16][64][64]
+    float* part_db;      // [pair][rank][2][64]
+    int N, H, W, C, K;
+    int sx, sy;          // strips per row pair, row pairs per image
+    int n_strips, strips_per_rank;
+    int c_blocks, n_pairs, ranks;
+};
+
+struct StripPos { int n, y0, x0; };
+
+__device__ __forceinline__ StripPos strip_decode(const WinoWgradArgs& a, int s) {
+    StripPos p;
+    const int per_img = a.sx * a.sy;
+    p.n = s / per_img;
+    const int rem = s - p.n * per_img;
+    const int ty = rem / a.sx;
+    p.y0 = 2 * ty;
+    p.x0 = (rem - ty * a.sx) * (2 * WW_TILES);
+    return p;
+}
+__device__ __forceinline__ void strip_next(const WinoWgradArgs& a, StripPos& p) {
+    p.x0 += 2 * WW_TILES;
+    if (p.x0 >= a.W) {
+        p.x0 = 0;
+        p.y0 += 2;
+        if (p.y0 >= a.H) { p.y0 = 0; ++p.n; }
+    }
+}
+
+__global__ __launch_bounds__(WW_THREADS, 1) void winograd_wgrad_kernel(const WinoWgradArgs a) {
+    __shared__ __attribute__((aligned(16))) float lds[WW_LDS_FLOATS];
+
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    // block -> (pair, rank): the 32 blocks of a die cover all pairs of a contiguous strip range, so the
+    // pairs that read the same x and dY strips run side by side on one L2
+    const int xcd = blockIdx.x % WG_XCD, slot = blockIdx.x / WG_XCD;
+    const int pair = slot % a.n_pairs, sub = slot / a.n_pairs;
+    const int rank = xcd * (32 / a.n_pairs) + sub;
+    const int kb = pair / a.c_blocks, cb = pair % a.c_blocks;
+    const int s_begin = rank * a.strips_per_rank;
+    int s_end = s_begin + a.strips_per_rank;
+    s_end = s_end < a.n_strips ? s_end : a.n_strips;
+    const int n_my = s_end > s_begin ? s_end - s_begin : 0;
+
+    // ---- stage 1 role: pieces p = tid + 512 j of the patch: row p / 320 (uniform in a wave), pixel
+    //      (p % 320) / 16 (pixels 18, 19 are padding of the piece grid), channels 4 (p % 16) .. +3.
+    //      A patch row is read through its own buffer descriptor that starts one pixel left of the
+    //      strip and ends with the image row, so columns beyond the image read 0; the column left of
+    //      the image (first strip of a row) is switched off per lane; rows outside the image get an
+    //      empty descriptor.
+    uint32_t xoff[3], xoff_first[3];
+    int raw_dst[3], prow[3];
+    bool live[3];
+#pragma unroll
+    for (int j = 0; j < 3; ++j) {
+        const int p = tid + WW_THREADS * j;
+        prow[j] = __builtin_amdgcn_readfirstlane(p / WW_ROW_PIECES);
+        const int rem = p % WW_ROW_PIECES, ppx = rem >> 4, pcg = rem & 15;
+        live[j] = ppx < WW_PATCH_W && p < 4 * WW_ROW_PIECES;
+        xoff[j] = live[j] ? (uint32_t)((ppx * a.C + pcg * 4) * 4) : 0x80000000u;
+        xoff_first[j] = ppx == 0 ? 0x80000000u : xoff[j];
+        raw_dst[j] = ((prow[j] & 3) * WW_PATCH_W + (live[j] ? ppx : 0)) * 64 + pcg * 4;
+    }
+    float4_t rawr[3];
+    auto load_raw = [&](const StripPos& p, bool valid) {
+#pragma unroll
+        for (int j = 0; j < 3; ++j) {
+            const int gy = p.y0 - 1 + prow[j];
+            const bool row_ok = valid && gy >= 0 && gy < a.H && (j < 2 || wave < 4);
+            const float* base = a.x + (((size_t)p.n * a.H + gy) * a.W + p.x0 - 1) * a.C + cb * 64;
+            const uint32_t bytes = row_ok ? (uint32_t)((a.W - p.x0 + 1) * a.C - cb * 64) * 4 : 0u;
+            const __amdgpu_buffer_rsrc_t r = __builtin_amdgcn_make_buffer_rsrc((void*)base, 0, bytes, 0x00020000);
+            rawr[j] = __builtin_bit_cast(
+                float4_t, __builtin_amdgcn_raw_buffer_load_b128(r, p.x0 == 0 ? xoff_first[j] : xoff[j], 0, 0));
+        }
+    };
+    auto store_raw = [&](int stage, int j) {
+        if (live[j]) *(float4_t*)(lds + WW_RAW_OFF + stage * WW_RAW_STAGE + raw_dst[j]) = rawr[j];
+    };
+
+    // ---- stage 2 role: tile tt (of the strip's 8), channels 4 cg .. +3, row ti of B^T d = Ra + sgn * Rb
+    const int ti = wave & 3;
+    const int tt = (wave >> 2) * 4 + (lane >> 4), cg = lane & 15;
+    const int row_a = ti == 0 ? 0 : ti == 2 ? 2 : 1;
+    const int row_b = ti == 2 ? 1 : ti == 3 ? 3 : 2;
+    const float sgn = ti == 1 ? 1.f : -1.f;
+    const int src_a = (row_a * WW_PATCH_W + 2 * tt) * 64 + cg * 4, src_b = (row_b * WW_PATCH_W + 2 * tt) * 64 + cg * 4;
+    const int v_dst = (ti * 4 * WW_TILES + tt) * 64 + ((cg * 4) ^ (32 * (tt & 1)));
+    float4_t t[4], dc[2], vout;
+    auto read_col = [&](const float* rs, int s) {
+        dc[0] = *(const float4_t*)(rs + src_a + s * 64);
+        dc[1] = *(const float4_t*)(rs + src_b + s * 64);
+    };
+    auto transform_col = [&](int s) { t[s] = dc[0] + sgn * dc[1]; };
+    auto transform_out = [&](int m) {
+        if (m == 0) vout = t[0] - t[2];
+        else if (m == 1) vout = t[1] + t[2];
+        else if (m == 2) vout = t[2] - t[1];
+        else vout = t[1] - t[3];
+    };
+    auto store_out = [&](float* vst, int m) { *(float4_t*)(vst + v_dst + m * (WW_TILES * 64)) = vout; };
+
+    // ---- stage 3 role: wave (gh, wm, wn): GEMMs gh*8..+7, out channels wm*32..+31, in channels wn*32..+31;
+    //      lane (h, cl): row/column cl, tiles 2j + h of the strip
+    const int gh = wave >> 2, wm = (wave >> 1) & 1, wn = wave & 1;
+    const int h = lane >> 5, cl = lane & 31;
+    const int b_src = (gh * 8 * WW_TILES + h) * 64 + ((wn ^ h) * 32 + cl);
+    // dY: value (row a, column b, tile 2j+h) of out channel k sits at (a*W + 4j + 2h + b) * K + k from the
+    // strip's first pixel; a row is read through a descriptor that ends with the image row
+    uint32_t dyoff[4][2];
+#pragma unroll
+    for (int j = 0; j < 4; ++j)
+#pragma unroll
+        for (int b = 0; b < 2; ++b) dyoff[j][b] = (uint32_t)((4 * j + 2 * h + b) * a.K + kb * 64 + wm * 32 + cl) * 4;
+    float dyr[2][2][4];                        // [row a][column b][j]
+    auto load_dy = [&](const StripPos& p, bool valid) {
+#pragma unroll
+        for (int r = 0; r < 2; ++r) {
+            const bool row_ok = valid && p.y0 + r < a.H;
+            const float* base = a.dy + (((size_t)p.n * a.H + p.y0 + r) * a.W + p.x0) * a.K;
+            const uint32_t bytes = row_ok ? (uint32_t)((a.W - p.x0) * a.K) * 4 : 0u;
+            const __amdgpu_buffer_rsrc_t rs = __builtin_amdgcn_make_buffer_rsrc((void*)base, 0, bytes, 0x00020000);
+#pragma unroll
+            for (int b = 0; b < 2; ++b)
+#pragma unroll
+                for (int j = 0; j < 4; ++j)
+                    dyr[r][b][j] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(rs, dyoff[j][b], 0, 0));
+        }
+    };
+    float rr[2][2][4];                         // rows 2gh, 2gh+1 of A dY (signs of row 3 left out): [ii][b][j]
+
+    float16_t acc[WG_GW];
+#pragma unroll
+    for (int g = 0; g < WG_GW; ++g)
+#pragma unroll
+        for (int e = 0; e < 16; ++e) acc[g][e] = 0.f;
+    float db_acc = 0.f;
+
+    if (n_my > 0) {
+        // cursors of the stages: strip of the next raw-x request (3 ahead of the multiply), of the next
+        // dY request (1 ahead)
+        StripPos lp = strip_decode(a, s_begin), dp = lp;
+        int l_left = n_my, d_left = n_my;      // strips not yet requested
+        auto next_l = [&]() { --l_left; strip_next(a, lp); };
+        auto next_d = [&]() { --d_left; strip_next(a, dp); };
+
+        // ---- prologue: strips 0 and 1 into LDS, strip 2 into registers, strip 0 transformed, dY of strip 0
+        load_raw(lp, l_left > 0); next_l();
+        load_dy(dp, d_left > 0); next_d();
+#pragma unroll
+        for (int j = 0; j < 3; ++j) store_raw(0, j);
+        load_raw(lp, l_left > 0); next_l();
+#pragma unroll
+        for (int j = 0; j < 3; ++j) store_raw(1, j);
+        load_raw(lp, l_left > 0); next_l();
+        __syncthreads();
+#pragma unroll
+        for (int s = 0; s < 4; ++s) { read_col(lds + WW_RAW_OFF, s); transform_col(s); }
+#pragma unroll
+        for (int m = 0; m < 4; ++m) { transform_out(m); store_out(lds, m); }
+        __builtin_amdgcn_s_waitcnt(0);
+        __syncthreads();
+        float bf[2][2][4];                     // B fragments of GEMM pair p wait in bf[p & 1]: [g of the pair][j]
+#pragma unroll
+        for (int g = 0; g < 2; ++g)
+#pragma unroll
+            for (int j = 0; j < 4; ++j) bf[0][g][j] = lds[b_src + (g * WW_TILES + 2 * j) * 64];
+        read_col(lds + WW_RAW_OFF + WW_RAW_STAGE, 0);
+
+        for (int q = 0; q < n_my; ++q) {
+            const float* vs = lds + (q & 1) * WW_V_STAGE + b_src;
+            const float* vs_next = lds + ((q + 1) & 1) * WW_V_STAGE + b_src;
+            float* vn = lds + ((q + 1) & 1) * WW_V_STAGE;
+            const float* rs = lds + WW_RAW_OFF + ((q + 1) & 1) * WW_RAW_STAGE;
+            const float* rs_next = lds + WW_RAW_OFF + (q & 1) * WW_RAW_STAGE;
+            // rows of A dY for this wave's GEMMs, from the dY values requested a step ago
+#pragma unroll
+            for (int b = 0; b < 2; ++b)
+#pragma unroll
+                for (int j = 0; j < 4; ++j) {
+                    rr[0][b][j] = gh ? dyr[0][b][j] - dyr[1][b][j] : dyr[0][b][j];
+                    rr[1][b][j] = gh ? dyr[1][b][j] : dyr[0][b][j] + dyr[1][b][j];
+                }
+            load_dy(dp, d_left > 0);           // strip q+1
+            next_d();
+            if (gh == 0) {
+#pragma unroll
+                for (int j = 0; j < 4; ++j) db_acc += rr[1][0][j] + rr[1][1][j];
+            }
+            __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+            for (int gp = 0; gp < WG_GW / 2; ++gp) {
+                const int g0 = 2 * gp, g1 = 2 * gp + 1, cur = gp & 1, ii = gp >> 1;
+                // A operands of the pair: columns (0, 1) or (2, 3) of  rr . A^T  (sign of column 3 left out)
+                float a0[4], a1[4];
+#pragma unroll
+                for (int j = 0; j < 4; ++j) {
+                    a0[j] = (gp & 1) ? rr[ii][0][j] - rr[ii][1][j] : rr[ii][0][j];
+                    a1[j] = (gp & 1) ? rr[ii][1][j] : rr[ii][0][j] + rr[ii][1][j];
+                }
+#pragma unroll
+                for (int k = 0; k < 8; ++k) {
+                    const int j = k >> 1;
+                    if ((k & 1) == 0)
+                        acc[g0] = __builtin_amdgcn_mfma_f32_32x32x2f32(a0[j], bf[cur][0][j], acc[g0], 0, 0, 0);
+                    else
+                        acc[g1] = __builtin_amdgcn_mfma_f32_32x32x2f32(a1[j], bf[cur][1][j], acc[g1], 0, 0, 0);
+                    if (k == 0) {
+                        if (gp < 3) {          // B fragments of the next section
+#pragma unroll
+                            for (int g = 0; g < 2; ++g)
+#pragma unroll
+                                for (int jj = 0; jj < 4; ++jj)
+                                    bf[cur ^ 1][g][jj] = vs[((g0 + 2 + g) * WW_TILES + 2 * jj) * 64];
+                        } else {
+                            store_out(vn, 3);
+                            __syncthreads();   // stage 2 of strip q+1 and stage 1 of strip q+2 are in LDS
+#pragma unroll
+                            for (int g = 0; g < 2; ++g)
+#pragma unroll
+                                for (int jj = 0; jj < 4; ++jj)
+                                    bf[0][g][jj] = vs_next[(g * WW_TILES + 2 * jj) * 64];
+                            read_col(rs_next, 0);
+                        }
+                    }
+                    // stage 2 of strip q+1
+                    if (gp == 0 && k == 2) transform_col(0);
+                    if (gp == 0 && k == 3) read_col(rs, 1);
+                    if (gp == 0 && k == 5) transform_col(1);
+                    if (gp == 0 && k == 6) read_col(rs, 2);
+                    if (gp == 1 && k == 1) transform_col(2);
+                    if (gp == 1 && k == 2) read_col(rs, 3);
+                    if (gp == 1 && k == 4) transform_col(3);
+                    if (gp == 2 && (k == 1 || k == 3 || k == 5)) transform_out(k >> 1);
+                    if (gp == 2 && (k == 2 || k == 4 || k == 6)) store_out(vn, (k >> 1) - 1);
+                    if (gp == 2 && k == 7) transform_out(3);
+                    // stage 1: the registers hold strip q+2 (requested a step ago); then request strip q+3
+                    if (gp == 1 && k >= 5) store_raw(q & 1, k - 5);
+                    if (gp == 2 && k == 0) { load_raw(lp, l_left > 0); next_l(); }
+                    __builtin_amdgcn_sched_barrier(0);
+                }
+            }
+        }
+    }
+
+    // ---- the block's sums: partial dU in [g][k][c] order, partial dbias per (tile half, k)
+    float* part = a.part + (size_t)(pair * a.ranks + rank) * WW_PART_FLOATS;
+#pragma unroll
+    for (int g = 0; g < WG_GW; ++g)
+#pragma unroll
+        for (int e = 0; e < 16; ++e) {
+            float v;
+            asm volatile("v_accvgpr_read_b32 %0, %1" : "=v"(v) : "a"(acc[g][e]));
+            const int k = wm * 32 + 8 * (e / 4) + 4 * h + (e % 4);
+            part[((gh * WG_GW + g) * 64 + k) * 64 + wn * 32 + cl] = v;
+        }
+    if (gh == 0 && wn == 0) a.part_db[((size_t)(pair * a.ranks + rank) * 2 + h) * 64 + wm * 32 + cl] = db_acc;
+}
+
+// Sum of the ranks' partial dU (and partial dbias) of every pair, in rank order.
+__global__ __launch_bounds__(256) void winograd_wgrad_sum_kernel(const float* __restrict__ part,
+                                                                 const float* __restrict__ part_db,
+                                                                 float* __restrict__ du, float* __restrict__ dbsum,
+                                                                 int n_pairs, int ranks) {
+    const int per_pair = WW_PART_FLOATS / 4;
+    const long id = (long)blockIdx.x * 256 + threadIdx.x;
+    if (id < (long)n_pairs * per_pair) {
+        const int pair = (int)(id / per_pair), i = (int)(id % per_pair);
+        const float4_t* src = (const float4_t*)part + (size_t)pair * ranks * per_pair + i;
+        float4_t s = {0.f, 0.f, 0.f, 0.f};
+        for (int r = 0; r < ranks; ++r) s += src[(size_t)r * per_pair];
+        ((float4_t*)du)[id] = s;
+    }
+    if (id < (long)n_pairs * 64) {
+        const int pair = (int)(id / 64), k = (int)(id % 64);
+        float s = 0.f;
+        for (int r = 0; r < ranks * 2; ++r) s += part_db[((size_t)pair * ranks * 2 + r) * 64 + k];
+        dbsum[id] = s;
+    }
+}
+
+// dw[k][r][s][c] = (G^T dU[.][k][c] G)[r][s] with the signs of A's last row / column restored, and dbias.
+__global__ __launch_bounds__(256) void winograd_wgrad_final_kernel(const float* __restrict__ du,
+                                                                   const float* __restrict__ dbsum,
+                                                                   float* __restrict__ dw, float* __restrict__ db,
+                                                                   int K, int C, int c_blocks) {
+    const long id = (long)blockIdx.x * 256 + threadIdx.x;
+    if (id >= (long)K * C) return;
+    const int c = (int)(id % C), k = (int)(id / C);
+    const int pair = (k / 64) * c_blocks + c / 64;
+    const float* src = du + (size_t)pair * WW_PART_FLOATS + (k % 64) * 64 + (c % 64);
+    float u[4][4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+#pragma unroll
+        for (int m = 0; m < 4; ++m) {
+            const float v = src[(i * 4 + m) * 64 * 64];
+            u[i][m] = ((i == 3) != (m == 3)) ? -v : v;
+        }
+    float t[4][3];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        t[i][0] = u[i][0] + 0.5f * (u[i][1] + u[i][2]);
+        t[i][1] = 0.5f * (u[i][1] - u[i][2]);
+        t[i][2] = u[i][3] + 0.5f * (u[i][1] + u[i][2]);
+    }
+    float* out = dw + (size_t)k * 9 * C + c;
+#pragma unroll
+    for (int s = 0; s < 3; ++s) {
+        out[(0 * 3 + s) * C] = t[0][s] + 0.5f * (t[1][s] + t[2][s]);
+        out[(1 * 3 + s) * C] = 0.5f * (t[1][s] - t[2][s]);
+        out[(2 * 3 + s) * C] = t[3][s] + 0.5f * (t[1][s] + t[2][s]);
+    }
+    if (db && c == 0) db[k] = dbsum[(size_t)((k / 64) * c_blocks) * 64 + (k % 64)];
+}
+
+bool wino_wgrad_shape_ok(int C, int K) {
+    if (C % 64 != 0 || K % 64 != 0) return false;
+    const int pairs = (C / 64) * (K / 64);
+    return pairs <= 32 && (pairs & (pairs - 1)) == 0;
+}
+
+}  // namespace
+
+extern "C" int pd_conv3x3_winograd_wgrad_supported(int C, int K) {
+    return (C > 0 && K > 0 && wino_wgrad_shape_ok(C, K)) ? 1 : 0;
+}
+
+extern "C" int pd_conv3x3_winograd_wgrad_workspace_bytes(int C, int K, uint64_t* bytes) {
+    PD_REQUIRE(bytes != nullptr, PD_EINVAL, "pd_conv3x3_winograd_wgrad_workspace_bytes: NULL pointer");
+    PD_REQUIRE(C > 0 && K > 0 && wino_wgrad_shape_ok(C, K), PD_ESHAPE,
+               "pd_conv3x3_winograd_wgrad_workspace_bytes: needs C and K multiples of 64 with C*K/4096 a power "
+               "of two <= 32 (C=%d K=%d)", C, K);
+    const uint64_t pairs = (uint64_t)(C / 64) * (K / 64);
+    // per block: partial dU and 2 x 64 partial dbias; per pair: summed dU and dbias
+    *bytes = ((uint64_t)WW_BLOCKS * (WW_PART_FLOATS + 128) + pairs * (WW_PART_FLOATS + 64)) * sizeof(float);
+    return PD_OK;
+}
+
+extern "C" int pd_conv3x3_winograd_wgrad_nhwc_f32(const float* x, const float* dy, float* dw, float* dbias,
+                                                  void* workspace, uint64_t workspace_bytes, int N, int H, int W,
+                                                  int C, int K, void* stream) {
+    const char* who = "pd_conv3x3_winograd_wgrad_nhwc_f32";
+    PD_REQUIRE(N > 0 && H > 0 && W > 0 && C > 0 && K > 0, PD_ESHAPE, "%s: dimensions must be positive", who);
+    PD_REQUIRE(wino_wgrad_shape_ok(C, K), PD_ESHAPE, "%s: unsupported channel counts C=%d K=%d", who, C, K);
+    PD_REQUIRE((long)W * (C > K ? C : K) < (1L << 28), PD_ESHAPE, "%s: image row too large", who);
+    PD_REQUIRE(x && dy && dw && workspace, PD_EINVAL, "%s: NULL pointer", who);
+    PD_REQUIRE(pd_aligned(x, 16) && pd_aligned(dy, 16) && pd_aligned(workspace, 16), PD_EINVAL,
+               "%s: tensors must be 16-byte aligned", who);
+    uint64_t need = 0;
+    pd_conv3x3_winograd_wgrad_workspace_bytes(C, K, &need);
+    PD_REQUIRE(workspace_bytes >= need, PD_EINVAL, "%s: workspace too small (%llu < %llu bytes)", who,
+               (unsigned long long)workspace_bytes, (unsigned long long)need);
+    WinoWgradArgs a;
+    a.x = x; a.dy = dy;
+    a.N = N; a.H = H; a.W = W; a.C = C; a.K = K;
+    a.sx = (W + 2 * WW_TILES - 1) / (2 * WW_TILES);
+    a.sy = (H + 1) / 2;
+    const long strips = (long)N * a.sx * a.sy;
+    PD_REQUIRE(strips <= 0x7ffffff0L, PD_ESHAPE, "%s: too many strips", who);
+    a.n_strips = (int)strips;
+    a.c_blocks = C / 64;
+    a.n_pairs = a.c_blocks * (K / 64);
+    a.ranks = WW_BLOCKS / a.n_pairs;
+    a.strips_per_rank = (int)((strips + a.ranks - 1) / a.ranks);
+    float* ws = (float*)workspace;
+    a.part = ws;
+    a.part_db = ws + (size_t)WW_BLOCKS * WW_PART_FLOATS;
+    float* du = a.part_db + (size_t)WW_BLOCKS * 128;
+    float* dbsum = du + (size_t)a.n_pairs * WW_PART_FLOATS;
+    hipStream_t s = (hipStream_t)stream;
+    winograd_wgrad_kernel<<<WW_BLOCKS, WW_THREADS, 0, s>>>(a);
+    PD_CHECK_LAUNCH(who);
+    const long sum_threads = (long)a.n_pairs * (WW_PART_FLOATS / 4);
+    winograd_wgrad_sum_kernel<<<(unsigned)((sum_threads + 255) / 256), 256, 0, s>>>(a.part, a.part_db, du, dbsum,
+                                                                                   a.n_pairs, a.ranks);
+    PD_CHECK_LAUNCH(who);
+    winograd_wgrad_final_kernel<<<(unsigned)(((long)K * C + 255) / 256), 256, 0, s>>>(du, dbsum, dw, dbias, K, C,
+                                                                                     a.c_blocks);
+    PD_CHECK_LAUNCH(who);
+    return PD_OK;
+}

@@ -379,6 +379,15 @@ def conv3x3_weight_grad(x, dy, with_bias=True, relu_out=None):
         raise ValueError("conv3x3_weight_grad: x %s and dy %s disagree" % (tuple(x.shape), tuple(dy.shape)))
     lib = _cabi.lib()
     nbytes = ctypes.c_uint64()
+    if relu_out is None and _CONV_ALGO != "direct" and lib.pd_conv3x3_winograd_wgrad_supported(c, k):
+        lib.pd_conv3x3_winograd_wgrad_workspace_bytes(c, k, ctypes.byref(nbytes))
+        ws = torch.empty(nbytes.value, dtype=torch.uint8, device=x.device)
+        dw = torch.empty((k, c, 3, 3), dtype=torch.float32, device=x.device, memory_format=torch.channels_last)
+        db = torch.empty(k, dtype=torch.float32, device=x.device) if with_bias else None
+        with _timed("conv3x3_winograd_wgrad", 18.0 * c * k * n * h * wd):
+            lib.pd_conv3x3_winograd_wgrad_nhwc_f32(_ptr(x), _ptr(dy), _ptr(dw), _ptr(db), _ptr(ws), nbytes.value,
+                                                   n, h, wd, c, k, _cabi.stream_ptr())
+        return dw, db
     lib.pd_conv3x3_wgrad_workspace_bytes(n, h, wd, c, k, ctypes.byref(nbytes))
     ws = torch.empty(nbytes.value, dtype=torch.uint8, device=x.device)
     dw = torch.empty((k, c, 3, 3), dtype=torch.float32, device=x.device, memory_format=torch.channels_last)

@@ -73,6 +73,8 @@ SHAPES = [
     (1, 8, 8, 1, 1),
     (1, 20, 70, 17, 33),     # channel counts that are not multiples of the tile
     (3, 5, 6, 8, 8),         # C not a multiple of 4: scalar load path
+    (1, 64, 64, 7, 19),      # odd height and width: half tiles at the image edges (Winograd strips)
+    (3, 128, 64, 9, 40),
 ]
 
 
