@@ -557,6 +557,7 @@ constexpr int WW_RAW_OFF = 2 * WW_V_STAGE;
 constexpr int WW_LDS_FLOATS = WW_RAW_OFF + 2 * WW_RAW_STAGE;
 constexpr int WW_BLOCKS = 256;                       // persistent blocks: 8 dies x 32
 constexpr int WW_PART_FLOATS = WG_G * 64 * 64;       // one block's partial dU
+constexpr int WW_PART_STRIDE = WW_PART_FLOATS;       // floats between two blocks' partials
 
 struct WinoWgradArgs {
     const float* x;      // [N,H,W,C]
@@ -808,7 +809,7 @@ __global__ __launch_bounds__(WW_THREADS, 1) void winograd_wgrad_kernel(const Win
     }
 
     // ---- the block's sums: partial dU in [g][k][c] order, partial dbias per (tile half, k)
-    float* part = a.part + (size_t)(pair * a.ranks + rank) * WW_PART_FLOATS;
+    float* part = a.part + (size_t)(pair * a.ranks + rank) * WW_PART_STRIDE;
 #pragma unroll
     for (int g = 0; g < WG_GW; ++g)
 #pragma unroll
@@ -821,44 +822,68 @@ __global__ __launch_bounds__(WW_THREADS, 1) void winograd_wgrad_kernel(const Win
     if (gh == 0 && wn == 0) a.part_db[((size_t)(pair * a.ranks + rank) * 2 + h) * 64 + wm * 32 + cl] = db_acc;
 }
 
-// Sum of the ranks' partial dU (and partial dbias) of every pair, in rank order.
+constexpr int WW_SUM_GROUPS = 4;   // rank groups summed by different blocks (more loads in flight)
+
+// Sums of the ranks' partial dU (and partial dbias) of every pair: blockIdx.y picks a quarter of the
+// ranks, a thread owns four consecutive elements and keeps eight 16-byte loads in flight.  The order of
+// all additions is fixed.  du4 / db4: [group][pair][...].
 __global__ __launch_bounds__(256) void winograd_wgrad_sum_kernel(const float* __restrict__ part,
                                                                  const float* __restrict__ part_db,
-                                                                 float* __restrict__ du, float* __restrict__ dbsum,
+                                                                 float* __restrict__ du4, float* __restrict__ db4,
                                                                  int n_pairs, int ranks) {
     const int per_pair = WW_PART_FLOATS / 4;
+    const int grp = blockIdx.y, r0 = grp * ranks / WW_SUM_GROUPS, r1 = (grp + 1) * ranks / WW_SUM_GROUPS;
     const long id = (long)blockIdx.x * 256 + threadIdx.x;
     if (id < (long)n_pairs * per_pair) {
         const int pair = (int)(id / per_pair), i = (int)(id % per_pair);
-        const float4_t* src = (const float4_t*)part + (size_t)pair * ranks * per_pair + i;
-        float4_t s = {0.f, 0.f, 0.f, 0.f};
-        for (int r = 0; r < ranks; ++r) s += src[(size_t)r * per_pair];
-        ((float4_t*)du)[id] = s;
+        const float* src = part + (size_t)pair * ranks * WW_PART_STRIDE + (size_t)i * 4;
+        float4_t acc[8];
+#pragma unroll
+        for (int u = 0; u < 8; ++u) acc[u] = float4_t{0.f, 0.f, 0.f, 0.f};
+        for (int r = r0; r < r1; r += 8) {
+#pragma unroll
+            for (int u = 0; u < 8; ++u)
+                if (r + u < r1) acc[u] += *(const float4_t*)(src + (size_t)(r + u) * WW_PART_STRIDE);
+        }
+        ((float4_t*)du4)[(size_t)grp * n_pairs * per_pair + id] =
+            ((acc[0] + acc[1]) + (acc[2] + acc[3])) + ((acc[4] + acc[5]) + (acc[6] + acc[7]));
     }
     if (id < (long)n_pairs * 64) {
         const int pair = (int)(id / 64), k = (int)(id % 64);
-        float s = 0.f;
-        for (int r = 0; r < ranks * 2; ++r) s += part_db[((size_t)pair * ranks * 2 + r) * 64 + k];
-        dbsum[id] = s;
+        float sb[16];
+#pragma unroll
+        for (int u = 0; u < 16; ++u) sb[u] = 0.f;
+        for (int r = 2 * r0; r < 2 * r1; r += 16) {
+#pragma unroll
+            for (int u = 0; u < 16; ++u)
+                if (r + u < 2 * r1) sb[u] += part_db[((size_t)pair * ranks * 2 + r + u) * 64 + k];
+        }
+#pragma unroll
+        for (int w = 8; w >= 1; w >>= 1)
+#pragma unroll
+            for (int u = 0; u < w; ++u) sb[u] += sb[u + w];
+        db4[(size_t)grp * n_pairs * 64 + id] = sb[0];
     }
 }
 
 // dw[k][r][s][c] = (G^T dU[.][k][c] G)[r][s] with the signs of A's last row / column restored, and dbias.
-__global__ __launch_bounds__(256) void winograd_wgrad_final_kernel(const float* __restrict__ du,
-                                                                   const float* __restrict__ dbsum,
+__global__ __launch_bounds__(256) void winograd_wgrad_final_kernel(const float* __restrict__ du4,
+                                                                   const float* __restrict__ db4,
                                                                    float* __restrict__ dw, float* __restrict__ db,
-                                                                   int K, int C, int c_blocks) {
+                                                                   int K, int C, int c_blocks, int n_pairs) {
     const long id = (long)blockIdx.x * 256 + threadIdx.x;
     if (id >= (long)K * C) return;
     const int c = (int)(id % C), k = (int)(id / C);
     const int pair = (k / 64) * c_blocks + c / 64;
-    const float* src = du + (size_t)pair * WW_PART_FLOATS + (k % 64) * 64 + (c % 64);
+    const float* src = du4 + (size_t)pair * WW_PART_FLOATS + (k % 64) * 64 + (c % 64);
+    const size_t gstride = (size_t)n_pairs * WW_PART_FLOATS;
     float u[4][4];
 #pragma unroll
     for (int i = 0; i < 4; ++i)
 #pragma unroll
         for (int m = 0; m < 4; ++m) {
-            const float v = src[(i * 4 + m) * 64 * 64];
+            const float* e = src + (i * 4 + m) * 64 * 64;
+            const float v = (e[0] + e[gstride]) + (e[2 * gstride] + e[3 * gstride]);
             u[i][m] = ((i == 3) != (m == 3)) ? -v : v;
         }
     float t[4][3];
@@ -875,7 +900,11 @@ __global__ __launch_bounds__(256) void winograd_wgrad_final_kernel(const float* 
         out[(1 * 3 + s) * C] = 0.5f * (t[1][s] - t[2][s]);
         out[(2 * 3 + s) * C] = t[3][s] + 0.5f * (t[1][s] + t[2][s]);
     }
-    if (db && c == 0) db[k] = dbsum[(size_t)((k / 64) * c_blocks) * 64 + (k % 64)];
+    if (db && c == 0) {
+        const float* e = db4 + (size_t)((k / 64) * c_blocks) * 64 + (k % 64);
+        const size_t bs = (size_t)n_pairs * 64;
+        db[k] = (e[0] + e[bs]) + (e[2 * bs] + e[3 * bs]);
+    }
 }
 
 bool wino_wgrad_shape_ok(int C, int K) {
@@ -896,8 +925,8 @@ extern "C" int pd_conv3x3_winograd_wgrad_workspace_bytes(int C, int K, uint64_t*
                "pd_conv3x3_winograd_wgrad_workspace_bytes: needs C and K multiples of 64 with C*K/4096 a power "
                "of two <= 32 (C=%d K=%d)", C, K);
     const uint64_t pairs = (uint64_t)(C / 64) * (K / 64);
-    // per block: partial dU and 2 x 64 partial dbias; per pair: summed dU and dbias
-    *bytes = ((uint64_t)WW_BLOCKS * (WW_PART_FLOATS + 128) + pairs * (WW_PART_FLOATS + 64)) * sizeof(float);
+    // per block: partial dU and 2 x 64 partial dbias; per pair and rank group: summed dU and dbias
+    *bytes = ((uint64_t)WW_BLOCKS * (WW_PART_STRIDE + 128) + WW_SUM_GROUPS * pairs * (WW_PART_FLOATS + 64)) * sizeof(float);
     return PD_OK;
 }
 
@@ -929,18 +958,18 @@ extern "C" int pd_conv3x3_winograd_wgrad_nhwc_f32(const float* x, const float* d
     a.strips_per_rank = (int)((strips + a.ranks - 1) / a.ranks);
     float* ws = (float*)workspace;
     a.part = ws;
-    a.part_db = ws + (size_t)WW_BLOCKS * WW_PART_FLOATS;
+    a.part_db = ws + (size_t)WW_BLOCKS * WW_PART_STRIDE;
     float* du = a.part_db + (size_t)WW_BLOCKS * 128;
-    float* dbsum = du + (size_t)a.n_pairs * WW_PART_FLOATS;
+    float* dbsum = du + (size_t)WW_SUM_GROUPS * a.n_pairs * WW_PART_FLOATS;
     hipStream_t s = (hipStream_t)stream;
     winograd_wgrad_kernel<<<WW_BLOCKS, WW_THREADS, 0, s>>>(a);
     PD_CHECK_LAUNCH(who);
     const long sum_threads = (long)a.n_pairs * (WW_PART_FLOATS / 4);
-    winograd_wgrad_sum_kernel<<<(unsigned)((sum_threads + 255) / 256), 256, 0, s>>>(a.part, a.part_db, du, dbsum,
-                                                                                   a.n_pairs, a.ranks);
+    winograd_wgrad_sum_kernel<<<dim3((unsigned)((sum_threads + 255) / 256), WW_SUM_GROUPS), 256, 0, s>>>(
+        a.part, a.part_db, du, dbsum, a.n_pairs, a.ranks);
     PD_CHECK_LAUNCH(who);
     winograd_wgrad_final_kernel<<<(unsigned)(((long)K * C + 255) / 256), 256, 0, s>>>(du, dbsum, dw, dbias, K, C,
-                                                                                     a.c_blocks);
+                                                                                     a.c_blocks, a.n_pairs);
     PD_CHECK_LAUNCH(who);
     return PD_OK;
 }
