@@ -857,25 +857,34 @@ __global__ __launch_bounds__(CONV_THREADS, 2) void conv3x3_wgrad_smallc_kernel(c
         }
     }
 
-    const int part = blockIdx.x * 4 + wave;
-    float* pw = a.part_w + (size_t)part * a.K * NC;
-    if (idx < NC) {
+    // the four waves' sums (each covered a quarter of every tile's pixels) are added in wave order
+    // through the now idle dy tile, so the block writes one partial instead of four
+    __syncthreads();
 #pragma unroll
-        for (int t = 0; t < 2; ++t)
+    for (int t = 0; t < 2; ++t)
 #pragma unroll
-            for (int e = 0; e < 16; ++e) {
-                const int k = k0 + t * 32 + 8 * (e / 4) + 4 * h + (e % 4);
-                if (k < a.K) pw[(size_t)k * NC + idx] = acc[t][e];
-            }
+        for (int e = 0; e < 16; ++e) dy_tile[(wave * 32 + t * 16 + e) * 64 + lane] = acc[t][e];
+    float* bsum_tile = dy_tile + 4 * 32 * 64;
+#pragma unroll
+    for (int t = 0; t < 2; ++t) {
+        const float tot = bsum[t] + __shfl_xor(bsum[t], 32, 64);
+        if (h == 0) bsum_tile[wave * 64 + t * 32 + idx] = tot;
     }
-    if (a.part_b) {
+    __syncthreads();
+    float* pw = a.part_w + (size_t)blockIdx.x * a.K * NC;
 #pragma unroll
-        for (int t = 0; t < 2; ++t) {
-            const float tot = bsum[t] + __shfl_xor(bsum[t], 32, 64);
-            const int k = k0 + t * 32 + idx;
-            if (h == 0 && k < a.K) a.part_b[(size_t)part * a.K + k] = tot;
-        }
+    for (int it = 0; it < 32 * 64 / CONV_THREADS; ++it) {
+        const int id = tid + it * CONV_THREADS;          // (t, e, lane) of an accumulator element
+        const int te = id / 64, ln = id % 64;
+        const float v = (dy_tile[te * 64 + ln] + dy_tile[(32 + te) * 64 + ln]) +
+                        (dy_tile[(64 + te) * 64 + ln] + dy_tile[(96 + te) * 64 + ln]);
+        const int t = te / 16, e = te % 16, col = ln % 32;
+        const int k = k0 + t * 32 + 8 * (e / 4) + 4 * (ln / 32) + (e % 4);
+        if (col < NC && k < a.K) pw[(size_t)k * NC + col] = v;
     }
+    if (a.part_b && tid < 64 && k0 + tid < a.K)
+        a.part_b[(size_t)blockIdx.x * a.K + k0 + tid] =
+            (bsum_tile[tid] + bsum_tile[64 + tid]) + (bsum_tile[128 + tid] + bsum_tile[192 + tid]);
 }
 
 // out[i] = sum_b part[b][i] in a fixed order (deterministic).  A block owns 64 outputs;
@@ -1009,9 +1018,8 @@ extern "C" int pd_conv3x3_wgrad_workspace_bytes(int N, int H, int W, int C, int 
     int rc = check_dims("pd_conv3x3_wgrad_workspace_bytes", N, H, W, C, K);
     if (rc != PD_OK) return rc;
     PD_REQUIRE(bytes != nullptr, PD_EINVAL, "pd_conv3x3_wgrad_workspace_bytes: NULL pointer");
-    // the few-channel kernel writes one partial per wave (4 per block)
-    // partial sums per pixel-range block: 4 in the few-channel kernel (one per wave), 2 in the pipelined one
-    const uint64_t nb = (uint64_t)wgrad_blocks(N, H, W, C, K) * (9 * C <= 32 ? 4 : 2);
+    // partial sums per pixel-range block: 1 in the few-channel kernel, 2 in the pipelined one
+    const uint64_t nb = (uint64_t)wgrad_blocks(N, H, W, C, K) * (9 * C <= 32 ? 1 : 2);
     *bytes = nb * ((uint64_t)K * 9 * C + (uint64_t)K) * sizeof(float);
     return PD_OK;
 }
@@ -1036,7 +1044,7 @@ extern "C" int pd_conv3x3_wgrad_nhwc_f32(const float* x, const float* dy, const 
     const bool small_c = 9 * C <= 32;
     const int nblk = wgrad_blocks(N, H, W, C, K);
     const bool vec = (C % 4 == 0) && pd_aligned(x, 16) && (K % 4 == 0) && pd_aligned(dy, 16) && (!relu_out || pd_aligned(relu_out, 16));
-    const int nb = nblk * (small_c ? 4 : (vec ? 2 : 1));     // number of partial sums
+    const int nb = nblk * (small_c ? 1 : (vec ? 2 : 1));     // number of partial sums
     a.part_w = (float*)workspace;
     a.part_b = dbias ? a.part_w + (size_t)nb * K * 9 * C : nullptr;
     a.c_vec = (C % 4 == 0) && pd_aligned(x, 16);
