@@ -572,22 +572,24 @@ struct WinoWgradArgs {
 
 struct StripPos { int n, y0, x0; };
 
+// Strips are numbered down the image first (row pair fastest), then across, then over images: a block's
+// consecutive strips share two of their four input rows, which the second one finds in cache.
 __device__ __forceinline__ StripPos strip_decode(const WinoWgradArgs& a, int s) {
     StripPos p;
     const int per_img = a.sx * a.sy;
     p.n = s / per_img;
     const int rem = s - p.n * per_img;
-    const int ty = rem / a.sx;
-    p.y0 = 2 * ty;
-    p.x0 = (rem - ty * a.sx) * (2 * WW_TILES);
+    const int tx = rem / a.sy;
+    p.x0 = tx * (2 * WW_TILES);
+    p.y0 = 2 * (rem - tx * a.sy);
     return p;
 }
 __device__ __forceinline__ void strip_next(const WinoWgradArgs& a, StripPos& p) {
-    p.x0 += 2 * WW_TILES;
-    if (p.x0 >= a.W) {
-        p.x0 = 0;
-        p.y0 += 2;
-        if (p.y0 >= a.H) { p.y0 = 0; ++p.n; }
+    p.y0 += 2;
+    if (p.y0 >= a.H) {
+        p.y0 = 0;
+        p.x0 += 2 * WW_TILES;
+        if (p.x0 >= a.W) { p.x0 = 0; ++p.n; }
     }
 }
 
