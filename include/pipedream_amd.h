@@ -216,7 +216,7 @@ int pd_conv3x3_winograd_fwd_nhwc_f32(const float* x, const float* u, const float
 /* Weight (and optional bias) gradient of the same convolution in the Winograd domain: sums
  * dU = sum over 2x2 output tiles of (A dY A^T) (B^T d B) in persistent blocks, adds the blocks' partial
  * sums in fixed order and applies G^T . G.  Deterministic; agrees with pd_conv3x3_wgrad_nhwc_f32 to
- * fp32 rounding.  Needs C and K multiples of 64 with (C/64)*(K/64) a power of two <= 32
+ * fp32 rounding.  Needs C and K multiples of 64 with (C/64)*(K/64) a power of two <= 256
  * (pd_conv3x3_winograd_wgrad_supported() returns 1) and a workspace of
  * pd_conv3x3_winograd_wgrad_workspace_bytes() bytes.  dw is [K][3][3][C]; dbias may be NULL.
  * (Backward of torch.nn.Conv2d, vgg16/gpus=4_straight/stage0.py:12-14.) */

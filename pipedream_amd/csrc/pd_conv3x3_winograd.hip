@@ -600,9 +600,15 @@ __global__ __launch_bounds__(WW_THREADS, 1) void winograd_wgrad_kernel(const Win
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     // block -> (pair, rank): the 32 blocks of a die cover all pairs of a contiguous strip range, so the
     // pairs that read the same x and dY strips run side by side on one L2
-    const int xcd = blockIdx.x % WG_XCD, slot = blockIdx.x / WG_XCD;
-    const int pair = slot % a.n_pairs, sub = slot / a.n_pairs;
-    const int rank = xcd * (32 / a.n_pairs) + sub;
+    int pair, rank;
+    if (a.n_pairs <= 32) {
+        const int xcd = blockIdx.x % WG_XCD, slot = blockIdx.x / WG_XCD;
+        pair = slot % a.n_pairs;
+        rank = xcd * (32 / a.n_pairs) + slot / a.n_pairs;
+    } else {                                   // more pairs than a die has blocks: plain round robin
+        pair = blockIdx.x % a.n_pairs;
+        rank = blockIdx.x / a.n_pairs;
+    }
     const int kb = pair / a.c_blocks, cb = pair % a.c_blocks;
     const int s_begin = rank * a.strips_per_rank;
     int s_end = s_begin + a.strips_per_rank;
@@ -912,7 +918,7 @@ __global__ __launch_bounds__(256) void winograd_wgrad_final_kernel(const float* 
 bool wino_wgrad_shape_ok(int C, int K) {
     if (C % 64 != 0 || K % 64 != 0) return false;
     const int pairs = (C / 64) * (K / 64);
-    return pairs <= 32 && (pairs & (pairs - 1)) == 0;
+    return pairs <= WW_BLOCKS && (pairs & (pairs - 1)) == 0;
 }
 
 }  // namespace
@@ -925,7 +931,7 @@ extern "C" int pd_conv3x3_winograd_wgrad_workspace_bytes(int C, int K, uint64_t*
     PD_REQUIRE(bytes != nullptr, PD_EINVAL, "pd_conv3x3_winograd_wgrad_workspace_bytes: NULL pointer");
     PD_REQUIRE(C > 0 && K > 0 && wino_wgrad_shape_ok(C, K), PD_ESHAPE,
                "pd_conv3x3_winograd_wgrad_workspace_bytes: needs C and K multiples of 64 with C*K/4096 a power "
-               "of two <= 32 (C=%d K=%d)", C, K);
+               "of two <= 256 (C=%d K=%d)", C, K);
     const uint64_t pairs = (uint64_t)(C / 64) * (K / 64);
     // per block: partial dU and 2 x 64 partial dbias; per pair and rank group: summed dU and dbias
     *bytes = ((uint64_t)WW_BLOCKS * (WW_PART_STRIDE + 128) + WW_SUM_GROUPS * pairs * (WW_PART_FLOATS + 64)) * sizeof(float);

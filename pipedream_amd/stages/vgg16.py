@@ -71,13 +71,17 @@ class Stage0(torch.nn.Module):
 
 
 class Stage1(torch.nn.Module):
+    """Stage 1 of the 4-way split.  Its last ReLU's backward is applied by ``Stage2`` (the first convolution
+    there masks its input gradient), so the gradient this stage receives must come from ``Stage2``."""
+
     def __init__(self):
         super(Stage1, self).__init__()
         self.layer2 = layers.MaxPool2d(2, 2, relu=True)    # layer1 ReLU + layer2 MaxPool
         self.layer3 = layers.Conv2d(64, 128, relu=True, grad_premasked=True)    # + layer4; masked by layer5
         self.layer5 = layers.Conv2d(128, 128, relu=True, grad_premasked=True, input_rectified=True)   # + layer6; masked by layer7
         self.layer7 = layers.MaxPool2d(2, 2, relu=True)
-        self.layer8 = layers.Conv2d(128, 256, relu=True)   # + layer9
+        # layer8's ReLU is undone for the gradient by the next stage's first convolution (input_rectified)
+        self.layer8 = layers.Conv2d(128, 256, relu=True, grad_premasked=True)   # + layer9
         _initialize_weights(self)
 
     def forward(self, input0):
@@ -87,14 +91,18 @@ class Stage1(torch.nn.Module):
 
 
 class Stage2(torch.nn.Module):
+    """Stage 2 of the 4-way split.  Takes ``Stage1``'s rectified output; its last ReLU's backward is applied
+    by the pooling layer that opens ``Stage3``."""
+
     def __init__(self):
         super(Stage2, self).__init__()
-        self.layer1 = layers.Conv2d(256, 256, relu=True, grad_premasked=True)   # + layer2; masked by layer3
+        self.layer1 = layers.Conv2d(256, 256, relu=True, grad_premasked=True, input_rectified=True)   # + layer2; masked by layer3
         self.layer3 = layers.Conv2d(256, 256, relu=True, grad_premasked=True, input_rectified=True)   # + layer4; masked by layer5
         self.layer5 = layers.MaxPool2d(2, 2, relu=True)
         self.layer6 = layers.Conv2d(256, 512, relu=True, grad_premasked=True)   # + layer7; masked by layer8
         self.layer8 = layers.Conv2d(512, 512, relu=True, grad_premasked=True, input_rectified=True)   # + layer9
-        self.layer10 = layers.Conv2d(512, 512, relu=True, input_rectified=True)  # + layer11
+        # layer10's ReLU is undone for the gradient by the next stage's pooling layer (relu=True)
+        self.layer10 = layers.Conv2d(512, 512, relu=True, grad_premasked=True, input_rectified=True)  # + layer11
         _initialize_weights(self)
 
     def forward(self, input0):
@@ -106,7 +114,7 @@ class Stage2(torch.nn.Module):
 class Stage3(torch.nn.Module):
     def __init__(self, dropout=0.5, num_classes=1000):
         super(Stage3, self).__init__()
-        self.layer1 = layers.MaxPool2d(2, 2)
+        self.layer1 = layers.MaxPool2d(2, 2, relu=True)
         self.layer2 = layers.Conv2d(512, 512, relu=True, grad_premasked=True)   # + layer3; masked by layer4
         self.layer4 = layers.Conv2d(512, 512, relu=True, grad_premasked=True, input_rectified=True)   # + layer5
         self.layer6 = layers.Conv2d(512, 512, relu=True, grad_premasked=True, input_rectified=True)   # + layer7; masked by layer8
