@@ -617,11 +617,11 @@ __global__ __launch_bounds__(WW_THREADS, 1) void winograd_wgrad_kernel(const Win
 
     // ---- stage 1 role: pieces p = tid + 512 j of the patch: row p / 320 (uniform in a wave), pixel
     //      (p % 320) / 16 (pixels 18, 19 are padding of the piece grid), channels 4 (p % 16) .. +3.
-    //      A patch row is read through its own buffer descriptor that starts one pixel left of the
-    //      strip and ends with the image row, so columns beyond the image read 0; the column left of
-    //      the image (first strip of a row) is switched off per lane; rows outside the image get an
-    //      empty descriptor.
-    uint32_t xoff[3], xoff_first[3];
+    //      A patch row is read through its own buffer descriptor over that image row (this block's 64
+    //      channels onwards): the pixel offset (x0 - 1 + pixel) * C is negative left of the image, which
+    //      as an unsigned offset lies beyond the descriptor's size like the columns right of the image,
+    //      so both read 0; rows outside the image get an empty descriptor.
+    uint32_t xoff[3];
     int raw_dst[3], prow[3];
     bool live[3];
 #pragma unroll
@@ -630,21 +630,20 @@ __global__ __launch_bounds__(WW_THREADS, 1) void winograd_wgrad_kernel(const Win
         prow[j] = __builtin_amdgcn_readfirstlane(p / WW_ROW_PIECES);
         const int rem = p % WW_ROW_PIECES, ppx = rem >> 4, pcg = rem & 15;
         live[j] = ppx < WW_PATCH_W && p < 4 * WW_ROW_PIECES;
-        xoff[j] = live[j] ? (uint32_t)((ppx * a.C + pcg * 4) * 4) : 0x80000000u;
-        xoff_first[j] = ppx == 0 ? 0x80000000u : xoff[j];
+        xoff[j] = live[j] ? (uint32_t)(((ppx - 1) * a.C + pcg * 4) * 4) : 0x80000000u;
         raw_dst[j] = ((prow[j] & 3) * WW_PATCH_W + (live[j] ? ppx : 0)) * 64 + pcg * 4;
     }
     float4_t rawr[3];
     auto load_raw = [&](const StripPos& p, bool valid) {
+        const uint32_t strip_off = (uint32_t)(p.x0 * a.C) * 4;
 #pragma unroll
         for (int j = 0; j < 3; ++j) {
             const int gy = p.y0 - 1 + prow[j];
             const bool row_ok = valid && gy >= 0 && gy < a.H && (j < 2 || wave < 4);
-            const float* base = a.x + (((size_t)p.n * a.H + gy) * a.W + p.x0 - 1) * a.C + cb * 64;
-            const uint32_t bytes = row_ok ? (uint32_t)((a.W - p.x0 + 1) * a.C - cb * 64) * 4 : 0u;
+            const float* base = a.x + ((size_t)(row_ok ? p.n : 0) * a.H + (row_ok ? gy : 0)) * a.W * a.C + cb * 64;
+            const uint32_t bytes = row_ok ? (uint32_t)(a.W * a.C - cb * 64) * 4 : 0u;
             const __amdgpu_buffer_rsrc_t r = __builtin_amdgcn_make_buffer_rsrc((void*)base, 0, bytes, 0x00020000);
-            rawr[j] = __builtin_bit_cast(
-                float4_t, __builtin_amdgcn_raw_buffer_load_b128(r, p.x0 == 0 ? xoff_first[j] : xoff[j], 0, 0));
+            rawr[j] = __builtin_bit_cast(float4_t, __builtin_amdgcn_raw_buffer_load_b128(r, xoff[j] + strip_off, 0, 0));
         }
     };
     auto store_raw = [&](int stage, int j) {
@@ -690,7 +689,8 @@ __global__ __launch_bounds__(WW_THREADS, 1) void winograd_wgrad_kernel(const Win
 #pragma unroll
         for (int r = 0; r < 2; ++r) {
             const bool row_ok = valid && p.y0 + r < a.H;
-            const float* base = a.dy + (((size_t)p.n * a.H + p.y0 + r) * a.W + p.x0) * a.K;
+            const float* base =
+                a.dy + (row_ok ? (((size_t)p.n * a.H + p.y0 + r) * a.W + p.x0) * a.K : (size_t)0);
             const uint32_t bytes = row_ok ? (uint32_t)((a.W - p.x0) * a.K) * 4 : 0u;
             const __amdgpu_buffer_rsrc_t rs = __builtin_amdgcn_make_buffer_rsrc((void*)base, 0, bytes, 0x00020000);
 #pragma unroll
