@@ -342,17 +342,38 @@ __global__ __launch_bounds__(CONV_THREADS, 2) void conv3x3_fwd_smallc_kernel(con
     const int y0 = ty * TH, x0 = tx * TW;
     const float* xn = a.x + (size_t)n * a.H * a.W * C;
 
-    // stage the halo tile ([pixel][4], zero padded) and the filter ([k][27 -> 32])
-    for (int id = tid; id < HALO * 4; id += CONV_THREADS) {
+    // stage the halo tile ([pixel][4], zero padded) and the filter ([k][27 -> 32]): all global loads
+    // are issued before the first LDS store, so a block waits for memory once, not once per element
+    constexpr int IN_ITERS = (HALO * 4 + CONV_THREADS - 1) / CONV_THREADS;
+    constexpr int W_ITERS = BN * 32 / CONV_THREADS;
+    float rin[IN_ITERS], rw[W_ITERS];
+#pragma unroll
+    for (int it = 0; it < IN_ITERS; ++it) {
+        const int id = tid + it * CONV_THREADS;
         const int p = id / 4, cc = id % 4;
         const int gy = y0 + p / HW_ - 1, gx = x0 + p % HW_ - 1;
-        const bool ok = cc < C && gy >= 0 && gy < a.H && gx >= 0 && gx < a.W;
-        in_tile[id] = ok ? xn[((size_t)gy * a.W + gx) * C + cc] : 0.f;
+        const bool ok = id < HALO * 4 && cc < C && gy >= 0 && gy < a.H && gx >= 0 && gx < a.W;
+        const float v = xn[ok ? ((size_t)gy * a.W + gx) * C + cc : 0];
+        rin[it] = ok ? v : 0.f;
+    }
+#pragma unroll
+    for (int it = 0; it < W_ITERS; ++it) {
+        const int id = tid + it * CONV_THREADS;
+        const int k = id / 32, kk = id % 32;
+        const bool ok = kk < NC && k0 + k < a.K;
+        const float v = a.w[ok ? (size_t)(k0 + k) * NC + kk : 0];
+        rw[it] = ok ? v : 0.f;
+    }
+#pragma unroll
+    for (int it = 0; it < IN_ITERS; ++it) {
+        const int id = tid + it * CONV_THREADS;
+        if (id < HALO * 4) in_tile[id] = rin[it];
     }
     if (tid < 4) in_tile[HALO * 4 + tid] = 0.f;
-    for (int id = tid; id < BN * 32; id += CONV_THREADS) {
-        const int k = id / 32, kk = id % 32;
-        w_tile[k * WP + kk] = (kk < NC && k0 + k < a.K) ? a.w[(size_t)(k0 + k) * NC + kk] : 0.f;
+#pragma unroll
+    for (int it = 0; it < W_ITERS; ++it) {
+        const int id = tid + it * CONV_THREADS;
+        w_tile[(id / 32) * WP + id % 32] = rw[it];
     }
     // per-lane gather offsets for the reduction indices kk = 8g + 4h + s
     int goff[4][4];
