@@ -801,7 +801,16 @@ __global__ __launch_bounds__(CONV_THREADS, 2) void conv3x3_wgrad_smallc_kernel(c
     float bsum[2] = {0.f, 0.f};
     if (tid == 0) x_tile[HALO * 4] = 0.f;
 
-    for (int tile = blockIdx.x; tile < a.n_tiles; tile += gridDim.x) {
+    constexpr int DY_ITERS = PIX * (CS / 4) / CONV_THREADS;
+    constexpr int X_ITERS = (HALO * 4 + CONV_THREADS - 1) / CONV_THREADS;
+    float4_t rdy[DY_ITERS];
+    float rx[X_ITERS];
+    uint32_t dy_ok = 0, x_ok = 0;              // which of them lie inside the image
+    // global -> registers for one pixel tile; the loads of tile i+1 are issued before the multiply
+    // loop of tile i and stay in flight over it (out-of-range elements read a safe address and are
+    // zeroed when the registers are written to LDS: a select here would wait for the loads)
+    auto load_tile = [&](int tile) {
+        dy_ok = x_ok = 0;
         int b = tile;
         const int tx = b % a.tiles_x;
         b /= a.tiles_x;
@@ -811,10 +820,6 @@ __global__ __launch_bounds__(CONV_THREADS, 2) void conv3x3_wgrad_smallc_kernel(c
         const float* xn = a.x + (size_t)n * a.H * a.W * C;
         const float* dyn = a.dy + (size_t)n * a.H * a.W * a.K;
         const float* mn = a.mask ? a.mask + (size_t)n * a.H * a.W * a.K : nullptr;
-
-        constexpr int DY_ITERS = PIX * (CS / 4) / CONV_THREADS;
-        const float4_t zero = {0.f, 0.f, 0.f, 0.f};
-        float4_t rdy[DY_ITERS];
 #pragma unroll
         for (int it = 0; it < DY_ITERS; ++it) {
             const int id = tid + it * CONV_THREADS;
@@ -841,29 +846,36 @@ __global__ __launch_bounds__(CONV_THREADS, 2) void conv3x3_wgrad_smallc_kernel(c
 #pragma unroll
                 for (int j = 0; j < 4; ++j) v[j] = m[j] > 0.f ? v[j] : 0.f;
             }
-            rdy[it] = ok ? v : zero;
+            rdy[it] = v;
+            dy_ok |= (uint32_t)ok << it;
         }
-        float rx[(HALO * 4 + CONV_THREADS - 1) / CONV_THREADS];
 #pragma unroll
-        for (int it = 0; it < (HALO * 4 + CONV_THREADS - 1) / CONV_THREADS; ++it) {
+        for (int it = 0; it < X_ITERS; ++it) {
             const int id = tid + it * CONV_THREADS;
             const int p = id / 4, cc = id % 4;
             const int gy = y0 + p / HW_ - 1, gx = x0 + p % HW_ - 1;
             const bool ok = id < HALO * 4 && cc < C && gy >= 0 && gy < a.H && gx >= 0 && gx < a.W;
-            rx[it] = ok ? xn[((size_t)gy * a.W + gx) * C + cc] : 0.f;
+            rx[it] = xn[ok ? ((size_t)gy * a.W + gx) * C + cc : 0];
+            x_ok |= (uint32_t)ok << it;
         }
+    };
+    if ((int)blockIdx.x < a.n_tiles) load_tile(blockIdx.x);
+
+    for (int tile = blockIdx.x; tile < a.n_tiles; tile += gridDim.x) {
         __syncthreads();  // previous tile fully consumed
 #pragma unroll
         for (int it = 0; it < DY_ITERS; ++it) {
             const int id = tid + it * CONV_THREADS;
-            *(float4_t*)(dy_tile + (id / (CS / 4)) * CS + (id % (CS / 4)) * 4) = rdy[it];
+            const float4_t zero = {0.f, 0.f, 0.f, 0.f};
+            *(float4_t*)(dy_tile + (id / (CS / 4)) * CS + (id % (CS / 4)) * 4) = (dy_ok >> it) & 1 ? rdy[it] : zero;
         }
 #pragma unroll
-        for (int it = 0; it < (HALO * 4 + CONV_THREADS - 1) / CONV_THREADS; ++it) {
+        for (int it = 0; it < X_ITERS; ++it) {
             const int id = tid + it * CONV_THREADS;
-            if (id < HALO * 4) x_tile[id] = rx[it];
+            if (id < HALO * 4) x_tile[id] = (x_ok >> it) & 1 ? rx[it] : 0.f;
         }
         __syncthreads();
+        if (tile + (int)gridDim.x < a.n_tiles) load_tile(tile + gridDim.x);
         // this wave's quarter of the pixels, two per MFMA
 #pragma unroll 4
         for (int pp = 0; pp < PIX / 8; ++pp) {
