@@ -158,8 +158,17 @@ def test_full_vgg16_four_stage_pipeline_matches_oracle():
             assert err <= tol, (si, key, err, tol)
 
 
-def test_full_size_conv_properties():
-    """Batch 64, 224x224, 64 -> 64 channels (the heaviest layer of the benchmark stage)."""
+@pytest.fixture(params=["direct", "winograd"])
+def conv_algorithm(request):
+    from pipedream_amd import ops
+    ops.set_conv_algorithm(request.param)
+    yield request.param
+    ops.set_conv_algorithm("auto")
+
+
+def test_full_size_conv_properties(conv_algorithm):
+    """Batch 64, 224x224, 64 -> 64 channels (the heaviest layer of the benchmark stage), under the direct and
+    the Winograd kernels: size-independent identities instead of an oracle run."""
     from pipedream_amd import ops
     gen = torch.Generator(device="cuda").manual_seed(0)
     x = torch.randn(64, 64, 224, 224, device="cuda", generator=gen).contiguous(memory_format=torch.channels_last)
@@ -187,3 +196,12 @@ def test_full_size_conv_properties():
     k[0, 0] = 1
     cnt = ops.conv3x3_forward(ones, k.contiguous(memory_format=torch.channels_last))[0, 0]
     assert cnt[0, 0] == 4 and cnt[0, 3] == 6 and cnt[3, 3] == 9 and cnt[7, 7] == 4
+    if conv_algorithm == "winograd":
+        # the two algorithms agree to fp32 rounding at full size (outputs are O(1): 576-term sums of N(0,1)/24)
+        del dx, dw
+        ops.set_conv_algorithm("direct")
+        y_direct = ops.conv3x3_forward(x, w)
+        assert float((y - y_direct).abs().max()) < 2e-5
+        dw_w, _ = (ops.set_conv_algorithm("winograd"), ops.conv3x3_weight_grad(x, dy))[1]
+        dw_d, _ = (ops.set_conv_algorithm("direct"), ops.conv3x3_weight_grad(x, dy))[1]
+        assert float((dw_w - dw_d).abs().max()) <= 1e-5 * float(dw_d.abs().max())
