@@ -409,7 +409,9 @@ __global__ __launch_bounds__(WG_THREADS, 1) void winograd_fwd_kernel(const WinoA
                     for (int i = 0; i < 4; ++i) prev[i] = add ? stg_lane[stg_index(e, i)] : 0.f;
 #pragma unroll
                     for (int i = 0; i < 4; ++i) stg_lane[stg_index(e, i)] = prev[i] + part[i];
-                    __builtin_amdgcn_sched_barrier(0);
+                    // four rows at a time may overlap (their chains of additions and LDS round trips are
+                    // independent); more would need more registers than a wave has left here
+                    if ((e & 3) == 3) __builtin_amdgcn_sched_barrier(0);
                 }
             };
             if (gh == 0) out_rows(false);
