@@ -38,6 +38,7 @@ struct GemmArgs {
     int a_vec, b_vec;   // 128-bit global loads allowed for A / B
     int k_per_split;    // blockIdx.z owns k in [z*k_per_split, (z+1)*k_per_split) and writes C + z*c_split
     long long c_split;  // elements between the partial results of consecutive splits
+    uint32_t a_bytes, b_bytes;  // extents of A and B for the fast path's buffer descriptors (0 = fast path off)
 };
 
 // Operand tile in LDS.  KC (k-contiguous): [ROWS][BK+4]; otherwise [BK][ROWS+4].
@@ -92,6 +93,25 @@ struct Tile {
         }
     }
 
+    // Fast path for full tiles of 16-byte-aligned operands: per-thread byte offsets of the chunk at k = 0
+    // (computed once), the chunk's k offset goes into the scalar offset of a buffer load, so the inner
+    // loop spends no vector instructions on addresses or bounds.
+    __device__ static void offsets(uint32_t (&off)[VEC_PER_THREAD], int ld, int row0, int tid) {
+#pragma unroll
+        for (int v = 0; v < VEC_PER_THREAD; ++v) {
+            const int id = tid + v * GEMM_THREADS;
+            if (KC) off[v] = (uint32_t)((row0 + id / (BK / 4)) * ld + (id % (BK / 4)) * 4) * 4;
+            else off[v] = (uint32_t)((id / (ROWS / 4)) * ld + row0 + (id % (ROWS / 4)) * 4) * 4;
+        }
+    }
+    __device__ static void load_fast(float4_t (&r)[VEC_PER_THREAD], __amdgpu_buffer_rsrc_t rs,
+                                     const uint32_t (&off)[VEC_PER_THREAD], int ld, int k) {
+        const int soff = (KC ? k : k * ld) * 4;
+#pragma unroll
+        for (int v = 0; v < VEC_PER_THREAD; ++v)
+            r[v] = __builtin_bit_cast(float4_t, __builtin_amdgcn_raw_buffer_load_b128(rs, off[v], soff, 0));
+    }
+
     __device__ static void store(float* lds, const float4_t (&r)[VEC_PER_THREAD], int tid) {
 #pragma unroll
         for (int v = 0; v < VEC_PER_THREAD; ++v) {
@@ -123,7 +143,7 @@ struct Tile {
     }
 };
 
-template <int BM, int BN, bool A_KC, bool B_KC>
+template <int BM, int BN, bool A_KC, bool B_KC, bool FULL>
 __global__ __launch_bounds__(GEMM_THREADS) void pd_gemm_f32_kernel(const GemmArgs a) {
     constexpr int TM = BM / 64, TN = BN / 64;  // MFMA tiles per wave in m / n
     using TA = Tile<BM, A_KC>;
@@ -150,8 +170,18 @@ __global__ __launch_bounds__(GEMM_THREADS) void pd_gemm_f32_kernel(const GemmArg
     const int k_end = min(a.K, k_begin + a.k_per_split);
     const int nk = (k_end - k_begin + BK - 1) / BK;
     float* const C = a.C + blockIdx.z * a.c_split;
-    TA::load(ra, a.A, a.lda, m0, k_begin, a.M, k_end, a.a_vec, tid);
-    TB::load(rb, a.B, a.ldb, n0, k_begin, a.N, k_end, a.b_vec, tid);
+    uint32_t oa[TA::VEC_PER_THREAD], ob[TB::VEC_PER_THREAD];
+    const __amdgpu_buffer_rsrc_t rsa = __builtin_amdgcn_make_buffer_rsrc((void*)a.A, 0, a.a_bytes, 0x00020000);
+    const __amdgpu_buffer_rsrc_t rsb = __builtin_amdgcn_make_buffer_rsrc((void*)a.B, 0, a.b_bytes, 0x00020000);
+    if (FULL) {
+        TA::offsets(oa, a.lda, m0, tid);
+        TB::offsets(ob, a.ldb, n0, tid);
+        TA::load_fast(ra, rsa, oa, a.lda, k_begin);
+        TB::load_fast(rb, rsb, ob, a.ldb, k_begin);
+    } else {
+        TA::load(ra, a.A, a.lda, m0, k_begin, a.M, k_end, a.a_vec, tid);
+        TB::load(rb, a.B, a.ldb, n0, k_begin, a.N, k_end, a.b_vec, tid);
+    }
     TA::store(lds_a[0], ra, tid);
     TB::store(lds_b[0], rb, tid);
     __syncthreads();
@@ -159,8 +189,13 @@ __global__ __launch_bounds__(GEMM_THREADS) void pd_gemm_f32_kernel(const GemmArg
     for (int kt = 0; kt < nk; ++kt) {
         const int cur = kt & 1;
         if (kt + 1 < nk) {  // prefetch the next chunk into registers while this one is multiplied
-            TA::load(ra, a.A, a.lda, m0, k_begin + (kt + 1) * BK, a.M, k_end, a.a_vec, tid);
-            TB::load(rb, a.B, a.ldb, n0, k_begin + (kt + 1) * BK, a.N, k_end, a.b_vec, tid);
+            if (FULL) {
+                TA::load_fast(ra, rsa, oa, a.lda, k_begin + (kt + 1) * BK);
+                TB::load_fast(rb, rsb, ob, a.ldb, k_begin + (kt + 1) * BK);
+            } else {
+                TA::load(ra, a.A, a.lda, m0, k_begin + (kt + 1) * BK, a.M, k_end, a.a_vec, tid);
+                TB::load(rb, a.B, a.ldb, n0, k_begin + (kt + 1) * BK, a.N, k_end, a.b_vec, tid);
+            }
         }
 #pragma unroll
         for (int g = 0; g < BK / 8; ++g) {
@@ -190,12 +225,12 @@ __global__ __launch_bounds__(GEMM_THREADS) void pd_gemm_f32_kernel(const GemmArg
 #pragma unroll
         for (int j = 0; j < TN; ++j) {
             const int col = n0 + wn * (BN / 2) + j * 32 + idx;
-            if (col >= a.N) continue;
+            if (!FULL && col >= a.N) continue;
             const float bv = a.bias ? a.bias[col] : 0.f;
 #pragma unroll
             for (int e = 0; e < 16; ++e) {
                 const int row = m0 + wm * (BM / 2) + i * 32 + 8 * (e / 4) + 4 * h + (e % 4);
-                if (row >= a.M) continue;
+                if (!FULL && row >= a.M) continue;
                 float* p = C + (size_t)row * a.ldc + col;
                 float v = acc[i][j][e] + bv;
                 if (a.beta != 0.f) v += a.beta * *p;
@@ -209,10 +244,20 @@ template <int BM, int BN>
 int launch_gemm(int trans_a, int trans_b, const GemmArgs& g, hipStream_t s, int splits = 1) {
     dim3 grid((g.N + BN - 1) / BN, (g.M + BM - 1) / BM, splits);
     // A is k-contiguous when it is NOT transposed; B (stored [K][N]) is k-contiguous when it IS.
-    if (!trans_a && trans_b) pd_gemm_f32_kernel<BM, BN, true, true><<<grid, GEMM_THREADS, 0, s>>>(g);
-    else if (!trans_a && !trans_b) pd_gemm_f32_kernel<BM, BN, true, false><<<grid, GEMM_THREADS, 0, s>>>(g);
-    else if (trans_a && !trans_b) pd_gemm_f32_kernel<BM, BN, false, false><<<grid, GEMM_THREADS, 0, s>>>(g);
-    else pd_gemm_f32_kernel<BM, BN, false, true><<<grid, GEMM_THREADS, 0, s>>>(g);
+    // Full tiles of aligned operands whose extents fit a 32-bit byte offset take the fast loader.
+    const int k_span = splits > 1 ? g.k_per_split : g.K;
+    const bool full = g.M % BM == 0 && g.N % BN == 0 && k_span % BK == 0 && g.K % BK == 0 && g.a_vec && g.b_vec &&
+                      g.a_bytes != 0 && g.b_bytes != 0;
+#define PD_GEMM_LAUNCH(AKC, BKC)                                                                 \
+    do {                                                                                          \
+        if (full) pd_gemm_f32_kernel<BM, BN, AKC, BKC, true><<<grid, GEMM_THREADS, 0, s>>>(g);    \
+        else pd_gemm_f32_kernel<BM, BN, AKC, BKC, false><<<grid, GEMM_THREADS, 0, s>>>(g);        \
+    } while (0)
+    if (!trans_a && trans_b) PD_GEMM_LAUNCH(true, true);
+    else if (!trans_a && !trans_b) PD_GEMM_LAUNCH(true, false);
+    else if (trans_a && !trans_b) PD_GEMM_LAUNCH(false, false);
+    else PD_GEMM_LAUNCH(false, true);
+#undef PD_GEMM_LAUNCH
     PD_CHECK_LAUNCH("pd_gemm_f32");
     return PD_OK;
 }
@@ -443,6 +488,13 @@ __global__ __launch_bounds__(256) void splitk_reduce_kernel(const float* __restr
 
 }  // namespace
 
+// Byte extent of an operand with `rows` rows of leading dimension `ld`, or 0 if it does not fit the 32-bit
+// offsets of the fast loader.
+static uint32_t operand_bytes(long rows, long ld) {
+    const long b = rows * ld * 4;
+    return b < (1L << 31) ? (uint32_t)b : 0u;
+}
+
 extern "C" int pd_gemm_f32(int trans_a, int trans_b, int M, int N, int K, const float* A, int lda, const float* B,
                            int ldb, float beta, float* C, int ldc, const float* bias, int relu, void* stream) {
     PD_REQUIRE(M >= 0 && N >= 0 && K >= 0, PD_ESHAPE, "pd_gemm_f32: negative dimension");
@@ -460,6 +512,8 @@ extern "C" int pd_gemm_f32(int trans_a, int trans_b, int M, int N, int K, const 
     g.b_vec = pd_aligned(B, 16) && ldb % 4 == 0;
     g.k_per_split = K;
     g.c_split = 0;
+    g.a_bytes = operand_bytes(trans_a ? K : M, lda);
+    g.b_bytes = operand_bytes(trans_b ? N : K, ldb);
     hipStream_t s = (hipStream_t)stream;
     // Small problems use 64x64 tiles so that more of the 256 CUs get a block.
     long tiles128 = (long)((M + 127) / 128) * ((N + 127) / 128);
@@ -484,6 +538,8 @@ extern "C" int pd_gemm_splitk_f32(int trans_a, int trans_b, int M, int N, int K,
     // every split gets a whole number of 16-wide k chunks; trailing splits may be empty and then write zeros
     g.k_per_split = (((K + splits - 1) / splits) + BK - 1) / BK * BK;
     g.c_split = (long long)M * N;
+    g.a_bytes = operand_bytes(trans_a ? K : M, lda);
+    g.b_bytes = operand_bytes(trans_b ? N : K, ldb);
     hipStream_t s = (hipStream_t)stream;
     if (!trans_a && M <= 128 && N % 4 == 0 && g.a_vec && g.b_vec && g.k_per_split % BK == 0 && K % BK == 0 &&
         (size_t)128 * (lda > ldb ? lda : ldb) * 4 < (1ull << 31)) {
