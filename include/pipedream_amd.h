@@ -318,6 +318,38 @@ int pd_cast_f32_to_bf16(const float* x, uint16_t* y, uint64_t n, void* stream);
 int pd_cast_bf16_to_f32(const uint16_t* x, float* y, uint64_t n, void* stream);
 int pd_colsum_bf16(const uint16_t* x, float* out, uint64_t M, int N, uint64_t ld, int splits, void* stream);
 
+/* The label-smoothing criterion of the translation stages, LabelSmoothing.forward
+ * (runtime/translation/seq2seq/train/smoothing.py:23-34): logits [R][V] (R = seq*batch rows of leading
+ * dimension ld), fp32 log-softmax per row,
+ *   row_loss = (1 - smoothing) * (lse - x[target]) + smoothing * (lse - mean(x)),  0 where target ==
+ *   padding_idx,   loss[0] = sum(row_loss) / divisor   (divisor = the batch size, smoothing.py:33).
+ * row_loss[R] and lse[R] are outputs; the backward pass reads lse:
+ *   dlogits = (softmax(x) - (1 - smoothing) * onehot(target) - smoothing / V) * grad_loss[0] / divisor,
+ * 0 in padding rows.  A target outside [0, V) other than padding_idx makes the loss NaN. */
+int pd_label_smoothing_fwd_f32(const float* logits, const int64_t* target, float* loss, float* row_loss,
+                               float* lse, int R, int V, int64_t ld, int64_t padding_idx, float smoothing,
+                               float divisor, void* stream);
+int pd_label_smoothing_bwd_f32(const float* logits, const int64_t* target, const float* lse,
+                               const float* grad_loss, float* dlogits, int R, int V, int64_t ld, int64_t ldd,
+                               int64_t padding_idx, float smoothing, float divisor, void* stream);
+
+/* revert_varlen_tensor (runtime/translation/seq2seq/csrc/pack_utils_kernel.cu:25-62, bound to Python at
+ * pack_utils.cpp:37): in/out are [T][B] rows of row_bytes bytes (any element type of 2 or 4 bytes),
+ * consecutive rows in_pitch / out_pitch bytes apart (= row_bytes for a dense tensor; larger when the rows
+ * are one half of a wider tensor, e.g. one direction of a bidirectional layer's [T][B][2H] output),
+ *   out[t][b] = t < lengths[b] ? in[lengths[b] - 1 - t][b] : 0.
+ * lengths is B int64 values in DEVICE memory (the reference takes a host tensor, builds T*B offsets on the
+ * host and uploads them on every call); 0 < lengths[b] <= T is the caller's duty.  in != out.
+ * pd_length_mask_apply: out[t][b] = t < lengths[b] ? in[t][b] : 0 -- the product with the mask of
+ * set_mask_cpp in EmuBidirLSTM.emu_bidir_lstm (seq2seq/models/encoder.py:51,55); in == out is allowed. */
+int pd_revert_varlen(const void* in, void* out, const int64_t* lengths, int64_t T, int64_t B, int64_t row_bytes,
+                     int64_t in_pitch, int64_t out_pitch, void* stream);
+int pd_length_mask_apply(const void* in, void* out, const int64_t* lengths, int64_t T, int64_t B,
+                         int64_t row_bytes, int64_t in_pitch, int64_t out_pitch, void* stream);
+/* set_mask_cpp (runtime/translation/seq2seq/csrc/pack_utils.cpp:13-31): host code on host memory, as in
+ * the reference: mask[t][b] = lengths[b] > t for t < T (the reference takes T = lengths[0]). */
+int pd_set_mask_u8(const int64_t* lengths, int64_t B, int64_t T, uint8_t* mask);
+
 #ifdef __cplusplus
 }
 #endif

@@ -177,6 +177,35 @@ class GnmtStage0(torch.nn.Module):
         return out16 + out13
 
 
+class GnmtBidirStage0(torch.nn.Module):
+    """gnmt_large/gpus=4/stage0.py:8-40 as generated (bidirectional first layer, two outputs)."""
+
+    def __init__(self, vocab=32320, hidden=1024, dropout=0.2):
+        super(GnmtBidirStage0, self).__init__()
+        from . import seq2seq_oracle
+        self.layer6 = torch.nn.Embedding(vocab, hidden, padding_idx=0)
+        self.layer7 = seq2seq_oracle.EmuBidirLSTM(hidden, hidden)
+        self.layer8 = torch.nn.Dropout(p=dropout)
+        self.layer9 = torch.nn.LSTM(2 * hidden, hidden)
+        self.layer11 = torch.nn.Dropout(p=dropout)
+        self.layer12 = torch.nn.LSTM(hidden, hidden)
+        self.layer15 = torch.nn.Dropout(p=dropout)
+        self.layer16 = torch.nn.LSTM(hidden, hidden)
+        self.layer19 = torch.nn.Dropout(p=dropout)
+        self.layer20 = torch.nn.LSTM(hidden, hidden)
+
+    def forward(self, input0, input1):
+        out0 = input0.clone()
+        out1 = input1.clone()
+        out6 = self.layer6(out0)
+        out7 = self.layer7(out6, out1)
+        out10 = self.layer9(self.layer8(out7))[0]
+        out13 = self.layer12(self.layer11(out10))[0] + out10
+        out17 = self.layer16(self.layer15(out13))[0] + out13
+        out21 = self.layer20(self.layer19(out17))[0]
+        return (out17, out21)
+
+
 # --------------------------------------------------------------------------------------
 # bf16 pre-LN transformer stage (fp32 master parameters, bf16 activations and products)
 # --------------------------------------------------------------------------------------

@@ -105,6 +105,11 @@ SIGNATURES = {
     "pd_cast_f32_to_bf16": (_i, [_vp, _vp, _u64, _vp], True),
     "pd_cast_bf16_to_f32": (_i, [_vp, _vp, _u64, _vp], True),
     "pd_colsum_bf16": (_i, [_vp, _vp, _u64, _i, _u64, _i, _vp], True),
+    "pd_label_smoothing_fwd_f32": (_i, [_vp, _vp, _vp, _vp, _vp, _i, _i, _i64, _i64, _f, _f, _vp], True),
+    "pd_label_smoothing_bwd_f32": (_i, [_vp, _vp, _vp, _vp, _vp, _i, _i, _i64, _i64, _i64, _f, _f, _vp], True),
+    "pd_revert_varlen": (_i, [_vp, _vp, _vp, _i64, _i64, _i64, _i64, _i64, _vp], True),
+    "pd_length_mask_apply": (_i, [_vp, _vp, _vp, _i64, _i64, _i64, _i64, _i64, _vp], True),
+    "pd_set_mask_u8": (_i, [_vp, _i64, _i64, _vp], True),
     "pd_xent_bwd_f32": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i64, _vp], True),
 }
 

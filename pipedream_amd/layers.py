@@ -326,6 +326,111 @@ class LSTM(torch.nn.Module):
         return _LSTMFn.apply(x, self.weight_ih_l0, self.weight_hh_l0, self.bias_ih_l0, self.bias_hh_l0), None
 
 
+class _RevertVarlenFn(torch.autograd.Function):
+    @staticmethod
+    def forward(ctx, x, lengths):
+        ctx.save_for_backward(lengths)
+        return ops.revert_varlen(x.contiguous(), lengths)
+
+    @staticmethod
+    def backward(ctx, dy):
+        (lengths,) = ctx.saved_tensors
+        return ops.revert_varlen(dy.contiguous(), lengths), None
+
+
+def _device_lengths(lengths, like, seq_len):
+    """``lengths`` as B int64 values on ``like``'s device.  A host tensor is checked the way
+    revert_varlen_tensor checks it (seq2seq/csrc/pack_utils_kernel.cu:17-36) -- all of it rather than the
+    last entry only, and against the sequence length, beyond which the reference reads out of bounds --
+    a device tensor is taken as it is (checking it would stall the stream)."""
+    if lengths.dim() != 1:
+        raise ValueError("'lengths' argument should be a 1D int64 tensor")
+    if lengths.numel() != like.shape[1]:
+        raise ValueError("Expected `len(lengths)` to be equal to batch_size, but got %d (batch_size=%d)"
+                         % (lengths.numel(), like.shape[1]))
+    if lengths.device.type == "cpu":
+        if lengths.numel() and (int(lengths.min()) <= 0 or int(lengths.max()) > seq_len):
+            raise ValueError("Length of all samples has to be greater than 0 and at most the sequence length, "
+                             "but found an element in 'lengths' outside (0, %d]" % seq_len)
+        lengths = lengths.to(torch.int64).to(like.device, non_blocking=True)
+    return lengths.to(torch.int64).contiguous()
+
+
+def revert_varlen(x, lengths):
+    """``Revert_varlen.apply`` of seq2seq/models/encoder.py:13-23: reverses every sequence of ``x`` [T, B, ...]
+    over its own length; its backward is the same operation on the gradient."""
+    return _RevertVarlenFn.apply(x, _device_lengths(lengths, x, x.shape[0]))
+
+
+class _BidirMergeFn(torch.autograd.Function):
+    """[forward-direction output masked by length | backward-direction output reverted] side by side:
+    ``torch.cat([out0 * mask, revert_varlen(out1, lengths)], dim=2)`` of encoder.py:51-57 without the
+    intermediate tensors (both kernels write their half of the result in place)."""
+
+    @staticmethod
+    def forward(ctx, out0, out1, lengths):
+        T, B, H = out0.shape
+        y = torch.empty((T, B, 2 * H), dtype=out0.dtype, device=out0.device)
+        ops.length_mask_apply(out0.contiguous(), lengths, out=y[:, :, :H])
+        ops.revert_varlen(out1.contiguous(), lengths, out=y[:, :, H:])
+        ctx.save_for_backward(lengths)
+        ctx.hidden = H
+        return y
+
+    @staticmethod
+    def backward(ctx, dy):
+        (lengths,) = ctx.saved_tensors
+        H = ctx.hidden
+        dy = dy.contiguous()
+        return (ops.length_mask_apply(dy[:, :, :H], lengths), ops.revert_varlen(dy[:, :, H:], lengths), None)
+
+
+class _BidirParameters(torch.nn.Module):
+    """The eight parameters of ``torch.nn.LSTM(input_size, hidden_size, bidirectional=True)`` under torch's
+    names and initialisation (uniform(-1/sqrt(H), 1/sqrt(H)))."""
+
+    def __init__(self, input_size, hidden_size):
+        super(_BidirParameters, self).__init__()
+        k = 1.0 / math.sqrt(hidden_size)
+        for suffix in ("", "_reverse"):
+            for name, shape in (("weight_ih_l0", (4 * hidden_size, input_size)),
+                                ("weight_hh_l0", (4 * hidden_size, hidden_size)),
+                                ("bias_ih_l0", (4 * hidden_size,)), ("bias_hh_l0", (4 * hidden_size,))):
+                setattr(self, name + suffix, torch.nn.Parameter(torch.empty(*shape).uniform_(-k, k)))
+
+
+class EmuBidirLSTM(torch.nn.Module):
+    """``EmuBidirLSTM`` of seq2seq/models/encoder.py:25-64: a bidirectional LSTM layer on padded
+    sequence-first input ``[T, B, I]`` with per-sample ``lengths``, built from two uni-directional layers;
+    the backward direction runs on the time-reversed sequences and its output is reversed back.  Output
+    ``[T, B, 2H]``, zeros behind every sequence's end.
+
+    Parameters live in ``bidir`` under ``torch.nn.LSTM(bidirectional=True)``'s names and are shared with
+    ``layer1`` (forward direction) and ``layer2`` (``*_reverse``), as in encoder.py:32-41, so the
+    ``state_dict()`` keys are the reference's.  The reference switches to cuDNN's packed-sequence
+    bidirectional LSTM for batches above 128 (encoder.py:60-64); this layer computes the same values with
+    the two-layer form at every batch size."""
+
+    def __init__(self, input_size, hidden_size, num_layers=1, bias=True, batch_first=False, bidirectional=True):
+        super(EmuBidirLSTM, self).__init__()
+        assert num_layers == 1, "emulation bidirectional lstm works for a single layer only"
+        assert batch_first is False, "emulation bidirectional lstm works for batch_first = False only"
+        assert bidirectional is True, "use for bidirectional lstm only"
+        assert bias is True, "only the layer with bias is built"
+        self.bidir = _BidirParameters(input_size, hidden_size)
+        self.layer1 = LSTM(input_size, hidden_size)
+        self.layer2 = LSTM(input_size, hidden_size)
+        for name in ("weight_ih_l0", "weight_hh_l0", "bias_ih_l0", "bias_hh_l0"):
+            setattr(self.layer1, name, getattr(self.bidir, name))
+            setattr(self.layer2, name, getattr(self.bidir, name + "_reverse"))
+
+    def forward(self, input, lengths):
+        lengths = _device_lengths(lengths, input, input.shape[0])
+        out1 = self.layer2(_RevertVarlenFn.apply(input, lengths))[0]
+        out0 = self.layer1(input)[0]
+        return _BidirMergeFn.apply(out0, out1, lengths)
+
+
 class _AddFn(torch.autograd.Function):
     @staticmethod
     def forward(ctx, a, b):
@@ -479,6 +584,44 @@ class _CrossEntropyFn(torch.autograd.Function):
         x2, t, lse, count = ctx.saved_tensors
         d = ops.cross_entropy_backward(x2, t, lse, count, grad_loss.contiguous(), ctx.ignore_index)
         return d.view(ctx.shape), None, None
+
+
+class _LabelSmoothingFn(torch.autograd.Function):
+    @staticmethod
+    def forward(ctx, logits, target, padding_idx, smoothing, divisor):
+        x2 = logits.reshape(-1, logits.shape[-1])
+        if x2.stride(-1) != 1 or (x2.shape[0] > 1 and x2.stride(0) < x2.shape[1]):
+            x2 = x2.contiguous()
+        t = target.reshape(-1).contiguous()
+        loss, lse = ops.label_smoothing_forward(x2, t, padding_idx, smoothing, divisor)
+        ctx.args = (padding_idx, smoothing, divisor)
+        ctx.shape = logits.shape
+        ctx.save_for_backward(x2, t, lse)
+        return loss
+
+    @staticmethod
+    def backward(ctx, grad_loss):
+        x2, t, lse = ctx.saved_tensors
+        d = ops.label_smoothing_backward(x2, t, lse, grad_loss.contiguous(), *ctx.args)
+        return d.view(ctx.shape), None, None, None, None
+
+
+class LabelSmoothing(torch.nn.Module):
+    """NLL loss with label smoothing, the criterion of the translation stages
+    (seq2seq/train/smoothing.py:7-34, created at seq2seq/utils.py:31): ``output`` is [T, B, V] logits,
+    ``target`` the T*B token ids; rows whose target is ``padding_idx`` are dropped, the sum over the other
+    rows of ``(1-smoothing) * nll + smoothing * mean(-log_softmax)`` is divided by the batch size B."""
+
+    def __init__(self, padding_idx, smoothing=0.0):
+        super(LabelSmoothing, self).__init__()
+        self.padding_idx = padding_idx
+        self.confidence = 1.0 - smoothing
+        self.smoothing = smoothing
+
+    def forward(self, output, target):
+        if output.dim() < 2:
+            raise ValueError("LabelSmoothing: output must be [T, B, V], got %s" % (tuple(output.shape),))
+        return _LabelSmoothingFn.apply(output, target, self.padding_idx, self.smoothing, float(output.size(1)))
 
 
 class CrossEntropyLoss(torch.nn.Module):

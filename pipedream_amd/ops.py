@@ -268,6 +268,106 @@ def cross_entropy_backward(logits, target, lse, count, grad_loss, ignore_index=-
     return d
 
 
+def label_smoothing_forward(logits, target, padding_idx, smoothing, divisor):
+    """NLL loss with label smoothing over rows of ``logits`` [R, V] (seq2seq/train/smoothing.py:23-34):
+    sum over non-padding rows of (1-smoothing)*nll + smoothing*mean(-logprob), divided by ``divisor``.
+    Returns (loss[()], lse[R]); lse feeds the backward."""
+    _rowmajor2d(logits, "logits")
+    _check(target, "target", torch.int64)
+    R, V = logits.shape
+    if R == 0 or V == 0:
+        raise ValueError("label_smoothing: empty logits %s" % (tuple(logits.shape),))
+    if target.numel() != R or not target.is_contiguous():
+        raise ValueError("label_smoothing: target must be a contiguous vector of %d rows" % R)
+    dev = logits.device
+    loss = torch.empty((), dtype=torch.float32, device=dev)
+    row_loss = torch.empty(R, dtype=torch.float32, device=dev)
+    lse = torch.empty(R, dtype=torch.float32, device=dev)
+    ld = logits.stride(0) if R > 1 else V
+    with _timed("label_smoothing_fwd", 4.0 * R * V):
+        _cabi.lib().pd_label_smoothing_fwd_f32(_ptr(logits), _ptr(target), _ptr(loss), _ptr(row_loss), _ptr(lse),
+                                               R, V, ld, int(padding_idx), float(smoothing), float(divisor),
+                                               _cabi.stream_ptr())
+    return loss, lse
+
+
+def label_smoothing_backward(logits, target, lse, grad_loss, padding_idx, smoothing, divisor):
+    R, V = logits.shape
+    _check(grad_loss, "grad_loss")
+    grad_loss = grad_loss.reshape(1).contiguous()
+    d = torch.empty((R, V), dtype=torch.float32, device=logits.device)
+    ld = logits.stride(0) if R > 1 else V
+    with _timed("label_smoothing_bwd", 8.0 * R * V):
+        _cabi.lib().pd_label_smoothing_bwd_f32(_ptr(logits), _ptr(target), _ptr(lse), _ptr(grad_loss), _ptr(d),
+                                               R, V, ld, V, int(padding_idx), float(smoothing), float(divisor),
+                                               _cabi.stream_ptr())
+    return d
+
+
+def _varlen_rows(x, name):
+    """(T, B, row_bytes, pitch_bytes) of a [T, B, ...] tensor whose (t, b) rows are dense and evenly spaced:
+    a contiguous tensor or a slice of the last dimension of one."""
+    _cabi.require_device(x, name)
+    if x.dim() < 2:
+        raise ValueError("%s: input must be [T, B, ...], got shape %s" % (name, tuple(x.shape)))
+    if x.element_size() not in (2, 4):
+        raise TypeError("%s: element size must be 2 or 4 bytes, got %s" % (name, x.dtype))
+    T, B = x.shape[0], x.shape[1]
+    row = 1
+    for d in reversed(range(2, x.dim())):
+        if x.shape[d] != 1 and x.stride(d) != row:
+            raise ValueError("%s: trailing dimensions must be dense, got shape %s stride %s"
+                             % (name, tuple(x.shape), x.stride()))
+        row *= x.shape[d]
+    pitch = x.stride(1) if B > 1 else (x.stride(0) // max(B, 1) if T > 1 else row)
+    if pitch < row or (T > 1 and x.stride(0) != B * pitch):
+        raise ValueError("%s: rows must be evenly spaced, got shape %s stride %s"
+                         % (name, tuple(x.shape), x.stride()))
+    return T, B, row * x.element_size(), pitch * x.element_size()
+
+
+def _varlen_call(fn, name, x, lengths, out):
+    T, B, row_bytes, in_pitch = _varlen_rows(x, name)
+    _check(lengths, "lengths", torch.int64)
+    if lengths.dim() != 1 or lengths.numel() != B or not lengths.is_contiguous():
+        raise ValueError("Expected `len(lengths)` to be equal to batch_size, but got %d (batch_size=%d)"
+                         % (lengths.numel(), B))
+    if out is None:
+        out = torch.empty(x.shape, dtype=x.dtype, device=x.device)
+    elif out.shape != x.shape or out.dtype != x.dtype:
+        raise ValueError("%s: out must have the input's shape and dtype" % name)
+    out_pitch = _varlen_rows(out, name + " (out)")[3]
+    with _timed(name, 2.0 * T * B * row_bytes):
+        fn(_ptr(x), _ptr(out), _ptr(lengths), T, B, row_bytes, in_pitch, out_pitch, _cabi.stream_ptr())
+    return out
+
+
+def revert_varlen(x, lengths, out=None):
+    """Every sequence of ``x`` [T, B, ...] reversed in time over its own length, zeros behind it
+    (seq2seq/csrc/pack_utils_kernel.cu:25-62).  ``lengths``: B int64 values on the device, 0 < length <= T.
+    ``x`` and ``out`` may be slices of the last dimension of wider tensors; they must not overlap."""
+    return _varlen_call(_cabi.lib().pd_revert_varlen, "revert_varlen", x, lengths, out)
+
+
+def length_mask_apply(x, lengths, out=None):
+    """``x * set_mask(lengths).unsqueeze(-1)``: positions t >= lengths[b] of ``x`` [T, B, ...] become 0
+    (seq2seq/models/encoder.py:51,55).  ``out`` may be ``x`` itself."""
+    return _varlen_call(_cabi.lib().pd_length_mask_apply, "length_mask_apply", x, lengths, out)
+
+
+def set_mask(lengths):
+    """``set_mask_cpp`` (seq2seq/csrc/pack_utils.cpp:13-31): host uint8 mask [lengths[0], B] of a 1-D host
+    int64 tensor of lengths."""
+    if lengths.dim() != 1 or lengths.device.type != "cpu" or lengths.dtype != torch.int64:
+        raise ValueError("'lengths' argument should be a 1D CPU int64 tensor")
+    lengths = lengths.contiguous()
+    B = lengths.numel()
+    T = int(lengths[0]) if B else 0
+    mask = torch.empty((T, B), dtype=torch.uint8)
+    _cabi.lib().pd_set_mask_u8(_vp(lengths.data_ptr()), B, T, _vp(mask.data_ptr()))
+    return mask
+
+
 # --------------------------------------------------------------------------------------
 # 3x3 convolution (stride 1, padding 1), NHWC activations, KRSC filter
 # --------------------------------------------------------------------------------------
