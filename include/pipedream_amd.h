@@ -166,6 +166,14 @@ int pd_mask_scale_f32(const float* x, const uint8_t* mask, float* y, uint64_t n,
 int pd_maxpool2x2_fwd_nhwc_f32(const float* x, float* y, int N, int H, int W, int C, int relu, void* stream);
 int pd_maxpool2x2_bwd_nhwc_f32(const float* x, const float* dy, float* dx, int N, int H, int W, int C,
                                int relu_mask, void* stream);
+/* The same pooling with an index tensor: the forward also writes one byte per output element (bits 0-1:
+ * position of the first maximum in the window, row-major; bit 2: the maximum is positive); the backward
+ * reads the pooled gradient and that byte instead of the whole input (5 instead of 20 bytes read per
+ * output element) and writes dx [N,H,W,C]. */
+int pd_maxpool2x2_fwd_idx_nhwc_f32(const float* x, float* y, uint8_t* idx, int N, int H, int W, int C, int relu,
+                                   void* stream);
+int pd_maxpool2x2_bwd_idx_nhwc_f32(const float* dy, const uint8_t* idx, float* dx, int N, int H, int W, int C,
+                                   int relu_mask, void* stream);
 
 /* torch.nn.CrossEntropyLoss(reduction='mean') -- the criterion the caller appends to
  * the module list (main_with_runtime.py:126, applied at runtime/runtime.py:523-526).
@@ -213,6 +221,15 @@ int pd_conv3x3_winograd_filter_f32(const float* w, float* u, int C, int K, int r
 int pd_conv3x3_winograd_fwd_nhwc_f32(const float* x, const float* u, const float* bias,
                                      const float* in_mask, const float* out_mask, float* y,
                                      int N, int H, int W, int C, int K, int relu, void* stream);
+/* The same forward followed by 2x2 / stride-2 max pooling in the kernel's epilogue (a convolution and the
+ * ReLU + MaxPool2d behind it: vgg16/gpus=4_straight/stage0.py:14 + stage1.py:10-11 when they share a
+ * stage, vgg16/gpus=2/stage0.py:16-17 + stage1.py:10-11).  Writes y_pool [N,H/2,W/2,K] and one index
+ * byte per pooled element (bits 0-1: position of the first maximum in the window, row-major; bit 2: the
+ * maximum is positive) instead of the full-resolution output; pd_maxpool2x2_bwd_idx_nhwc_f32 turns the
+ * pooled gradient back into the convolution's output gradient. */
+int pd_conv3x3_winograd_fwd_pool_nhwc_f32(const float* x, const float* u, const float* bias, float* y_pool,
+                                          uint8_t* idx, int N, int H, int W, int C, int K, int relu,
+                                          void* stream);
 /* Weight (and optional bias) gradient of the same convolution in the Winograd domain: sums
  * dU = sum over 2x2 output tiles of (A dY A^T) (B^T d B) in persistent blocks, adds the blocks' partial
  * sums in fixed order and applies G^T . G.  Deterministic; agrees with pd_conv3x3_wgrad_nhwc_f32 to

@@ -80,6 +80,9 @@ SIGNATURES = {
     "pd_conv3x3_winograd_filter_bytes": (_i, [_i, _i, ctypes.POINTER(_u64)], True),
     "pd_conv3x3_winograd_filter_f32": (_i, [_vp, _vp, _i, _i, _i, _vp], True),
     "pd_conv3x3_winograd_fwd_nhwc_f32": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _vp], True),
+    "pd_conv3x3_winograd_fwd_pool_nhwc_f32": (_i, [_vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _vp], True),
+    "pd_maxpool2x2_fwd_idx_nhwc_f32": (_i, [_vp, _vp, _vp, _i, _i, _i, _i, _i, _vp], True),
+    "pd_maxpool2x2_bwd_idx_nhwc_f32": (_i, [_vp, _vp, _vp, _i, _i, _i, _i, _i, _vp], True),
     "pd_conv3x3_winograd_wgrad_supported": (_i, [_i, _i], False),
     "pd_conv3x3_winograd_wgrad_workspace_bytes": (_i, [_i, _i, ctypes.POINTER(_u64)], True),
     "pd_conv3x3_winograd_wgrad_nhwc_f32": (_i, [_vp, _vp, _vp, _vp, _vp, _u64, _i, _i, _i, _i, _i, _vp], True),

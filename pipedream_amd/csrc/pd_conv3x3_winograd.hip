@@ -67,6 +67,8 @@ struct WinoArgs {
     const float* mask;      // [N,H,W,C] or null: x is taken as 0 where mask <= 0
     const float* out_mask;  // [N,H,W,K] or null: y is written as 0 where out_mask <= 0
     float* y;               // [N,H,W,K]
+    float* pool_y;          // pooling variant: [N,H/2,W/2,K], written instead of y
+    uint8_t* pool_idx;      // pooling variant: [N,H/2,W/2,K] window position (bits 0-1) and sign (bit 2)
     int N, H, W, C, K;
     int relu;
     int tiles_x, tiles_y, k_blocks, n_chunks;
@@ -148,7 +150,7 @@ __device__ __forceinline__ WinoItem wino_decode(const WinoArgs& a, int item) {
 //             last use.
 // One barrier per step.  After the last chunk of an item: output transform, cross-wave sum in LDS, bias,
 // ReLU, output mask and 128-bit NHWC stores.
-template <bool MASK>
+template <bool MASK, bool POOL>
 __global__ __launch_bounds__(WG_THREADS, 1) void winograd_fwd_kernel(const WinoArgs a) {
     __shared__ __attribute__((aligned(16))) float lds[WG_LDS_FLOATS];
 
@@ -418,41 +420,95 @@ __global__ __launch_bounds__(WG_THREADS, 1) void winograd_fwd_kernel(const WinoA
             __syncthreads();
             if (gh == 1) out_rows(true);
             __syncthreads();
-            // bias, ReLU, output mask and the NHWC stores.  Thread -> pixel column (tid >> 4) & 15, channels
-            // k4..k4+3, pixel rows (tid >> 8) + 2 it: one base offset, a scalar stride per row pair.  Pixels
-            // outside the image get an offset beyond the buffer's size: such a store is dropped.
-            constexpr int NV = 256 * (WG_BN / 4) / WG_THREADS;
-            const int k4 = (tid & 15) * 4, pcol = (tid >> 4) & 15, prow = tid >> 8;
-            float4_t b4 = {0.f, 0.f, 0.f, 0.f};
-            if (a.bias) {
+            if constexpr (POOL) {
+                // 2x2 max pooling of the tile (bias and ReLU first), written with one index byte per element
+                // instead of the full-resolution output: bits 0-1 = position of the first maximum in the
+                // window (row-major), bit 2 = "maximum > 0".  Thread -> channels k4..k4+3, pooled column
+                // (tid >> 4) & 7, pooled rows (tid >> 7) + 4 it; tiles start at even pixels, so no window
+                // straddles two tiles.
+                const int Hp = a.H >> 1, Wp = a.W >> 1;
+                const int k4 = (tid & 15) * 4, pc = (tid >> 4) & 7, pr0 = tid >> 7;
+                float4_t b4 = {0.f, 0.f, 0.f, 0.f};
+                if (a.bias) {
 #pragma unroll
-                for (int c = 0; c < 4; ++c) b4[c] = k0 + k4 + c < a.K ? a.bias[k0 + k4 + c] : 0.f;
-            }
-            const uint32_t out_bytes = (uint32_t)a.H * a.W * a.K * 4;
-            const __amdgpu_buffer_rsrc_t yr =
-                __builtin_amdgcn_make_buffer_rsrc((void*)(a.y + oimg), 0, out_bytes, 0x00020000);
-            const __amdgpu_buffer_rsrc_t omr = __builtin_amdgcn_make_buffer_rsrc(
-                (void*)((a.out_mask ? a.out_mask : a.y) + oimg), 0, out_bytes, 0x00020000);
-            const bool col_ok = w.x0 + pcol < a.W && k0 + k4 < a.K;
-            const uint32_t obase = (uint32_t)(((w.y0 + prow) * a.W + w.x0 + pcol) * a.K + k0 + k4) * 4;
-            const int row_stride = 2 * a.W * a.K * 4;
-            const float* src = stg + (prow * WG_PIX + pcol) * WG_OP + k4;
-#pragma unroll
-            for (int it = 0; it < NV; ++it) {
-                const uint32_t voff = (col_ok && w.y0 + prow + 2 * it < a.H) ? obase : 0x80000000u;
-                float4_t v = *(const float4_t*)(src + it * 2 * WG_PIX * WG_OP) + b4;
-                if (a.relu) {
-#pragma unroll
-                    for (int c = 0; c < 4; ++c) v[c] = v[c] > 0.f ? v[c] : 0.f;
+                    for (int c = 0; c < 4; ++c) b4[c] = k0 + k4 + c < a.K ? a.bias[k0 + k4 + c] : 0.f;
                 }
-                if (a.out_mask) {
-                    const float4_t mk = __builtin_bit_cast(
-                        float4_t, __builtin_amdgcn_raw_buffer_load_b128(omr, voff, it * row_stride, 2));
+                const size_t pimg = (size_t)w.n * Hp * Wp * a.K;
+                const uint32_t pool_elems = (uint32_t)Hp * Wp * a.K;
+                const __amdgpu_buffer_rsrc_t pyr =
+                    __builtin_amdgcn_make_buffer_rsrc((void*)(a.pool_y + pimg), 0, pool_elems * 4, 0x00020000);
+                const __amdgpu_buffer_rsrc_t pir =
+                    __builtin_amdgcn_make_buffer_rsrc((void*)(a.pool_idx + pimg), 0, pool_elems, 0x00020000);
+                const int py0 = w.y0 >> 1, px0 = w.x0 >> 1;
+                const bool col_ok = px0 + pc < Wp && k0 + k4 < a.K;
 #pragma unroll
-                    for (int c = 0; c < 4; ++c) v[c] = mk[c] > 0.f ? v[c] : 0.f;
+                for (int it = 0; it < 2; ++it) {
+                    const int pr = pr0 + 4 * it;
+                    const bool ok = col_ok && py0 + pr < Hp;
+                    const uint32_t eoff = (uint32_t)(((py0 + pr) * Wp + px0 + pc) * a.K + k0 + k4);
+                    const float* src = stg + ((2 * pr) * WG_PIX + 2 * pc) * WG_OP + k4;
+                    float4_t v[4];
+                    v[0] = *(const float4_t*)(src) + b4;
+                    v[1] = *(const float4_t*)(src + WG_OP) + b4;
+                    v[2] = *(const float4_t*)(src + WG_PIX * WG_OP) + b4;
+                    v[3] = *(const float4_t*)(src + (WG_PIX + 1) * WG_OP) + b4;
+                    float4_t best;
+                    uint32_t packed = 0;
+#pragma unroll
+                    for (int c = 0; c < 4; ++c) {
+                        float q[4];
+#pragma unroll
+                        for (int j = 0; j < 4; ++j) q[j] = (a.relu && !(v[j][c] > 0.f)) ? 0.f : v[j][c];   // as the plain epilogue
+                        float b = q[0];
+                        uint32_t arg = 0;
+#pragma unroll
+                        for (int j = 1; j < 4; ++j)
+                            if (q[j] > b || q[j] != q[j]) { b = q[j]; arg = j; }
+                        best[c] = b;
+                        packed |= (arg | (b > 0.f ? 4u : 0u)) << (8 * c);
+                    }
+                    typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+                    __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(u32x4, best), pyr,
+                                                           ok ? eoff * 4 : 0x80000000u, 0, 0);
+                    __builtin_amdgcn_raw_buffer_store_b32(packed, pir, ok ? eoff : 0x80000000u, 0, 0);
                 }
-                typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
-                __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(u32x4, v), yr, voff, it * row_stride, 2);
+            } else {
+                // bias, ReLU, output mask and the NHWC stores.  Thread -> pixel column (tid >> 4) & 15, channels
+                // k4..k4+3, pixel rows (tid >> 8) + 2 it: one base offset, a scalar stride per row pair.  Pixels
+                // outside the image get an offset beyond the buffer's size: such a store is dropped.
+                constexpr int NV = 256 * (WG_BN / 4) / WG_THREADS;
+                const int k4 = (tid & 15) * 4, pcol = (tid >> 4) & 15, prow = tid >> 8;
+                float4_t b4 = {0.f, 0.f, 0.f, 0.f};
+                if (a.bias) {
+    #pragma unroll
+                    for (int c = 0; c < 4; ++c) b4[c] = k0 + k4 + c < a.K ? a.bias[k0 + k4 + c] : 0.f;
+                }
+                const uint32_t out_bytes = (uint32_t)a.H * a.W * a.K * 4;
+                const __amdgpu_buffer_rsrc_t yr =
+                    __builtin_amdgcn_make_buffer_rsrc((void*)(a.y + oimg), 0, out_bytes, 0x00020000);
+                const __amdgpu_buffer_rsrc_t omr = __builtin_amdgcn_make_buffer_rsrc(
+                    (void*)((a.out_mask ? a.out_mask : a.y) + oimg), 0, out_bytes, 0x00020000);
+                const bool col_ok = w.x0 + pcol < a.W && k0 + k4 < a.K;
+                const uint32_t obase = (uint32_t)(((w.y0 + prow) * a.W + w.x0 + pcol) * a.K + k0 + k4) * 4;
+                const int row_stride = 2 * a.W * a.K * 4;
+                const float* src = stg + (prow * WG_PIX + pcol) * WG_OP + k4;
+    #pragma unroll
+                for (int it = 0; it < NV; ++it) {
+                    const uint32_t voff = (col_ok && w.y0 + prow + 2 * it < a.H) ? obase : 0x80000000u;
+                    float4_t v = *(const float4_t*)(src + it * 2 * WG_PIX * WG_OP) + b4;
+                    if (a.relu) {
+    #pragma unroll
+                        for (int c = 0; c < 4; ++c) v[c] = v[c] > 0.f ? v[c] : 0.f;
+                    }
+                    if (a.out_mask) {
+                        const float4_t mk = __builtin_bit_cast(
+                            float4_t, __builtin_amdgcn_raw_buffer_load_b128(omr, voff, it * row_stride, 2));
+    #pragma unroll
+                        for (int c = 0; c < 4; ++c) v[c] = mk[c] > 0.f ? v[c] : 0.f;
+                    }
+                    typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+                    __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(u32x4, v), yr, voff, it * row_stride, 2);
+                }
             }
         }
         // the next epilogue's staging writes come after at least one more barrier (n_chunks >= 1)
@@ -485,19 +541,21 @@ extern "C" int pd_conv3x3_winograd_filter_f32(const float* w, float* u, int C, i
     return PD_OK;
 }
 
-extern "C" int pd_conv3x3_winograd_fwd_nhwc_f32(const float* x, const float* u, const float* bias,
-                                                const float* in_mask, const float* out_mask, float* y, int N, int H,
-                                                int W, int C, int K, int relu, void* stream) {
-    const char* who = "pd_conv3x3_winograd_fwd_nhwc_f32";
+namespace {
+
+int wino_fwd_launch(const char* who, const float* x, const float* u, const float* bias, const float* in_mask,
+                    const float* out_mask, float* y, float* pool_y, uint8_t* pool_idx, int N, int H, int W, int C,
+                    int K, int relu, void* stream) {
     PD_REQUIRE(N > 0 && H > 0 && W > 0 && C > 0 && K > 0, PD_ESHAPE, "%s: dimensions must be positive", who);
     PD_REQUIRE(wino_shape_ok(C, K), PD_ESHAPE, "%s: needs C %% 8 == 0 and K %% 4 == 0 (C=%d K=%d)", who, C, K);
     PD_REQUIRE((long)H * W * (C > K ? C : K) < (1L << 29), PD_ESHAPE, "%s: image too large", who);
     PD_REQUIRE((long)C * WG_G * WG_BN * 4 < (1L << 31), PD_ESHAPE, "%s: too many input channels", who);
-    PD_REQUIRE(x && u && y, PD_EINVAL, "%s: NULL pointer", who);
+    PD_REQUIRE(x && u, PD_EINVAL, "%s: NULL pointer", who);
     PD_REQUIRE(pd_aligned(x, 16) && pd_aligned(u, 16) && pd_aligned(y, 16) && pd_aligned(in_mask, 16) &&
                    pd_aligned(out_mask, 16), PD_EINVAL, "%s: tensors must be 16-byte aligned", who);
     WinoArgs a;
     a.x = x; a.u = u; a.bias = bias; a.mask = in_mask; a.out_mask = out_mask; a.y = y;
+    a.pool_y = pool_y; a.pool_idx = pool_idx;
     a.N = N; a.H = H; a.W = W; a.C = C; a.K = K;
     a.relu = relu != 0;
     a.tiles_x = (W + WG_PIX - 1) / WG_PIX;
@@ -517,10 +575,32 @@ extern "C" int pd_conv3x3_winograd_fwd_nhwc_f32(const float* x, const float* u, 
     if (blocks > (long)a.items_per_xcd * WG_XCD) blocks = (long)a.items_per_xcd * WG_XCD;
     dim3 grid((unsigned)blocks);
     hipStream_t s = (hipStream_t)stream;
-    if (in_mask) winograd_fwd_kernel<true><<<grid, WG_THREADS, 0, s>>>(a);
-    else winograd_fwd_kernel<false><<<grid, WG_THREADS, 0, s>>>(a);
+    if (a.pool_y) winograd_fwd_kernel<false, true><<<grid, WG_THREADS, 0, s>>>(a);
+    else if (in_mask) winograd_fwd_kernel<true, false><<<grid, WG_THREADS, 0, s>>>(a);
+    else winograd_fwd_kernel<false, false><<<grid, WG_THREADS, 0, s>>>(a);
     PD_CHECK_LAUNCH(who);
     return PD_OK;
+}
+
+}  // namespace
+
+extern "C" int pd_conv3x3_winograd_fwd_nhwc_f32(const float* x, const float* u, const float* bias,
+                                                const float* in_mask, const float* out_mask, float* y, int N, int H,
+                                                int W, int C, int K, int relu, void* stream) {
+    const char* who = "pd_conv3x3_winograd_fwd_nhwc_f32";
+    PD_REQUIRE(y, PD_EINVAL, "%s: NULL pointer", who);
+    return wino_fwd_launch(who, x, u, bias, in_mask, out_mask, y, nullptr, nullptr, N, H, W, C, K, relu, stream);
+}
+
+extern "C" int pd_conv3x3_winograd_fwd_pool_nhwc_f32(const float* x, const float* u, const float* bias,
+                                                     float* y_pool, uint8_t* idx, int N, int H, int W, int C, int K,
+                                                     int relu, void* stream) {
+    const char* who = "pd_conv3x3_winograd_fwd_pool_nhwc_f32";
+    PD_REQUIRE(H >= 2 && W >= 2, PD_ESHAPE, "%s: the image must hold at least one 2x2 window", who);
+    PD_REQUIRE(y_pool && idx, PD_EINVAL, "%s: NULL pointer", who);
+    PD_REQUIRE(pd_aligned(y_pool, 16) && pd_aligned(idx, 4), PD_EINVAL,
+               "%s: the pooled output must be 16-byte aligned, the index bytes 4-byte aligned", who);
+    return wino_fwd_launch(who, x, u, bias, nullptr, nullptr, nullptr, y_pool, idx, N, H, W, C, K, relu, stream);
 }
 
 // =====================================================================================================

@@ -146,6 +146,93 @@ __global__ __launch_bounds__(PW_THREADS) void maxpool2_bwd_kernel(const float* _
     *(float4_t*)(dx + off + (uint64_t)W * C + C) = o[3];
 }
 
+// ---- the same pooling with an index tensor ---------------------------------------------
+// The forward also writes one byte per output element: bits 0-1 = position of the maximum in the window
+// (scan order as above), bit 2 = "the maximum is positive".  The backward then needs the pooled gradient
+// and that byte instead of the whole input: 4 + 1 bytes read per output element instead of 4 + 16.
+__device__ __forceinline__ uint32_t pool_pick(float v0, float v1, float v2, float v3, float* best_out) {
+    float best = v0;
+    uint32_t arg = 0;
+    if (pool_better(v1, best)) { best = v1; arg = 1; }
+    if (pool_better(v2, best)) { best = v2; arg = 2; }
+    if (pool_better(v3, best)) { best = v3; arg = 3; }
+    *best_out = best;
+    return arg | (best > 0.f ? 4u : 0u);
+}
+
+__global__ __launch_bounds__(PW_THREADS) void maxpool2_fwd_idx_kernel(const float* __restrict__ x,
+                                                                      float* __restrict__ y,
+                                                                      uint32_t* __restrict__ idx, int N, int H, int W,
+                                                                      int C, int relu) {
+    const int Ho = H / 2, Wo = W / 2, C4 = C / 4;
+    uint64_t id = (uint64_t)blockIdx.x * PW_THREADS + threadIdx.x;
+    uint64_t total = (uint64_t)N * Ho * Wo * C4;
+    if (id >= total) return;
+    int c4 = id % C4;
+    uint64_t p = id / C4;
+    int ox = p % Wo;
+    p /= Wo;
+    int oy = p % Ho;
+    int n = p / Ho;
+    const float* base = x + (((uint64_t)n * H + 2 * oy) * W + 2 * ox) * C + c4 * 4;
+    const float4_t v0 = *(const float4_t*)base;
+    const float4_t v1 = *(const float4_t*)(base + C);
+    const float4_t v2 = *(const float4_t*)(base + (uint64_t)W * C);
+    const float4_t v3 = *(const float4_t*)(base + (uint64_t)W * C + C);
+    float4_t best;
+    uint32_t packed = 0;
+#pragma unroll
+    for (int k = 0; k < 4; ++k) {
+        float b;
+        packed |= pool_pick(v0[k], v1[k], v2[k], v3[k], &b) << (8 * k);
+        if (relu && b < 0.f) b = 0.f;
+        best[k] = b;
+    }
+    const uint64_t o = (((uint64_t)n * Ho + oy) * Wo + ox) * C + c4 * 4;
+    *(float4_t*)(y + o) = best;
+    idx[o / 4] = packed;
+}
+
+// dx [N,H,W,C] from dy [N,H/2,W/2,C] and the index bytes: the window position named by the byte gets the
+// gradient (0 if relu_mask is set and the maximum was not positive), the other three and the ragged edge 0.
+__global__ __launch_bounds__(PW_THREADS) void maxpool2_bwd_idx_kernel(const float* __restrict__ dy,
+                                                                      const uint32_t* __restrict__ idx,
+                                                                      float* __restrict__ dx, int N, int H, int W, int C,
+                                                                      int relu_mask) {
+    const int Ho = H / 2, Wo = W / 2, C4 = C / 4;
+    const int Hc = (H + 1) / 2, Wc = (W + 1) / 2;  // windows incl. the ragged edge
+    uint64_t id = (uint64_t)blockIdx.x * PW_THREADS + threadIdx.x;
+    uint64_t total = (uint64_t)N * Hc * Wc * C4;
+    if (id >= total) return;
+    int c4 = id % C4;
+    uint64_t p = id / C4;
+    int ox = p % Wc;
+    p /= Wc;
+    int oy = p % Hc;
+    int n = p / Hc;
+    const bool inside = oy < Ho && ox < Wo;
+    const uint64_t off = (((uint64_t)n * H + 2 * oy) * W + 2 * ox) * C + c4 * 4;
+    const bool has_x1 = 2 * ox + 1 < W, has_y1 = 2 * oy + 1 < H;
+    const float4_t zero = {0.f, 0.f, 0.f, 0.f};
+    float4_t o[4] = {zero, zero, zero, zero};
+    if (inside) {
+        const uint64_t po = (((uint64_t)n * Ho + oy) * Wo + ox) * C + c4 * 4;
+        const float4_t g = *(const float4_t*)(dy + po);
+        const uint32_t packed = idx[po / 4];
+#pragma unroll
+        for (int k = 0; k < 4; ++k) {
+            const uint32_t b = (packed >> (8 * k)) & 0xffu;
+            const float gk = (relu_mask && !(b & 4u)) ? 0.f : g[k];
+#pragma unroll
+            for (int j = 0; j < 4; ++j) o[j][k] = (j == (int)(b & 3u)) ? gk : 0.f;
+        }
+    }
+    *(float4_t*)(dx + off) = o[0];
+    if (has_x1) *(float4_t*)(dx + off + C) = o[1];
+    if (has_y1) *(float4_t*)(dx + off + (uint64_t)W * C) = o[2];
+    if (has_x1 && has_y1) *(float4_t*)(dx + off + (uint64_t)W * C + C) = o[3];
+}
+
 // ---- softmax cross-entropy ------------------------------------------------------------
 __device__ __forceinline__ float wave_max(float v) {
 #pragma unroll
@@ -336,6 +423,43 @@ extern "C" int pd_maxpool2x2_bwd_nhwc_f32(const float* x, const float* dy, float
     PD_REQUIRE(blocks_for(total, &blocks) == 0, PD_ESHAPE, "pd_maxpool2x2_bwd: too large");
     maxpool2_bwd_kernel<<<dim3(blocks), dim3(PW_THREADS), 0, (hipStream_t)stream>>>(x, dy, dx, N, H, W, C, relu_mask);
     PD_CHECK_LAUNCH("pd_maxpool2x2_bwd");
+    return PD_OK;
+}
+
+extern "C" int pd_maxpool2x2_fwd_idx_nhwc_f32(const float* x, float* y, uint8_t* idx, int N, int H, int W, int C,
+                                              int relu, void* stream) {
+    const char* who = "pd_maxpool2x2_fwd_idx";
+    PD_REQUIRE(N >= 0 && H >= 0 && W >= 0 && C >= 0, PD_ESHAPE, "%s: negative dimension", who);
+    PD_REQUIRE(C % 4 == 0, PD_ESHAPE, "%s: channels must be a multiple of 4 (got %d)", who, C);
+    uint64_t total = (uint64_t)N * (H / 2) * (W / 2) * (C / 4);
+    if (total == 0) return PD_OK;
+    PD_REQUIRE(x && y && idx, PD_EINVAL, "%s: NULL pointer", who);
+    PD_REQUIRE(pd_aligned(x, 16) && pd_aligned(y, 16) && pd_aligned(idx, 4), PD_EINVAL,
+               "%s: tensors must be 16-byte aligned (index bytes: 4)", who);
+    unsigned blocks;
+    PD_REQUIRE(blocks_for(total, &blocks) == 0, PD_ESHAPE, "%s: too large", who);
+    maxpool2_fwd_idx_kernel<<<dim3(blocks), dim3(PW_THREADS), 0, (hipStream_t)stream>>>(x, y, (uint32_t*)idx, N, H, W,
+                                                                                    C, relu);
+    PD_CHECK_LAUNCH(who);
+    return PD_OK;
+}
+
+extern "C" int pd_maxpool2x2_bwd_idx_nhwc_f32(const float* dy, const uint8_t* idx, float* dx, int N, int H, int W,
+                                              int C, int relu_mask, void* stream) {
+    const char* who = "pd_maxpool2x2_bwd_idx";
+    PD_REQUIRE(N >= 0 && H >= 0 && W >= 0 && C >= 0, PD_ESHAPE, "%s: negative dimension", who);
+    PD_REQUIRE(C % 4 == 0, PD_ESHAPE, "%s: channels must be a multiple of 4 (got %d)", who, C);
+    uint64_t total = (uint64_t)N * ((H + 1) / 2) * ((W + 1) / 2) * (C / 4);
+    if (total == 0) return PD_OK;
+    PD_REQUIRE(dx, PD_EINVAL, "%s: NULL pointer", who);
+    PD_REQUIRE((dy && idx) || (uint64_t)(H / 2) * (W / 2) == 0, PD_EINVAL, "%s: NULL pointer", who);
+    PD_REQUIRE(pd_aligned(dy, 16) && pd_aligned(dx, 16) && pd_aligned(idx, 4), PD_EINVAL,
+               "%s: tensors must be 16-byte aligned (index bytes: 4)", who);
+    unsigned blocks;
+    PD_REQUIRE(blocks_for(total, &blocks) == 0, PD_ESHAPE, "%s: too large", who);
+    maxpool2_bwd_idx_kernel<<<dim3(blocks), dim3(PW_THREADS), 0, (hipStream_t)stream>>>(dy, (const uint32_t*)idx, dx, N,
+                                                                                    H, W, C, relu_mask);
+    PD_CHECK_LAUNCH(who);
     return PD_OK;
 }
 

@@ -81,12 +81,20 @@ class Linear(torch.nn.Module):
 # --------------------------------------------------------------------------------------
 class _Conv3x3Fn(torch.autograd.Function):
     @staticmethod
-    def forward(ctx, x, weight, bias, relu, grad_premasked=False, input_rectified=False):
+    def forward(ctx, x, weight, bias, relu, grad_premasked=False, input_rectified=False, pool=False):
         x = ops.to_nhwc(x)
         ctx.input_rectified = input_rectified
-        y = ops.conv3x3_forward(x, weight, bias, relu)
         ctx.relu = relu
         ctx.has_bias = bias is not None
+        ctx.pool = pool
+        if pool:
+            # convolution (+ReLU) and the 2x2 pooling behind it in one kernel: the backward rebuilds the
+            # convolution's output gradient from the pooled gradient and the index bytes, already masked
+            # by the ReLU, so the full-resolution output is neither written nor kept
+            y, idx = ops.conv3x3_forward_pool(x, weight, bias, relu)
+            ctx.save_for_backward(x, weight, idx)
+            return y
+        y = ops.conv3x3_forward(x, weight, bias, relu)
         # with grad_premasked the consumer's backward (a pooling layer with relu=True) has already
         # zeroed dy wherever y == 0, so the gradient kernels need not read y at all
         ctx.save_for_backward(x, weight, y if (relu and not grad_premasked) else None)
@@ -96,6 +104,9 @@ class _Conv3x3Fn(torch.autograd.Function):
     def backward(ctx, dy):
         x, weight, y = ctx.saved_tensors
         dy = ops.to_nhwc(dy)
+        if ctx.pool:
+            dy = ops.maxpool2x2_idx_backward(dy, y, x.shape[2], x.shape[3], relu_mask=ctx.relu)
+            y = None
         # the ReLU backward (dy where y > 0) is applied by the gradient kernels while they
         # load dy, so no masked copy of dy is ever written
         dx = dw = db = None
@@ -103,7 +114,7 @@ class _Conv3x3Fn(torch.autograd.Function):
             dx = ops.conv3x3_input_grad(dy, weight, relu_out=y, x_rectified=x if ctx.input_rectified else None)
         if ctx.needs_input_grad[1] or (ctx.has_bias and ctx.needs_input_grad[2]):
             dw, db = ops.conv3x3_weight_grad(x, dy, with_bias=ctx.has_bias, relu_out=y)
-        return dx, dw, db, None, None, None
+        return dx, dw, db, None, None, None, None
 
 
 class Conv2d(torch.nn.Module):
@@ -118,10 +129,15 @@ class Conv2d(torch.nn.Module):
     not be applied (and the output not be read) again here.  ``input_rectified=True`` makes this layer
     such a consumer: it declares that the layer's input is the output of a ReLU (a preceding
     ``Conv2d(relu=True, grad_premasked=True)``) and zeroes the input gradient where the input is zero
-    as it is stored.  Results are identical either way."""
+    as it is stored.  Results are identical either way.
+
+    ``pool=True`` appends ``MaxPool2d(2, 2)`` to the layer (after the ReLU, if any): the layer returns the
+    pooled tensor, computed in the convolution kernel's epilogue where that kernel supports it, and the
+    pooling module that follows in the reference's layer list is declared with
+    ``MaxPool2d(..., applied_by_producer=True)``."""
 
     def __init__(self, in_channels, out_channels, kernel_size=3, stride=1, padding=1, bias=True, relu=False,
-                 grad_premasked=False, input_rectified=False):
+                 grad_premasked=False, input_rectified=False, pool=False):
         super(Conv2d, self).__init__()
         norm = lambda v: tuple(v) if isinstance(v, (tuple, list)) else (v, v)
         if norm(kernel_size) != (3, 3) or norm(stride) != (1, 1) or norm(padding) != (1, 1):
@@ -133,6 +149,7 @@ class Conv2d(torch.nn.Module):
             raise ValueError("grad_premasked only makes sense with relu=True")
         self.grad_premasked = grad_premasked
         self.input_rectified = input_rectified
+        self.pool = pool
         w = torch.empty(out_channels, in_channels, 3, 3)
         torch.nn.init.kaiming_uniform_(w, a=math.sqrt(5))
         self.weight = torch.nn.Parameter(w.contiguous(memory_format=torch.channels_last))
@@ -143,7 +160,8 @@ class Conv2d(torch.nn.Module):
             self.bias = None
 
     def forward(self, x):
-        return _Conv3x3Fn.apply(x, self.weight, self.bias, self.relu, self.grad_premasked, self.input_rectified)
+        return _Conv3x3Fn.apply(x, self.weight, self.bias, self.relu, self.grad_premasked, self.input_rectified,
+                                self.pool)
 
     def extra_repr(self):
         return "{}, {}, kernel_size=(3, 3), stride=(1, 1), padding=(1, 1), relu={}".format(
@@ -182,29 +200,37 @@ class _MaxPool2x2Fn(torch.autograd.Function):
     @staticmethod
     def forward(ctx, x, relu):
         x = ops.to_nhwc(x)
-        y = ops.maxpool2x2(x, relu=relu)
+        y, idx = ops.maxpool2x2_idx(x, relu=relu)
         ctx.relu = relu
-        ctx.save_for_backward(x)
+        ctx.hw = (x.shape[2], x.shape[3])
+        ctx.save_for_backward(idx)      # one byte per output element; the input is not needed again
         return y
 
     @staticmethod
     def backward(ctx, dy):
-        (x,) = ctx.saved_tensors
-        return ops.maxpool2x2_backward(x, dy, relu_mask=ctx.relu), None
+        (idx,) = ctx.saved_tensors
+        return ops.maxpool2x2_idx_backward(dy, idx, ctx.hw[0], ctx.hw[1], relu_mask=ctx.relu), None
 
 
 class MaxPool2d(torch.nn.Module):
-    """``torch.nn.MaxPool2d(kernel_size=2, stride=2)`` on NHWC activations."""
+    """``torch.nn.MaxPool2d(kernel_size=2, stride=2)`` on NHWC activations.  ``relu=True``: a ReLU in front
+    of the pooling (stage1.py:10-11), fused.  ``applied_by_producer=True``: the convolution in front of
+    this module was built with ``pool=True`` and has already pooled (and rectified) its output; the module
+    keeps its place in the layer list and passes the tensor through."""
 
-    def __init__(self, kernel_size=2, stride=2, padding=0, dilation=1, ceil_mode=False, relu=False):
+    def __init__(self, kernel_size=2, stride=2, padding=0, dilation=1, ceil_mode=False, relu=False,
+                 applied_by_producer=False):
         super(MaxPool2d, self).__init__()
-        self.relu = relu  # a ReLU in front of the pooling (stage1.py:10-11), fused
+        self.relu = relu
+        self.applied_by_producer = applied_by_producer
         ks = kernel_size if isinstance(kernel_size, int) else kernel_size[0]
         st = ks if stride is None else (stride if isinstance(stride, int) else stride[0])
         if ks != 2 or st != 2 or padding not in (0, (0, 0)) or dilation not in (1, (1, 1)) or ceil_mode:
             raise NotImplementedError("only MaxPool2d(kernel_size=2, stride=2) has a HIP kernel")
 
     def forward(self, x):
+        if self.applied_by_producer:
+            return x
         return _MaxPool2x2Fn.apply(x, self.relu)
 
 

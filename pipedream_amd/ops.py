@@ -239,6 +239,38 @@ def maxpool2x2_backward(x, dy, relu_mask=False):
     return dx
 
 
+def maxpool2x2_idx(x, relu=False):
+    """2x2/stride-2 max pooling that also returns one index byte per output element (bits 0-1: position of
+    the first maximum in its window, row-major; bit 2: the maximum is positive) -- all the backward needs."""
+    _check(x, "x")
+    x = to_nhwc(x)
+    n, h, w, c = _nhwc_dims(x)
+    y = torch.empty((n, c, h // 2, w // 2), dtype=torch.float32, device=x.device,
+                    memory_format=torch.channels_last)
+    idx = torch.empty((n, c, h // 2, w // 2), dtype=torch.uint8, device=x.device,
+                      memory_format=torch.channels_last)
+    with _timed("maxpool2x2_fwd_idx", 4.0 * n * c * (h * w + 1.25 * (h // 2) * (w // 2))):
+        _cabi.lib().pd_maxpool2x2_fwd_idx_nhwc_f32(_ptr(x), _ptr(y), _ptr(idx), n, h, w, c, int(relu),
+                                                   _cabi.stream_ptr())
+    return y, idx
+
+
+def maxpool2x2_idx_backward(dy, idx, h, w, relu_mask=False):
+    """dx [N,C,h,w] of a 2x2 pooling from the pooled gradient and the forward's index bytes."""
+    _check(dy, "dy")
+    _check(idx, "idx", torch.uint8)
+    dy = to_nhwc(dy)
+    n, ho, wo, c = _nhwc_dims(dy)
+    if (ho, wo) != (h // 2, w // 2) or idx.shape != dy.shape or not idx.is_contiguous(memory_format=torch.channels_last):
+        raise ValueError("maxpool2x2_idx_backward: dy %s / idx %s do not belong to a %dx%d input"
+                         % (tuple(dy.shape), tuple(idx.shape), h, w))
+    dx = torch.empty((n, c, h, w), dtype=torch.float32, device=dy.device, memory_format=torch.channels_last)
+    with _timed("maxpool2x2_bwd_idx", 4.0 * n * c * (h * w + 1.25 * ho * wo)):
+        _cabi.lib().pd_maxpool2x2_bwd_idx_nhwc_f32(_ptr(dy), _ptr(idx), _ptr(dx), n, h, w, c, int(relu_mask),
+                                                   _cabi.stream_ptr())
+    return dx
+
+
 def cross_entropy_forward(logits, target, ignore_index=-100):
     """Mean softmax cross-entropy.  Returns (loss[()], (lse, count)) for the backward."""
     _rowmajor2d(logits, "logits")
@@ -433,6 +465,36 @@ def conv3x3_forward(x, w, bias=None, relu=False):
         _cabi.lib().pd_conv3x3_fwd_nhwc_f32(_ptr(x), _ptr(w), _ptr(bias), _ptr(y), n, h, wd, c, k, int(relu),
                                             _cabi.stream_ptr())
     return y
+
+
+def conv3x3_forward_pool(x, w, bias=None, relu=False):
+    """``maxpool2x2_idx(conv3x3_forward(x, w, bias, relu))``: returns (pooled output, index bytes).  Where the
+    Winograd kernel applies, the pooling happens in its epilogue and the full-resolution output is never
+    written."""
+    _check(x, "x")
+    n, h, wd, c = _nhwc_dims(x)
+    k, cw = _filter_dims(w)
+    if cw != c:
+        raise ValueError("conv3x3: input has %d channels, filter expects %d" % (c, cw))
+    if not (_use_winograd(c, k) and h >= 2 and wd >= 2):
+        return maxpool2x2_idx(conv3x3_forward(x, w, bias, relu))
+    if bias is not None:
+        _check(bias, "bias")
+        if bias.numel() != k or not bias.is_contiguous():
+            raise ValueError("conv3x3: bias must be a contiguous vector of K=%d" % k)
+    lib = _cabi.lib()
+    nbytes = ctypes.c_uint64()
+    lib.pd_conv3x3_winograd_filter_bytes(c, k, ctypes.byref(nbytes))
+    u = torch.empty(nbytes.value // 4, dtype=torch.float32, device=x.device)
+    lib.pd_conv3x3_winograd_filter_f32(_ptr(w), _ptr(u), c, k, 0, _cabi.stream_ptr())
+    y = torch.empty((n, k, h // 2, wd // 2), dtype=torch.float32, device=x.device,
+                    memory_format=torch.channels_last)
+    idx = torch.empty((n, k, h // 2, wd // 2), dtype=torch.uint8, device=x.device,
+                      memory_format=torch.channels_last)
+    with _timed("conv3x3_winograd_kernel", 18.0 * c * k * n * h * wd):
+        lib.pd_conv3x3_winograd_fwd_pool_nhwc_f32(_ptr(x), _ptr(u), _ptr(bias), _ptr(y), _ptr(idx), n, h, wd, c, k,
+                                                  int(relu), _cabi.stream_ptr())
+    return y, idx
 
 
 def conv3x3_input_grad(dy, w, relu_out=None, x_rectified=None):

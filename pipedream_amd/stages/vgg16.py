@@ -45,11 +45,13 @@ class FrontStage(torch.nn.Module):
         # a pooling layer with relu=True is the identity on the rectified output of the convolution
         # before it and masks the gradient in its backward kernel, so that convolution's gradient
         # kernels read no mask (grad_premasked)
-        self.layer4 = layers.Conv2d(64, 64, relu=True, grad_premasked=True, input_rectified=True)
-        self.layer6 = layers.MaxPool2d(2, 2, relu=True)
+        # (with pool=True the convolution kernel pools in its epilogue; the pooling module keeps its place
+        # in the layer list and passes the tensor through)
+        self.layer4 = layers.Conv2d(64, 64, relu=True, input_rectified=True, pool=True)
+        self.layer6 = layers.MaxPool2d(2, 2, relu=True, applied_by_producer=True)
         self.layer7 = layers.Conv2d(64, 128, relu=True, grad_premasked=True)
-        self.layer9 = layers.Conv2d(128, 128, relu=True, grad_premasked=True, input_rectified=True)
-        self.layer11 = layers.MaxPool2d(2, 2, relu=True)
+        self.layer9 = layers.Conv2d(128, 128, relu=True, input_rectified=True, pool=True)
+        self.layer11 = layers.MaxPool2d(2, 2, relu=True, applied_by_producer=True)
         _initialize_weights(self)
 
     def forward(self, input0):
@@ -78,8 +80,8 @@ class Stage1(torch.nn.Module):
         super(Stage1, self).__init__()
         self.layer2 = layers.MaxPool2d(2, 2, relu=True)    # layer1 ReLU + layer2 MaxPool
         self.layer3 = layers.Conv2d(64, 128, relu=True, grad_premasked=True)    # + layer4; masked by layer5
-        self.layer5 = layers.Conv2d(128, 128, relu=True, grad_premasked=True, input_rectified=True)   # + layer6; masked by layer7
-        self.layer7 = layers.MaxPool2d(2, 2, relu=True)
+        self.layer5 = layers.Conv2d(128, 128, relu=True, input_rectified=True, pool=True)   # + layer6 + layer7
+        self.layer7 = layers.MaxPool2d(2, 2, relu=True, applied_by_producer=True)
         # layer8's ReLU is undone for the gradient by the next stage's first convolution (input_rectified)
         self.layer8 = layers.Conv2d(128, 256, relu=True, grad_premasked=True)   # + layer9
         _initialize_weights(self)
@@ -97,8 +99,8 @@ class Stage2(torch.nn.Module):
     def __init__(self):
         super(Stage2, self).__init__()
         self.layer1 = layers.Conv2d(256, 256, relu=True, grad_premasked=True, input_rectified=True)   # + layer2; masked by layer3
-        self.layer3 = layers.Conv2d(256, 256, relu=True, grad_premasked=True, input_rectified=True)   # + layer4; masked by layer5
-        self.layer5 = layers.MaxPool2d(2, 2, relu=True)
+        self.layer3 = layers.Conv2d(256, 256, relu=True, input_rectified=True, pool=True)   # + layer4 + layer5
+        self.layer5 = layers.MaxPool2d(2, 2, relu=True, applied_by_producer=True)
         self.layer6 = layers.Conv2d(256, 512, relu=True, grad_premasked=True)   # + layer7; masked by layer8
         self.layer8 = layers.Conv2d(512, 512, relu=True, grad_premasked=True, input_rectified=True)   # + layer9
         # layer10's ReLU is undone for the gradient by the next stage's pooling layer (relu=True)
@@ -117,8 +119,8 @@ class Stage3(torch.nn.Module):
         self.layer1 = layers.MaxPool2d(2, 2, relu=True)
         self.layer2 = layers.Conv2d(512, 512, relu=True, grad_premasked=True)   # + layer3; masked by layer4
         self.layer4 = layers.Conv2d(512, 512, relu=True, grad_premasked=True, input_rectified=True)   # + layer5
-        self.layer6 = layers.Conv2d(512, 512, relu=True, grad_premasked=True, input_rectified=True)   # + layer7; masked by layer8
-        self.layer8 = layers.MaxPool2d(2, 2, relu=True)
+        self.layer6 = layers.Conv2d(512, 512, relu=True, input_rectified=True, pool=True)   # + layer7 + layer8
+        self.layer8 = layers.MaxPool2d(2, 2, relu=True, applied_by_producer=True)
         self.flatten = layers.Flatten()
         self.layer11 = layers.Linear(25088, 4096, relu=True)   # + layer12
         self.layer13 = layers.Dropout(p=dropout)

@@ -164,6 +164,49 @@ def test_premasked_layer_chain_matches_unfused_chain():
         assert torch.equal(pa.grad, pb.grad)
 
 
+@pytest.mark.parametrize("N,C,K,H,W", [(2, 16, 32, 12, 12),     # one tile per image
+                                        (1, 64, 64, 32, 48),     # several tiles, one channel block
+                                        (2, 24, 100, 17, 19),    # ragged tiles, odd sizes, K % 64 != 0
+                                        (1, 128, 128, 14, 14),   # the last VGG16 block's size
+                                        (3, 8, 16, 2, 2),        # a single window
+                                        (1, 3, 8, 10, 10)])      # few channels: separate pooling kernel
+def test_convolution_with_pooling_in_its_epilogue_equals_the_two_layers(N, C, K, H, W):
+    """Conv2d(relu=True, pool=True) against the two layers it replaces, under the same algorithm: the pooled
+    output and every gradient bit for bit (the fused epilogue pools the same sums, and both backward passes
+    hand the same masked gradient to the same gradient kernels); the module that keeps the pooling's place
+    in the layer list passes its input through.  The values themselves are checked against torch in fp64,
+    the gradients against the unfused, unflagged layers at the usual tolerance."""
+    torch.manual_seed(N + C + K)
+    plain = torch.nn.Sequential(layers.Conv2d(C, K, relu=True, grad_premasked=True),
+                                layers.MaxPool2d(2, 2, relu=True)).cuda()
+    fused = torch.nn.Sequential(layers.Conv2d(C, K, relu=True, pool=True),
+                                layers.MaxPool2d(2, 2, relu=True, applied_by_producer=True)).cuda()
+    fused.load_state_dict(plain.state_dict())
+    x = torch.randn(N, C, H, W).cuda()
+    xa, xb = x.clone().requires_grad_(True), x.clone().requires_grad_(True)
+    ya, yb = plain(xa), fused(xb)
+    assert ya.shape == (N, K, H // 2, W // 2)
+    assert torch.equal(ya, yb)
+    dy = torch.randn_like(ya)
+    ya.backward(dy)
+    yb.backward(dy)
+    assert torch.equal(xa.grad, xb.grad)
+    for pa, pb in zip(plain.parameters(), fused.parameters()):
+        assert torch.equal(pa.grad, pb.grad)
+    # and against torch (fp64) for the values themselves
+    ref = F.max_pool2d(F.relu(F.conv2d(x.cpu().double(), plain[0].weight.detach().cpu().double(),
+                                       plain[0].bias.detach().cpu().double(), padding=1)), 2, 2)
+    torch.testing.assert_close(yb.detach().cpu().double(), ref, rtol=1e-5, atol=2e-5)
+    simple = torch.nn.Sequential(layers.Conv2d(C, K, relu=True), layers.MaxPool2d(2, 2)).cuda()
+    simple.load_state_dict(plain.state_dict())
+    xc = x.clone().requires_grad_(True)
+    simple(xc).backward(dy)
+    scale = float(xc.grad.abs().max())
+    torch.testing.assert_close(xb.grad, xc.grad, rtol=1e-5, atol=1e-5 * scale)
+    for pc, pb in zip(simple.parameters(), fused.parameters()):
+        torch.testing.assert_close(pb.grad, pc.grad, rtol=1e-5, atol=1e-5 * float(pc.grad.abs().max()))
+
+
 def test_winograd_impulse_response_and_brute_force():
     # the Winograd path on shapes it accepts: (a) brute-force direct convolution of a small case with
     # random (asymmetric) filters; (b) a unit impulse must return the flipped filter taps around it

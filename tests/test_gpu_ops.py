@@ -140,6 +140,43 @@ def test_maxpool_forward_backward_bit_exact(shape):
     assert torch.equal(dxm.cpu(), dx.cpu() * (x.detach() > 0))
 
 
+@pytest.mark.parametrize("shape", [(2, 8, 6, 6), (3, 4, 7, 9), (1, 64, 224, 224), (2, 12, 2, 5), (1, 4, 1, 3)])
+@pytest.mark.parametrize("relu", [False, True])
+def test_maxpool_with_index_bytes_bit_exact(shape, relu):
+    """The pooling the layers use: the forward also writes one byte per output element (window position of
+    the first maximum, sign of the maximum), the backward reads only the pooled gradient and that byte.
+    Against torch's max_pool2d and its autograd (after a ReLU when relu=True), bit for bit, with ties."""
+    g = torch.Generator().manual_seed(3)
+    x = (torch.randn(shape, generator=g) * 2).round() / 2
+    x.requires_grad_(True)
+    if shape[2] >= 2 and shape[3] >= 2:
+        y_ref = F.max_pool2d(F.relu(x) if relu else x, 2, 2)
+    else:       # no window fits (torch refuses such an input): empty output, zero input gradient
+        y_ref = torch.zeros(shape[0], shape[1], shape[2] // 2, shape[3] // 2)
+    dy = torch.randn(y_ref.shape, generator=g)
+    if y_ref.numel():
+        y_ref.backward(dy)
+    want_dx = x.grad if x.grad is not None else torch.zeros(shape)
+    xg = x.detach().cuda().contiguous(memory_format=torch.channels_last)
+    y, idx = ops.maxpool2x2_idx(xg, relu=relu)
+    assert y.shape == y_ref.shape and torch.equal(y.cpu(), y_ref.detach())
+    assert idx.dtype == torch.uint8 and idx.shape == y.shape
+    dx = ops.maxpool2x2_idx_backward(dy.cuda(), idx, shape[2], shape[3], relu_mask=relu)
+    assert dx.shape == x.shape
+    # (relu=True: torch's ReLU passes no gradient at x <= 0; at a window whose maximum is not positive
+    # max_pool2d sends the gradient to its first zero, which the ReLU then drops: zeros either way)
+    assert torch.equal(dx.cpu(), want_dx)
+    # the byte itself: position bits address the maximum, bit 2 says whether it is positive
+    if y.numel():
+        n, c, h, w = shape
+        win = x.detach()[:, :, :h // 2 * 2, :w // 2 * 2].reshape(n, c, h // 2, 2, w // 2, 2).permute(0, 1, 2, 4, 3, 5)
+        win = win.reshape(n, c, h // 2, w // 2, 4)
+        b = idx.cpu().long()
+        picked = torch.gather(win, 4, (b & 3).unsqueeze(-1)).squeeze(-1)
+        assert torch.equal(picked, win.max(dim=4).values)
+        assert torch.equal((b & 4) != 0, picked > 0) and int((b >> 3).max()) == 0
+
+
 @pytest.mark.parametrize("B,C", [(64, 10), (64, 1000), (7, 32320), (1, 3)])
 def test_cross_entropy_vs_torch(B, C):
     g = torch.Generator().manual_seed(2)
