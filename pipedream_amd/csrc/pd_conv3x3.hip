@@ -29,6 +29,8 @@
 //   gradient falls out of the same dY tile.
 #include "pd_internal.h"
 
+#include <type_traits>
+
 typedef float float4_t __attribute__((ext_vector_type(4)));
 typedef float float16_t __attribute__((ext_vector_type(16)));
 
@@ -315,11 +317,15 @@ __global__ __launch_bounds__(CONV_THREADS, 2) void conv3x3_fwd_kernel(const Conv
 // Forward for very few input channels (9*C <= 32: the first VGG layer, C = 3).  The whole
 // reduction (9 taps x C) fits one 32-wide k range, so instead of padding C to 8 per tap the
 // (tap, channel) pairs are packed densely: 16 MFMA k-steps per tile instead of 36.  The A
-// operand is gathered straight from the halo tile with per-lane precomputed offsets; the
-// kernel is bound by writing the output.
-template <int TH, int TW>
+// operand is gathered straight from the halo tile with per-lane offsets.  The kernel writes 64 output
+// values per input value, and its 64 MFMAs per wave are few: everything else a wave executes (index
+// arithmetic, bounds checks, address formation) has to stay well below them, hence C as a template
+// parameter (CT = 0: any C, divisions at run time), halo rows loaded as contiguous runs, and stores
+// whose row and column offsets are scalar.
+template <int TH, int TW, int CT>
 __global__ __launch_bounds__(CONV_THREADS, 2) void conv3x3_fwd_smallc_kernel(const ConvArgs a) {
     static_assert(TH * TW == 256, "a block owns 256 pixels");
+    static_assert(TW == 8 || TW == 16 || TW == 32, "tile widths the pixel mapping of the epilogue assumes");
     constexpr int HW_ = TW + 2;
     constexpr int HALO = (TH + 2) * (TW + 2);
     constexpr int WP = 36;   // filter row pitch (32 k + 4)
@@ -329,7 +335,7 @@ __global__ __launch_bounds__(CONV_THREADS, 2) void conv3x3_fwd_smallc_kernel(con
     const int tid = threadIdx.x;
     const int wave = tid / 64, lane = tid % 64;
     const int idx = lane % 32, h = lane / 32;
-    const int C = a.C, NC = 9 * a.C;
+    const int C = CT ? CT : a.C, NC = 9 * C;
 
     const int xcd = blockIdx.x % N_XCD, seq = blockIdx.x / N_XCD;
     int b = xcd * a.tiles_per_xcd + seq / a.k_blocks;
@@ -340,66 +346,81 @@ __global__ __launch_bounds__(CONV_THREADS, 2) void conv3x3_fwd_smallc_kernel(con
     const int ty = b % a.tiles_y;
     const int n = b / a.tiles_y;
     const int y0 = ty * TH, x0 = tx * TW;
-    const float* xn = a.x + (size_t)n * a.H * a.W * C;
 
-    // stage the halo tile ([pixel][4], zero padded) and the filter ([k][27 -> 32]): all global loads
-    // are issued before the first LDS store, so a block waits for memory once, not once per element
-    constexpr int IN_ITERS = (HALO * 4 + CONV_THREADS - 1) / CONV_THREADS;
-    constexpr int W_ITERS = BN * 32 / CONV_THREADS;
+    // Stage the halo tile ([pixel][4], zero padded) and the filter ([k][9C -> 32]); all global loads are
+    // issued before the first LDS store, so a block waits for memory once.  A halo row is one contiguous
+    // run of (TW + 2) * C floats and the filter block one run of 64 * 9C floats: buffer loads with
+    // out-of-range offsets supply the zero padding.
+    constexpr int ROW_MAX = HW_ * (CT ? CT : 3);              // floats per halo row (9C <= 32: C <= 3)
+    constexpr int IN_ITERS = ((TH + 2) * ROW_MAX + CONV_THREADS - 1) / CONV_THREADS;
+    constexpr int W_ITERS = (BN * 9 * (CT ? CT : 3) + CONV_THREADS - 1) / CONV_THREADS;
+    const int row_len = HW_ * C;
+    const __amdgpu_buffer_rsrc_t xr = __builtin_amdgcn_make_buffer_rsrc(
+        (void*)(a.x + (size_t)n * a.H * a.W * C), 0, (uint32_t)a.H * a.W * C * 4, 0x00020000);
+    const int kn = a.K - k0 < BN ? a.K - k0 : BN;             // filters of this block
+    const __amdgpu_buffer_rsrc_t wr = __builtin_amdgcn_make_buffer_rsrc(
+        (void*)(a.w + (size_t)k0 * NC), 0, (uint32_t)kn * NC * 4, 0x00020000);
     float rin[IN_ITERS], rw[W_ITERS];
 #pragma unroll
     for (int it = 0; it < IN_ITERS; ++it) {
         const int id = tid + it * CONV_THREADS;
-        const int p = id / 4, cc = id % 4;
-        const int gy = y0 + p / HW_ - 1, gx = x0 + p % HW_ - 1;
-        const bool ok = id < HALO * 4 && cc < C && gy >= 0 && gy < a.H && gx >= 0 && gx < a.W;
-        const float v = xn[ok ? ((size_t)gy * a.W + gx) * C + cc : 0];
-        rin[it] = ok ? v : 0.f;
+        const int r = id / row_len, col = id - r * row_len;  // halo row, float within the row
+        const int gy = y0 + r - 1, gxc = (x0 - 1) * C + col;  // image row, float within the image row
+        const bool ok = r < TH + 2 && gy >= 0 && gy < a.H && gxc >= 0 && gxc < a.W * C;
+        rin[it] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(
+                                                xr, ok ? (uint32_t)(gy * a.W * C + gxc) * 4 : 0x80000000u, 0, 0));
     }
 #pragma unroll
-    for (int it = 0; it < W_ITERS; ++it) {
-        const int id = tid + it * CONV_THREADS;
-        const int k = id / 32, kk = id % 32;
-        const bool ok = kk < NC && k0 + k < a.K;
-        const float v = a.w[ok ? (size_t)(k0 + k) * NC + kk : 0];
-        rw[it] = ok ? v : 0.f;
+    for (int it = 0; it < W_ITERS; ++it)
+        rw[it] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(
+                                               wr, (uint32_t)(tid + it * CONV_THREADS) * 4, 0, 0));
+    // the pad lanes of the two tiles (channel 3 of every pixel, reduction indices 9C..31) are zeroed first
+    for (int id = tid; id < HALO + 1; id += CONV_THREADS) in_tile[id * 4 + 3] = 0.f;
+    if (C < 3)
+        for (int id = tid; id < HALO; id += CONV_THREADS) in_tile[id * 4 + 2] = 0.f;
+    if (C < 2)
+        for (int id = tid; id < HALO; id += CONV_THREADS) in_tile[id * 4 + 1] = 0.f;
+    if (tid < 3) in_tile[HALO * 4 + tid] = 0.f;
+    for (int id = tid; id < BN * (32 - NC); id += CONV_THREADS) {
+        const int k = id / (32 - NC);
+        w_tile[k * WP + NC + (id - k * (32 - NC))] = 0.f;
     }
 #pragma unroll
     for (int it = 0; it < IN_ITERS; ++it) {
         const int id = tid + it * CONV_THREADS;
-        if (id < HALO * 4) in_tile[id] = rin[it];
+        const int r = id / row_len, col = id - r * row_len;
+        const int px = col / C, cc = col - px * C;
+        if (r < TH + 2) in_tile[(r * HW_ + px) * 4 + cc] = rin[it];
     }
-    if (tid < 4) in_tile[HALO * 4 + tid] = 0.f;
 #pragma unroll
     for (int it = 0; it < W_ITERS; ++it) {
         const int id = tid + it * CONV_THREADS;
-        w_tile[(id / 32) * WP + id % 32] = rw[it];
+        const int k = id / NC;
+        if (k < BN) w_tile[k * WP + (id - k * NC)] = rw[it];
     }
-    // per-lane gather offsets for the reduction indices kk = 8g + 4h + s
+    // per-lane gather offsets for the reduction indices kk = 8g + 4h + s (two candidates per (g, s), known
+    // at compile time when C is)
     int goff[4][4];
 #pragma unroll
     for (int g = 0; g < 4; ++g)
 #pragma unroll
         for (int s = 0; s < 4; ++s) {
-            const int kk = 8 * g + 4 * h + s;
-            const int tap = kk / C, c = kk % C;
-            goff[g][s] = kk < NC ? ((tap / 3) * HW_ + (tap % 3)) * 4 + c : -1;
+            auto off_of = [&](int kk) {
+                const int tap = kk / C, c = kk % C;
+                return kk < NC ? ((tap / 3) * HW_ + (tap % 3)) * 4 + c : -1;
+            };
+            goff[g][s] = h ? off_of(8 * g + 4 + s) : off_of(8 * g + s);
         }
     __syncthreads();
 
     float16_t acc[2][2];
-#pragma unroll
-    for (int i = 0; i < 2; ++i)
-#pragma unroll
-        for (int j = 0; j < 2; ++j)
-#pragma unroll
-            for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.f;
     int pbase[2];
 #pragma unroll
     for (int i = 0; i < 2; ++i) {
         const int q = (wave * 2 + i) * 32 + idx;
         pbase[i] = ((q / TW) * HW_ + (q % TW)) * 4;
     }
+    const float16_t zero16 = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
 #pragma unroll
     for (int g = 0; g < 4; ++g) {
         float4_t fb[2];
@@ -414,29 +435,46 @@ __global__ __launch_bounds__(CONV_THREADS, 2) void conv3x3_fwd_smallc_kernel(con
             for (int i = 0; i < 2; ++i)
 #pragma unroll
                 for (int j = 0; j < 2; ++j)
-                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(fa[i], fb[j][s], acc[i][j], 0, 0, 0);
+                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(fa[i], fb[j][s],
+                                                                     (g == 0 && s == 0) ? zero16 : acc[i][j], 0, 0, 0);
         }
     }
 
-    float* yn = a.y + (size_t)n * a.H * a.W * a.K;
+    // Epilogue: 64 dword stores per lane (lanes 0-31 = 32 consecutive channels of one pixel: 128-byte runs).
+    // One per-lane byte offset; the pixel's row and column go into a scalar offset.  Accumulator element e
+    // of tile i is pixel q = (wave*2 + i)*32 + 8*(e/4) + 4h + e%4 of the block, row q / TW, column q % TW (the
+    // column part 4h + e%4 < 8 never carries into the row).  Pixels and channels outside the tensor get an
+    // offset beyond the buffer, which drops the store; a block whose tile lies inside the image skips the
+    // per-pixel test.
+    const uint32_t img_bytes = (uint32_t)a.H * a.W * a.K * 4;
+    const __amdgpu_buffer_rsrc_t yr = __builtin_amdgcn_make_buffer_rsrc(
+        (void*)(a.y + (size_t)n * a.H * a.W * a.K), 0, img_bytes, 0x00020000);
+    const bool full_tile = y0 + TH <= a.H && x0 + TW <= a.W;          // block-uniform
+    const int rows_left = a.H - y0 - wave * (64 / TW);                 // wave-uniform
+    const int cols_left = a.W - x0 - 4 * h;
+    auto store_all = [&](auto full) {
 #pragma unroll
-    for (int j = 0; j < 2; ++j) {
-        const int k = k0 + j * 32 + idx;
-        if (k >= a.K) continue;
-        const float bv = a.bias ? a.bias[k] : 0.f;
+        for (int j = 0; j < 2; ++j) {
+            const int k = k0 + j * 32 + idx;
+            const float bv = (a.bias && k < a.K) ? a.bias[k] : 0.f;
+            const uint32_t lane_off = k < a.K ? (uint32_t)((y0 * a.W + x0 + 4 * h) * a.K + k) * 4 : 0x80000000u;
 #pragma unroll
-        for (int i = 0; i < 2; ++i)
+            for (int i = 0; i < 2; ++i)
 #pragma unroll
-            for (int e = 0; e < 16; ++e) {
-                const int q = (wave * 2 + i) * 32 + 8 * (e / 4) + 4 * h + (e % 4);
-                const int gy = y0 + q / TW, gx = x0 + q % TW;
-                if (gy < a.H && gx < a.W) {
+                for (int e = 0; e < 16; ++e) {
+                    const int qq = i * 32 + 8 * (e / 4) + (e % 4);
+                    const int r_rel = qq / TW, c_rel = qq % TW;              // compile-time
+                    const int soff = ((wave * (64 / TW) + r_rel) * a.W + c_rel) * (a.K * 4);   // wave-uniform
                     float v = acc[i][j][e] + bv;
                     if (a.relu) v = v > 0.f ? v : 0.f;
-                    yn[((size_t)gy * a.W + gx) * a.K + k] = v;
+                    const uint32_t voff =
+                        (decltype(full)::value || (r_rel < rows_left && c_rel < cols_left)) ? lane_off : 0x80000000u;
+                    __builtin_amdgcn_raw_buffer_store_b32(__builtin_bit_cast(uint32_t, v), yr, voff, soff, 0);
                 }
-            }
-    }
+        }
+    };
+    if (full_tile) store_all(std::true_type{});
+    else store_all(std::false_type{});
 }
 
 // w[K][3][3][C]  ->  out[C][3][3][K] with out[c][r][s][k] = w[k][2-r][2-s][c].
@@ -920,6 +958,147 @@ __global__ __launch_bounds__(CONV_THREADS, 2) void conv3x3_wgrad_smallc_kernel(c
             (bsum_tile[tid] + bsum_tile[64 + tid]) + (bsum_tile[128 + tid] + bsum_tile[192 + tid]);
 }
 
+// The same few-channel weight gradient with the per-MFMA overhead removed (dY rows of whole float4, no
+// ReLU mask, an image addressable with 32-bit byte offsets): the multiply loop is fully unrolled and every
+// LDS address in it is a per-lane base plus a compile-time offset (lanes of unused columns point at a
+// region of zeros, the lanes of column 9C at a region of ones, so that column accumulates the bias
+// gradient); tiles are fetched with buffer loads whose out-of-range offsets supply the zero padding, with
+// per-lane offsets computed once and the tile's position as a scalar offset.
+template <int TH, int TW>
+__global__ __launch_bounds__(CONV_THREADS, 2) void conv3x3_wgrad_smallc_fast_kernel(const WgradArgs a) {
+    constexpr int PIX = TH * TW;
+    constexpr int HW_ = TW + 2;
+    constexpr int HALO = (TH + 2) * (TW + 2);
+    constexpr int CS = 64;
+    constexpr int WROWS = PIX / 4 / TW;                          // pixel rows per wave
+    static_assert(PIX % (4 * TW) == 0 && TW % 2 == 0, "a wave owns whole pixel rows, pixels in pairs");
+    constexpr int ZR = ((WROWS - 1) * HW_ + TW) * 4 + 4;        // floats a compile-time offset can reach
+    __shared__ __attribute__((aligned(16))) float dy_tile[PIX * CS];
+    __shared__ float x_tile[HALO * 4 + 2 * ZR];                 // [halo pixel][4], zeros, ones
+
+    const int tid = threadIdx.x;
+    const int wave = tid / 64, lane = tid % 64;
+    const int idx = lane % 32, h = lane / 32;
+    const int k0 = blockIdx.y * 64;
+    const int C = a.C, NC = 9 * a.C;
+    const int tap = idx / C, c = idx % C;
+    const int xbase = idx < NC ? (wave * WROWS * HW_ + h) * 4 + ((tap / 3) * HW_ + (tap % 3)) * 4 + c
+                               : (idx == NC ? HALO * 4 + ZR : HALO * 4);
+    const int dybase = (wave * (PIX / 4) + h) * CS + idx;
+    for (int i = tid; i < ZR; i += CONV_THREADS) {
+        x_tile[HALO * 4 + i] = 0.f;
+        x_tile[HALO * 4 + ZR + i] = 1.f;
+    }
+
+    float16_t acc[2];
+#pragma unroll
+    for (int t = 0; t < 2; ++t)
+#pragma unroll
+        for (int e = 0; e < 16; ++e) acc[t][e] = 0.f;
+
+    // loader roles, fixed for the whole kernel
+    constexpr int DY_ITERS = PIX * (CS / 4) / CONV_THREADS;
+    constexpr int X_ITERS = ((TH + 2) * HW_ * 3 + CONV_THREADS - 1) / CONV_THREADS;     // C <= 3
+    const int row_len = HW_ * C;
+    int dy_row[DY_ITERS], dy_col[DY_ITERS];
+    uint32_t dy_lane[DY_ITERS];              // byte offset inside the tile's part of the image
+#pragma unroll
+    for (int it = 0; it < DY_ITERS; ++it) {
+        const int id = tid + it * CONV_THREADS;
+        const int p = id / (CS / 4), q4 = (id % (CS / 4)) * 4;
+        dy_row[it] = k0 + q4 < a.K ? p / TW : (1 << 30);        // channels beyond K: never inside
+        dy_col[it] = p % TW;
+        dy_lane[it] = (uint32_t)(((p / TW) * a.W + p % TW) * a.K + q4) * 4;
+    }
+    int x_row[X_ITERS], x_col[X_ITERS], x_lds[X_ITERS], x_lane[X_ITERS];
+#pragma unroll
+    for (int it = 0; it < X_ITERS; ++it) {
+        const int id = tid + it * CONV_THREADS;
+        const int r = id / row_len, col = id - r * row_len;
+        x_row[it] = r < TH + 2 ? r : (1 << 30);
+        x_col[it] = col;
+        x_lds[it] = r < TH + 2 ? (r * HW_ + col / C) * 4 + col % C : -1;
+        x_lane[it] = (r * a.W * C + col) * 4;
+    }
+    const uint32_t dy_img_bytes = (uint32_t)a.H * a.W * a.K * 4, x_img_bytes = (uint32_t)a.H * a.W * C * 4;
+
+    float4_t rdy[DY_ITERS];
+    float rx[X_ITERS];
+    auto load_tile = [&](int tile) {
+        int b = tile;
+        const int tx = b % a.tiles_x;
+        b /= a.tiles_x;
+        const int ty = b % a.tiles_y;
+        const int n = b / a.tiles_y;
+        const int y0 = ty * TH, x0 = tx * TW;
+        const __amdgpu_buffer_rsrc_t dr = __builtin_amdgcn_make_buffer_rsrc(
+            (void*)(a.dy + (size_t)n * a.H * a.W * a.K), 0, dy_img_bytes, 0x00020000);
+        const __amdgpu_buffer_rsrc_t xr = __builtin_amdgcn_make_buffer_rsrc(
+            (void*)(a.x + (size_t)n * a.H * a.W * C), 0, x_img_bytes, 0x00020000);
+        const int rows_left = a.H - y0, cols_left = a.W - x0;
+        const int dy_soff = ((y0 * a.W + x0) * a.K + k0) * 4;
+#pragma unroll
+        for (int it = 0; it < DY_ITERS; ++it) {
+            const bool ok = dy_row[it] < rows_left && dy_col[it] < cols_left;
+            rdy[it] = __builtin_bit_cast(
+                float4_t, __builtin_amdgcn_raw_buffer_load_b128(dr, ok ? dy_lane[it] : 0x80000000u, dy_soff, 0));
+        }
+        // halo rows start one pixel up and left of the tile: the tile's offset may be negative, so it
+        // goes into the per-lane offset
+        const int x_toff = ((y0 - 1) * a.W + (x0 - 1)) * C * 4;
+        const int xc0 = (x0 - 1) * C;
+#pragma unroll
+        for (int it = 0; it < X_ITERS; ++it) {
+            const int gy = y0 - 1 + x_row[it], gxc = xc0 + x_col[it];
+            const bool ok = gy >= 0 && gy < a.H && gxc >= 0 && gxc < a.W * C;
+            rx[it] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(
+                                                   xr, ok ? (uint32_t)(x_lane[it] + x_toff) : 0x80000000u, 0, 0));
+        }
+    };
+    if ((int)blockIdx.x < a.n_tiles) load_tile(blockIdx.x);
+
+    for (int tile = blockIdx.x; tile < a.n_tiles; tile += gridDim.x) {
+        __syncthreads();  // previous tile fully consumed
+#pragma unroll
+        for (int it = 0; it < DY_ITERS; ++it) *(float4_t*)(dy_tile + (tid + it * CONV_THREADS) * 4) = rdy[it];
+#pragma unroll
+        for (int it = 0; it < X_ITERS; ++it)
+            if (x_lds[it] >= 0) x_tile[x_lds[it]] = rx[it];
+        __syncthreads();
+        if (tile + (int)gridDim.x < a.n_tiles) load_tile(tile + gridDim.x);
+        // this wave's quarter of the pixels, two per MFMA (pixel 2pp + h of the wave's rows)
+#pragma unroll
+        for (int pp = 0; pp < PIX / 8; ++pp) {
+            const float a0 = dy_tile[dybase + 2 * pp * CS];
+            const float a1 = dy_tile[dybase + 2 * pp * CS + 32];
+            const float bv = x_tile[xbase + (((2 * pp) / TW) * HW_ + (2 * pp) % TW) * 4];
+            acc[0] = __builtin_amdgcn_mfma_f32_32x32x2f32(a0, bv, acc[0], 0, 0, 0);
+            acc[1] = __builtin_amdgcn_mfma_f32_32x32x2f32(a1, bv, acc[1], 0, 0, 0);
+        }
+    }
+
+    // the four waves' sums (each covered a quarter of every tile's pixels) are added in wave order
+    // through the now idle dy tile, so the block writes one partial; column 9C is the bias gradient
+    __syncthreads();
+#pragma unroll
+    for (int t = 0; t < 2; ++t)
+#pragma unroll
+        for (int e = 0; e < 16; ++e) dy_tile[(wave * 32 + t * 16 + e) * 64 + lane] = acc[t][e];
+    __syncthreads();
+    float* pw = a.part_w + (size_t)blockIdx.x * a.K * NC;
+#pragma unroll
+    for (int it = 0; it < 32 * 64 / CONV_THREADS; ++it) {
+        const int id = tid + it * CONV_THREADS;          // (t, e, lane) of an accumulator element
+        const int te = id / 64, ln = id % 64;
+        const float v = (dy_tile[te * 64 + ln] + dy_tile[(32 + te) * 64 + ln]) +
+                        (dy_tile[(64 + te) * 64 + ln] + dy_tile[(96 + te) * 64 + ln]);
+        const int t = te / 16, e = te % 16, col = ln % 32;
+        const int k = k0 + t * 32 + 8 * (e / 4) + 4 * (ln / 32) + (e % 4);
+        if (col < NC && k < a.K) pw[(size_t)k * NC + col] = v;
+        if (col == NC && k < a.K && a.part_b) a.part_b[(size_t)blockIdx.x * a.K + k] = v;
+    }
+}
+
 // out[i] = sum_b part[b][i] in a fixed order (deterministic).  A block owns 64 outputs;
 // its 4 waves each sum a quarter of the partials, then combine through LDS.
 __global__ __launch_bounds__(256) void reduce_partials_kernel(const float* __restrict__ part, float* __restrict__ out,
@@ -1007,9 +1186,12 @@ static int conv3x3_fwd_launch(const float* x, const float* w, const float* bias,
     dim3 grid((unsigned)nblk);                       // one block per (pixel tile, out-channel block)
     hipStream_t s = (hipStream_t)stream;
     const bool small_c = C <= 8;
+    // the few-channel kernel addresses one image with 32-bit byte offsets
+    const bool dense_taps = 9 * C <= 32 && !mask && !out_mask && (long)H * W * (K > C ? K : C) * 4 < (1L << 31);
 #define PD_LAUNCH_FWD(TH_, TW_)                                                                        \
     do {                                                                                               \
-        if (9 * C <= 32 && !mask && !out_mask) conv3x3_fwd_smallc_kernel<TH_, TW_><<<grid, CONV_THREADS, 0, s>>>(a); \
+        if (dense_taps && C == 3) conv3x3_fwd_smallc_kernel<TH_, TW_, 3><<<grid, CONV_THREADS, 0, s>>>(a);  \
+        else if (dense_taps) conv3x3_fwd_smallc_kernel<TH_, TW_, 0><<<grid, CONV_THREADS, 0, s>>>(a);       \
         else if (!a.c_vec && mask) conv3x3_fwd_kernel<TH_, TW_, 8, true, false><<<grid, CONV_THREADS, 0, s>>>(a); \
         else if (!a.c_vec) conv3x3_fwd_kernel<TH_, TW_, 8, false, false><<<grid, CONV_THREADS, 0, s>>>(a);  \
         else if (small_c && mask) conv3x3_fwd_kernel<TH_, TW_, 8, true, true><<<grid, CONV_THREADS, 0, s>>>(a); \
@@ -1085,7 +1267,11 @@ extern "C" int pd_conv3x3_wgrad_nhwc_f32(const float* x, const float* dy, const 
     hipStream_t s = (hipStream_t)stream;
     if (small_c) {
         dim3 grid(nblk, (K + 63) / 64);
-        conv3x3_wgrad_smallc_kernel<WGRAD_TH, WGRAD_TW><<<grid, CONV_THREADS, 0, s>>>(a);
+        // the lean kernel: whole float4 of dY, no ReLU mask, 32-bit byte offsets inside one image
+        if (a.k_vec && !relu_out && (long)H * W * (K > C ? K : C) * 4 < (1L << 31))
+            conv3x3_wgrad_smallc_fast_kernel<WGRAD_TH, WGRAD_TW><<<grid, CONV_THREADS, 0, s>>>(a);
+        else
+            conv3x3_wgrad_smallc_kernel<WGRAD_TH, WGRAD_TW><<<grid, CONV_THREADS, 0, s>>>(a);
     } else {
         dim3 grid(nblk, (K + 63) / 64, (C + 63) / 64);
         if (a.c_vec && a.k_vec && relu_out) conv3x3_wgrad_pipe_kernel<WGRAD_TH, WGRAD_TW, true><<<grid, WGP_THREADS, 0, s>>>(a);

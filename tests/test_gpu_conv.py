@@ -75,6 +75,11 @@ SHAPES = [
     (3, 5, 6, 8, 8),         # C not a multiple of 4: scalar load path
     (1, 64, 64, 7, 19),      # odd height and width: half tiles at the image edges (Winograd strips)
     (3, 128, 64, 9, 40),
+    (2, 3, 64, 17, 19),      # 3 channels, ragged tiles on both edges
+    (1, 3, 40, 9, 70),       # 3 channels, wide-tile shape, fewer filters than a block
+    (2, 3, 100, 40, 7),      # 3 channels, tall-tile shape, two filter blocks (the second ragged)
+    (1, 2, 8, 5, 40),        # 2 and 1 channels: the dense-tap kernel with run-time channel count
+    (2, 1, 16, 33, 9),
 ]
 
 
