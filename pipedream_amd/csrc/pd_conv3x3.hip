@@ -477,6 +477,200 @@ __global__ __launch_bounds__(CONV_THREADS, 2) void conv3x3_fwd_smallc_kernel(con
     else store_all(std::false_type{});
 }
 
+// The same kernel for a layer with a single block of output channels (K <= 64), as a persistent loop: a
+// block keeps the filter in LDS, walks over pixel tiles of its die's range and requests tile t+1's halo
+// rows before it multiplies and stores tile t, so that neither the load latency nor the draining of the
+// stores sits between two tiles' MFMAs (the loads are older than the stores, so waiting for them leaves
+// the stores in flight).  One barrier per tile: the halo tile is double-buffered.
+template <int TH, int TW, int CT>
+__global__ __launch_bounds__(CONV_THREADS, 4) void conv3x3_fwd_smallc_persist_kernel(const ConvArgs a) {
+    constexpr int KT = BN;          // exactly one full block of output channels: column offsets of the
+                                    // stores become instruction immediates
+    static_assert(TH * TW == 256, "a block owns 256 pixels");
+    static_assert(TW == 8 || TW == 16 || TW == 32, "tile widths the pixel mapping of the epilogue assumes");
+    constexpr int HW_ = TW + 2;
+    constexpr int HALO = (TH + 2) * (TW + 2);
+    constexpr int WP = 36;
+    constexpr int IN_STAGE = HALO * 4 + 4;
+    __shared__ float in_tile[2 * IN_STAGE];
+    __shared__ __attribute__((aligned(16))) float w_tile[BN * WP];
+
+    const int tid = threadIdx.x;
+    const int wave = tid / 64, lane = tid % 64;
+    const int idx = lane % 32, h = lane / 32;
+    const int C = CT ? CT : a.C, NC = 9 * C;
+
+    // tiles xcd * tiles_per_xcd + slot + i * slots of die xcd = blockIdx.x % 8
+    const int xcd = blockIdx.x % N_XCD, slot = blockIdx.x / N_XCD, slots = gridDim.x / N_XCD;
+    int t_lim = a.n_tiles - xcd * a.tiles_per_xcd;
+    t_lim = t_lim < a.tiles_per_xcd ? t_lim : a.tiles_per_xcd;
+    if (slot >= t_lim) return;                                   // whole block, before any barrier
+    const int tile0 = xcd * a.tiles_per_xcd + slot;
+    const int n_my = (t_lim - slot + slots - 1) / slots;
+
+    constexpr int ROW_MAX = HW_ * (CT ? CT : 3);
+    constexpr int IN_ITERS = ((TH + 2) * ROW_MAX + CONV_THREADS - 1) / CONV_THREADS;
+    constexpr int W_ITERS = (BN * 9 * (CT ? CT : 3) + CONV_THREADS - 1) / CONV_THREADS;
+    const int row_len = HW_ * C;
+    // loader roles, fixed for the whole kernel: halo row r, float col of that row
+    int in_row[IN_ITERS], in_col[IN_ITERS], in_lds[IN_ITERS];
+#pragma unroll
+    for (int it = 0; it < IN_ITERS; ++it) {
+        const int id = tid + it * CONV_THREADS;
+        const int r = id / row_len, col = id - r * row_len;
+        const int px = col / C, cc = col - px * C;
+        in_row[it] = r < TH + 2 ? r : (1 << 30);
+        in_col[it] = col;
+        in_lds[it] = r < TH + 2 ? (r * HW_ + px) * 4 + cc : -1;
+    }
+    const uint32_t x_img_bytes = (uint32_t)a.H * a.W * C * 4;
+    float rin[IN_ITERS];
+    struct Pos { int n, y0, x0; };
+    auto decode = [&](int tile) {
+        Pos p;
+        int b = tile;
+        const int tx = b % a.tiles_x;
+        b /= a.tiles_x;
+        p.y0 = (b % a.tiles_y) * TH;
+        p.n = b / a.tiles_y;
+        p.x0 = tx * TW;
+        return p;
+    };
+    auto load_halo = [&](int tile) {
+        const Pos p = decode(tile);
+        const __amdgpu_buffer_rsrc_t xr = __builtin_amdgcn_make_buffer_rsrc(
+            (void*)(a.x + (size_t)p.n * a.H * a.W * C), 0, x_img_bytes, 0x00020000);
+        const int xc0 = (p.x0 - 1) * C;
+#pragma unroll
+        for (int it = 0; it < IN_ITERS; ++it) {
+            const int gy = p.y0 - 1 + in_row[it], gxc = xc0 + in_col[it];
+            const bool ok = gy >= 0 && gy < a.H && gxc >= 0 && gxc < a.W * C;
+            rin[it] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(
+                                                    xr, ok ? (uint32_t)(gy * a.W * C + gxc) * 4 : 0x80000000u, 0, 0));
+        }
+    };
+    auto store_halo = [&](int stage) {
+#pragma unroll
+        for (int it = 0; it < IN_ITERS; ++it)
+            if (in_lds[it] >= 0) in_tile[stage * IN_STAGE + in_lds[it]] = rin[it];
+    };
+
+    load_halo(tile0);
+    {
+        // the filter block ([k][9C -> 32], zero padded), once
+        const __amdgpu_buffer_rsrc_t wr =
+            __builtin_amdgcn_make_buffer_rsrc((void*)a.w, 0, (uint32_t)KT * NC * 4, 0x00020000);
+        float rw[W_ITERS];
+#pragma unroll
+        for (int it = 0; it < W_ITERS; ++it)
+            rw[it] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(
+                                                   wr, (uint32_t)(tid + it * CONV_THREADS) * 4, 0, 0));
+        for (int id = tid; id < BN * (32 - NC); id += CONV_THREADS) {
+            const int k = id / (32 - NC);
+            w_tile[k * WP + NC + (id - k * (32 - NC))] = 0.f;
+        }
+#pragma unroll
+        for (int it = 0; it < W_ITERS; ++it) {
+            const int id = tid + it * CONV_THREADS;
+            const int k = id / NC;
+            if (k < BN) w_tile[k * WP + (id - k * NC)] = rw[it];
+        }
+    }
+    // pad lanes of both halo stages (channels C..3 of every pixel, and the all-zero pixel behind the tile)
+    for (int id = tid; id < 2 * IN_STAGE; id += CONV_THREADS) {
+        const int o = id % IN_STAGE;
+        if (o >= HALO * 4 || (o & 3) >= C) in_tile[id] = 0.f;
+    }
+    store_halo(0);
+
+    int goff[4][4];
+#pragma unroll
+    for (int g = 0; g < 4; ++g)
+#pragma unroll
+        for (int s = 0; s < 4; ++s) {
+            auto off_of = [&](int kk) {
+                const int tap = kk / C, c = kk % C;
+                return kk < NC ? ((tap / 3) * HW_ + (tap % 3)) * 4 + c : HALO * 4 - 0;
+            };
+            goff[g][s] = h ? off_of(8 * g + 4 + s) : off_of(8 * g + s);
+        }
+    // per-lane LDS offsets of the two pixels this lane feeds; unused reduction indices read the zero
+    // pixel (its offset is absolute: the pixel base must not be added, hence the flag)
+    int pbase[2];
+#pragma unroll
+    for (int i = 0; i < 2; ++i) {
+        const int q = (wave * 2 + i) * 32 + idx;
+        pbase[i] = ((q / TW) * HW_ + (q % TW)) * 4;
+    }
+    const float bv0 = a.bias ? a.bias[idx] : 0.f;
+    const float bv1 = a.bias ? a.bias[32 + idx] : 0.f;
+    const uint32_t y_img_bytes = (uint32_t)a.H * a.W * KT * 4;
+    const float16_t zero16 = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+    __syncthreads();
+
+    for (int ti = 0; ti < n_my; ++ti) {
+        const int tile = tile0 + ti * slots;
+        const float* cur = in_tile + (ti & 1) * IN_STAGE;
+        if (ti + 1 < n_my) load_halo(tile + slots);
+        float16_t acc[2][2];
+#pragma unroll
+        for (int g = 0; g < 4; ++g) {
+            float4_t fb[2];
+#pragma unroll
+            for (int j = 0; j < 2; ++j) fb[j] = *(const float4_t*)(w_tile + (j * 32 + idx) * WP + 8 * g + 4 * h);
+#pragma unroll
+            for (int s = 0; s < 4; ++s) {
+                const bool used = goff[g][s] < HALO * 4;
+                float fa[2];
+#pragma unroll
+                for (int i = 0; i < 2; ++i) fa[i] = cur[used ? pbase[i] + goff[g][s] : HALO * 4];
+#pragma unroll
+                for (int i = 0; i < 2; ++i)
+#pragma unroll
+                    for (int j = 0; j < 2; ++j)
+                        acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(
+                            fa[i], fb[j][s], (g == 0 && s == 0) ? zero16 : acc[i][j], 0, 0, 0);
+            }
+        }
+        // The next tile's halo goes to LDS before this tile's stores are issued: the memory counter retires
+        // in order, so waiting for those loads behind 64 fresh stores would wait for the stores to drain.
+        if (ti + 1 < n_my) store_halo((ti + 1) & 1);
+        // stores: see conv3x3_fwd_smallc_kernel
+        const Pos p = decode(tile);
+        const __amdgpu_buffer_rsrc_t yr = __builtin_amdgcn_make_buffer_rsrc(
+            (void*)(a.y + (size_t)p.n * a.H * a.W * KT), 0, y_img_bytes, 0x00020000);
+        const bool full_tile = p.y0 + TH <= a.H && p.x0 + TW <= a.W;
+        const int rows_left = a.H - p.y0 - wave * (64 / TW);
+        const int cols_left = a.W - p.x0 - 4 * h;
+        auto store_all = [&](auto full) {
+#pragma unroll
+            for (int j = 0; j < 2; ++j) {
+                const int k = j * 32 + idx;
+                const float bv = j ? bv1 : bv0;
+                const uint32_t lane_off = (uint32_t)((p.y0 * a.W + p.x0 + 4 * h) * KT + k) * 4;
+#pragma unroll
+                for (int i = 0; i < 2; ++i)
+#pragma unroll
+                    for (int e = 0; e < 16; ++e) {
+                        const int qq = i * 32 + 8 * (e / 4) + (e % 4);
+                        const int r_rel = qq / TW, c_rel = qq % TW;
+                        const int soff = (wave * (64 / TW) + r_rel) * a.W * (KT * 4);     // row: scalar
+                        float v = acc[i][j][e] + bv;
+                        if (a.relu) v = v > 0.f ? v : 0.f;
+                        const uint32_t voff = (decltype(full)::value || (r_rel < rows_left && c_rel < cols_left))
+                                                  ? lane_off : 0x80000000u;
+                        // column: a constant, folded into the instruction's offset field
+                        __builtin_amdgcn_raw_buffer_store_b32(__builtin_bit_cast(uint32_t, v), yr,
+                                                              voff + c_rel * (KT * 4), soff, 0);
+                    }
+            }
+        };
+        if (full_tile) store_all(std::true_type{});
+        else store_all(std::false_type{});
+        __syncthreads();
+    }
+}
+
 // w[K][3][3][C]  ->  out[C][3][3][K] with out[c][r][s][k] = w[k][2-r][2-s][c].
 __global__ __launch_bounds__(256) void filter_rot180_kernel(const float* __restrict__ w, float* __restrict__ out,
                                                             int K, int C) {
@@ -1187,10 +1381,20 @@ static int conv3x3_fwd_launch(const float* x, const float* w, const float* bias,
     hipStream_t s = (hipStream_t)stream;
     const bool small_c = C <= 8;
     // the few-channel kernel addresses one image with 32-bit byte offsets
+    // persistent variant: four blocks per CU, in multiples of the number of dies
+    int dev = 0, cus = 0;
+    PD_HIP(hipGetDevice(&dev));
+    PD_HIP(hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev));
+    long pblocks = 4L * (cus / N_XCD) * N_XCD;
+    if (pblocks < N_XCD) pblocks = N_XCD;
+    if (pblocks > (long)a.tiles_per_xcd * N_XCD) pblocks = (long)a.tiles_per_xcd * N_XCD;
+    const dim3 pgrid((unsigned)pblocks);
     const bool dense_taps = 9 * C <= 32 && !mask && !out_mask && (long)H * W * (K > C ? K : C) * 4 < (1L << 31);
 #define PD_LAUNCH_FWD(TH_, TW_)                                                                        \
     do {                                                                                               \
-        if (dense_taps && C == 3) conv3x3_fwd_smallc_kernel<TH_, TW_, 3><<<grid, CONV_THREADS, 0, s>>>(a);  \
+        if (dense_taps && K == BN && C == 3)                                                            \
+            conv3x3_fwd_smallc_persist_kernel<TH_, TW_, 3><<<pgrid, CONV_THREADS, 0, s>>>(a);          \
+        else if (dense_taps && C == 3) conv3x3_fwd_smallc_kernel<TH_, TW_, 3><<<grid, CONV_THREADS, 0, s>>>(a);  \
         else if (dense_taps) conv3x3_fwd_smallc_kernel<TH_, TW_, 0><<<grid, CONV_THREADS, 0, s>>>(a);       \
         else if (!a.c_vec && mask) conv3x3_fwd_kernel<TH_, TW_, 8, true, false><<<grid, CONV_THREADS, 0, s>>>(a); \
         else if (!a.c_vec) conv3x3_fwd_kernel<TH_, TW_, 8, false, false><<<grid, CONV_THREADS, 0, s>>>(a);  \
