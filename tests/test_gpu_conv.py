@@ -106,6 +106,61 @@ def test_forward_backward_vs_library(N, C, K, H, W):
     torch.testing.assert_close(db.cpu().double(), bd.grad, rtol=1e-5, atol=4e-7 * math.sqrt(R) * 4)
 
 
+def _random_shapes(count, seed):
+    rng = np.random.RandomState(seed)
+    shapes = []
+    for _ in range(count):
+        c = int(rng.choice([1, 2, 3, 4, 5, 8, 12, 16, 24, 40, 64, 72, 128]))
+        k = int(rng.choice([1, 4, 6, 8, 20, 32, 36, 64, 100, 128]))
+        shapes.append((int(rng.randint(1, 4)), c, k, int(rng.randint(1, 41)), int(rng.randint(1, 41))))
+    return shapes
+
+
+@pytest.mark.parametrize("N,C,K,H,W", _random_shapes(24, seed=20))
+def test_layer_on_random_shapes_vs_library(N, C, K, H, W):
+    """Seeded sweep over channel counts and image sizes on both sides of every kernel's dispatch conditions
+    (few-channel, vector / scalar loads, Winograd and its ragged tiles, partial filter blocks): the layer
+    with fused ReLU, and with the pooling in its epilogue where a window fits, against torch in fp64 --
+    output, input gradient, weight and bias gradients."""
+    g = torch.Generator().manual_seed(N + 10 * C + 1000 * K + H * W)
+    x = torch.randn(N, C, H, W, generator=g)
+    # (the pooling kernels take channel counts that are multiples of 4)
+    for pool in ([False, True] if H >= 2 and W >= 2 and K % 4 == 0 else [False]):
+        layer = layers.Conv2d(C, K, relu=True, pool=pool)
+        w, b = layer.weight.detach().clone(), layer.bias.detach().clone()
+        layer = layer.cuda()
+        xd, wd, bd = x.double().requires_grad_(), w.double().requires_grad_(), b.double().requires_grad_()
+        y_ref = F.relu(F.conv2d(xd, wd, bd, padding=1))
+        if pool:
+            y_ref = F.max_pool2d(y_ref, 2, 2)
+        dy = torch.randn(y_ref.shape, generator=g)
+        # A pre-activation within rounding of 0, or two window elements within rounding of each other, may
+        # fall on the other side in fp32 and move a gradient entry to another place: such outputs get no
+        # upstream gradient (a handful at most; the values themselves are still compared).
+        pre = F.conv2d(xd.detach(), wd.detach(), bd.detach(), padding=1)
+        if pool:
+            r = F.relu(pre)[:, :, :H // 2 * 2, :W // 2 * 2]
+            win = r.reshape(N, K, H // 2, 2, W // 2, 2).permute(0, 1, 2, 4, 3, 5).reshape(N, K, H // 2, W // 2, 4)
+            top = win.sort(dim=4, descending=True).values
+            pw = pre[:, :, :H // 2 * 2, :W // 2 * 2].reshape(N, K, H // 2, 2, W // 2, 2).permute(0, 1, 2, 4, 3, 5)
+            clear = (pw.reshape(N, K, H // 2, W // 2, 4).abs() > 1e-4).all(dim=4)
+            safe = clear & ((top[..., 0] == 0) | (top[..., 0] - top[..., 1] > 1e-4))
+        else:
+            safe = pre.abs() > 1e-4
+        dy = dy * safe
+        y_ref.backward(dy.double())
+        xg = x.cuda().requires_grad_(True)
+        y = layer(xg)
+        assert y.shape == y_ref.shape
+        torch.testing.assert_close(y.detach().cpu().double(), y_ref.detach(), rtol=1e-5,
+                                   atol=4e-7 * math.sqrt(9 * C) * 4)
+        y.backward(dy.cuda())
+        scale = lambda t: float(t.abs().max()) + 1e-30
+        torch.testing.assert_close(xg.grad.cpu().double(), xd.grad, rtol=1e-5, atol=2e-5 * scale(xd.grad))
+        torch.testing.assert_close(layer.weight.grad.cpu().double(), wd.grad, rtol=1e-5, atol=2e-5 * scale(wd.grad))
+        torch.testing.assert_close(layer.bias.grad.cpu().double(), bd.grad, rtol=1e-5, atol=2e-5 * scale(bd.grad))
+
+
 def test_fused_relu_and_no_bias():
     g = torch.Generator().manual_seed(7)
     x = torch.randn(2, 16, 12, 12, generator=g)
