@@ -272,3 +272,33 @@ def test_reference_gnmt_stage0_with_criterion_and_stashed_adam_matches_oracle():
         torch.testing.assert_close(got[key].cpu(), v, rtol=1e-5, atol=5e-2 * kw["lr"],
                                    msg=lambda m, key=key: "%s: %s" % (key, m))
         assert float((got[key].cpu().double() - v.double()).norm() / v.double().norm()) < 1e-5, key
+
+
+def test_full_size_reference_gnmt_stage0_forward_backward():
+    """The reference's stage 0 at its real size (vocabulary 32320, hidden 1024, T = 50, batch 128, sequence
+    lengths between 1 and 50, 91 million parameters): one forward/backward against the CPU oracle, compared
+    in relative L2 norm."""
+    from pipedream_amd.stages import gnmt
+    torch.manual_seed(9)
+    ref = models.GnmtBidirStage0(dropout=0.0)
+    mine = _copy_params(gnmt.BidirStage0(dropout=0.0), ref)
+    g = torch.Generator().manual_seed(10)
+    T, B = 50, 128
+    lt = torch.randint(1, T + 1, (B,), generator=g).sort(descending=True).values
+    lt[0] = T
+    ids = torch.randint(1, 32320, (T, B), generator=g) * sq.set_mask(lt).long()
+    d17 = torch.randn(T, B, 1024, generator=g) * 1e-2
+    d21 = torch.randn(T, B, 1024, generator=g) * 1e-2
+    r17, r21 = ref(ids, lt)
+    torch.autograd.backward([r17, r21], [d17, d21])
+    m17, m21 = mine(ids.cuda(), lt.cuda())
+    torch.autograd.backward([m17, m21], [d17.cuda(), d21.cuda()])
+
+    def rel(a, b):
+        a, b = a.detach().cpu().double(), b.detach().double()
+        return float((a - b).norm() / (b.norm() + 1e-300))
+
+    assert rel(m17, r17) < 1e-5 and rel(m21, r21) < 1e-5
+    grads = dict((k, p.grad) for k, p in mine.named_parameters())
+    for k, p in ref.named_parameters():
+        assert rel(grads[k], p.grad) < 2e-5, (k, rel(grads[k], p.grad))
