@@ -29,8 +29,6 @@
 //   gradient falls out of the same dY tile.
 #include "pd_internal.h"
 
-#include <type_traits>
-
 typedef float float4_t __attribute__((ext_vector_type(4)));
 typedef float float16_t __attribute__((ext_vector_type(16)));
 
@@ -314,6 +312,47 @@ __global__ __launch_bounds__(CONV_THREADS, 2) void conv3x3_fwd_kernel(const Conv
     }
 }
 
+// Epilogue of the few-channel forward kernels: the 2 x 2 accumulator tiles of a wave (32 pixels x 32
+// channels each) to y, 64 dword stores per lane (lanes 0-31 = 32 consecutive channels of one pixel: 128-byte
+// runs).  Accumulator element e of tile i is pixel q = (wave*2 + i)*32 + 8*(e/4) + 4h + e%4 of the block's TH x
+// TW pixels, row q / TW, column q % TW (the column part 4h + e%4 < 8 never carries into the row).  One
+// per-lane byte offset; the pixel's row goes into a scalar offset, its column too -- or, when the channel
+// count is a compile-time constant (KT != 0), into the instruction's offset field.  Pixels and channels
+// outside the tensor get an offset beyond the buffer, which drops the store; FULL = the tile lies inside
+// the image, no per-pixel test.
+template <int TW, int KT, bool FULL>
+__device__ __forceinline__ void smallc_store_tile(const float16_t (&acc)[2][2], const __amdgpu_buffer_rsrc_t yr,
+                                                  const float (&bv)[2], int y0, int x0, int k0, int H, int W,
+                                                  int K_rt, bool relu, int wave, int idx, int h) {
+    static_assert(TW == 8 || TW == 16 || TW == 32, "tile widths the pixel mapping assumes");
+    const int K = KT ? KT : K_rt;
+    const int rows_left = H - y0 - wave * (64 / TW);                   // wave-uniform
+    const int cols_left = W - x0 - 4 * h;
+#pragma unroll
+    for (int j = 0; j < 2; ++j) {
+        const int k = k0 + j * 32 + idx;
+        const uint32_t lane_off = k < K ? (uint32_t)((y0 * W + x0 + 4 * h) * K + k) * 4 : 0x80000000u;
+#pragma unroll
+        for (int i = 0; i < 2; ++i)
+#pragma unroll
+            for (int e = 0; e < 16; ++e) {
+                const int qq = i * 32 + 8 * (e / 4) + (e % 4);
+                const int r_rel = qq / TW, c_rel = qq % TW;              // compile-time
+                float v = acc[i][j][e] + bv[j];
+                if (relu) v = v > 0.f ? v : 0.f;
+                const uint32_t voff = (FULL || (r_rel < rows_left && c_rel < cols_left)) ? lane_off : 0x80000000u;
+                if (KT) {
+                    const int soff = (wave * (64 / TW) + r_rel) * W * (KT * 4);
+                    __builtin_amdgcn_raw_buffer_store_b32(__builtin_bit_cast(uint32_t, v), yr, voff + c_rel * (KT * 4),
+                                                          soff, 0);
+                } else {
+                    const int soff = ((wave * (64 / TW) + r_rel) * W + c_rel) * (K * 4);
+                    __builtin_amdgcn_raw_buffer_store_b32(__builtin_bit_cast(uint32_t, v), yr, voff, soff, 0);
+                }
+            }
+    }
+}
+
 // Forward for very few input channels (9*C <= 32: the first VGG layer, C = 3).  The whole
 // reduction (9 taps x C) fits one 32-wide k range, so instead of padding C to 8 per tap the
 // (tap, channel) pairs are packed densely: 16 MFMA k-steps per tile instead of 36.  The A
@@ -440,41 +479,16 @@ __global__ __launch_bounds__(CONV_THREADS, 2) void conv3x3_fwd_smallc_kernel(con
         }
     }
 
-    // Epilogue: 64 dword stores per lane (lanes 0-31 = 32 consecutive channels of one pixel: 128-byte runs).
-    // One per-lane byte offset; the pixel's row and column go into a scalar offset.  Accumulator element e
-    // of tile i is pixel q = (wave*2 + i)*32 + 8*(e/4) + 4h + e%4 of the block, row q / TW, column q % TW (the
-    // column part 4h + e%4 < 8 never carries into the row).  Pixels and channels outside the tensor get an
-    // offset beyond the buffer, which drops the store; a block whose tile lies inside the image skips the
-    // per-pixel test.
     const uint32_t img_bytes = (uint32_t)a.H * a.W * a.K * 4;
     const __amdgpu_buffer_rsrc_t yr = __builtin_amdgcn_make_buffer_rsrc(
         (void*)(a.y + (size_t)n * a.H * a.W * a.K), 0, img_bytes, 0x00020000);
-    const bool full_tile = y0 + TH <= a.H && x0 + TW <= a.W;          // block-uniform
-    const int rows_left = a.H - y0 - wave * (64 / TW);                 // wave-uniform
-    const int cols_left = a.W - x0 - 4 * h;
-    auto store_all = [&](auto full) {
+    float bv[2];
 #pragma unroll
-        for (int j = 0; j < 2; ++j) {
-            const int k = k0 + j * 32 + idx;
-            const float bv = (a.bias && k < a.K) ? a.bias[k] : 0.f;
-            const uint32_t lane_off = k < a.K ? (uint32_t)((y0 * a.W + x0 + 4 * h) * a.K + k) * 4 : 0x80000000u;
-#pragma unroll
-            for (int i = 0; i < 2; ++i)
-#pragma unroll
-                for (int e = 0; e < 16; ++e) {
-                    const int qq = i * 32 + 8 * (e / 4) + (e % 4);
-                    const int r_rel = qq / TW, c_rel = qq % TW;              // compile-time
-                    const int soff = ((wave * (64 / TW) + r_rel) * a.W + c_rel) * (a.K * 4);   // wave-uniform
-                    float v = acc[i][j][e] + bv;
-                    if (a.relu) v = v > 0.f ? v : 0.f;
-                    const uint32_t voff =
-                        (decltype(full)::value || (r_rel < rows_left && c_rel < cols_left)) ? lane_off : 0x80000000u;
-                    __builtin_amdgcn_raw_buffer_store_b32(__builtin_bit_cast(uint32_t, v), yr, voff, soff, 0);
-                }
-        }
-    };
-    if (full_tile) store_all(std::true_type{});
-    else store_all(std::false_type{});
+    for (int j = 0; j < 2; ++j) bv[j] = (a.bias && k0 + j * 32 + idx < a.K) ? a.bias[k0 + j * 32 + idx] : 0.f;
+    if (y0 + TH <= a.H && x0 + TW <= a.W)           // block-uniform
+        smallc_store_tile<TW, 0, true>(acc, yr, bv, y0, x0, k0, a.H, a.W, a.K, a.relu, wave, idx, h);
+    else
+        smallc_store_tile<TW, 0, false>(acc, yr, bv, y0, x0, k0, a.H, a.W, a.K, a.relu, wave, idx, h);
 }
 
 // The same kernel for a layer with a single block of output channels (K <= 64), as a persistent loop: a
@@ -602,8 +616,7 @@ __global__ __launch_bounds__(CONV_THREADS, 4) void conv3x3_fwd_smallc_persist_ke
         const int q = (wave * 2 + i) * 32 + idx;
         pbase[i] = ((q / TW) * HW_ + (q % TW)) * 4;
     }
-    const float bv0 = a.bias ? a.bias[idx] : 0.f;
-    const float bv1 = a.bias ? a.bias[32 + idx] : 0.f;
+    const float bv[2] = {a.bias ? a.bias[idx] : 0.f, a.bias ? a.bias[32 + idx] : 0.f};
     const uint32_t y_img_bytes = (uint32_t)a.H * a.W * KT * 4;
     const float16_t zero16 = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
     __syncthreads();
@@ -635,38 +648,13 @@ __global__ __launch_bounds__(CONV_THREADS, 4) void conv3x3_fwd_smallc_persist_ke
         // The next tile's halo goes to LDS before this tile's stores are issued: the memory counter retires
         // in order, so waiting for those loads behind 64 fresh stores would wait for the stores to drain.
         if (ti + 1 < n_my) store_halo((ti + 1) & 1);
-        // stores: see conv3x3_fwd_smallc_kernel
         const Pos p = decode(tile);
         const __amdgpu_buffer_rsrc_t yr = __builtin_amdgcn_make_buffer_rsrc(
             (void*)(a.y + (size_t)p.n * a.H * a.W * KT), 0, y_img_bytes, 0x00020000);
-        const bool full_tile = p.y0 + TH <= a.H && p.x0 + TW <= a.W;
-        const int rows_left = a.H - p.y0 - wave * (64 / TW);
-        const int cols_left = a.W - p.x0 - 4 * h;
-        auto store_all = [&](auto full) {
-#pragma unroll
-            for (int j = 0; j < 2; ++j) {
-                const int k = j * 32 + idx;
-                const float bv = j ? bv1 : bv0;
-                const uint32_t lane_off = (uint32_t)((p.y0 * a.W + p.x0 + 4 * h) * KT + k) * 4;
-#pragma unroll
-                for (int i = 0; i < 2; ++i)
-#pragma unroll
-                    for (int e = 0; e < 16; ++e) {
-                        const int qq = i * 32 + 8 * (e / 4) + (e % 4);
-                        const int r_rel = qq / TW, c_rel = qq % TW;
-                        const int soff = (wave * (64 / TW) + r_rel) * a.W * (KT * 4);     // row: scalar
-                        float v = acc[i][j][e] + bv;
-                        if (a.relu) v = v > 0.f ? v : 0.f;
-                        const uint32_t voff = (decltype(full)::value || (r_rel < rows_left && c_rel < cols_left))
-                                                  ? lane_off : 0x80000000u;
-                        // column: a constant, folded into the instruction's offset field
-                        __builtin_amdgcn_raw_buffer_store_b32(__builtin_bit_cast(uint32_t, v), yr,
-                                                              voff + c_rel * (KT * 4), soff, 0);
-                    }
-            }
-        };
-        if (full_tile) store_all(std::true_type{});
-        else store_all(std::false_type{});
+        if (p.y0 + TH <= a.H && p.x0 + TW <= a.W)
+            smallc_store_tile<TW, KT, true>(acc, yr, bv, p.y0, p.x0, 0, a.H, a.W, KT, a.relu, wave, idx, h);
+        else
+            smallc_store_tile<TW, KT, false>(acc, yr, bv, p.y0, p.x0, 0, a.H, a.W, KT, a.relu, wave, idx, h);
         __syncthreads();
     }
 }
