@@ -19,18 +19,16 @@ import torch
 
 
 def label_smoothing(output, target, padding_idx, smoothing):
-    """smoothing.py:23-34, line by line."""
-    confidence = 1.0 - smoothing
-    x = output.view(output.size(0) * output.size(1), -1)                                  # :24
-    logprobs = torch.nn.functional.log_softmax(x, dim=-1, dtype=torch.float32)            # :25
-    non_pad_mask = (target != padding_idx)                                                # :27
-    nll_loss = -logprobs.gather(dim=-1, index=target.unsqueeze(1))                        # :28
-    nll_loss = nll_loss.squeeze(1)[non_pad_mask]                                          # :29
-    smooth_loss = -logprobs.mean(dim=-1)[non_pad_mask]                                    # :30
-    loss = confidence * nll_loss + smoothing * smooth_loss                                # :31
-    loss = loss.sum()                                                                     # :32
-    loss = loss / output.size(1)                                                          # :33
-    return loss
+    """The criterion of smoothing.py:23-34: fp32 log-softmax over the last dimension of the [T, B, V] logits
+    (:24-25); per row the negative log-probability of the target (:28) and the negative mean log-probability
+    (:30), mixed with weights 1 - smoothing and smoothing (:31); rows whose target is the padding index are
+    dropped (:27, :29-30); the sum over the other rows is divided by the batch size B (:32-33)."""
+    rows = output.reshape(-1, output.shape[-1])
+    logp = torch.log_softmax(rows, dim=-1, dtype=torch.float32)
+    keep = target.ne(padding_idx)
+    picked = logp[torch.arange(rows.shape[0]), target]
+    per_row = (1.0 - smoothing) * (-picked) + smoothing * (-logp.mean(dim=-1))
+    return per_row[keep].sum() / output.shape[1]
 
 
 def revert_varlen_offsets(lengths, seq_length, batch_size, feature_size):
@@ -103,13 +101,14 @@ class EmuBidirLSTM(torch.nn.Module):
             setattr(self.layer2, name, getattr(self.bidir, name + "_reverse"))
 
     def forward(self, input, lengths):
-        lengths = lengths.cpu().long()                                                              # :59
-        mask = set_mask(lengths)
-        # :51 builds the mask with lengths[0] rows; it multiplies a [T, B, H] tensor, so T == lengths[0]
-        assert mask.shape[0] == input.shape[0], "the longest sequence must fill the tensor"
-        mask = mask.unsqueeze(-1).type_as(input)
-        inputl1 = _RevertVarlen.apply(input, lengths)                                               # :52
-        out1 = self.layer2(inputl1)                                                                 # :53
-        outputs = _RevertVarlen.apply(out1[0], lengths)                                             # :54
-        out0 = self.layer1(input)[0] * mask                                                         # :55
-        return torch.cat([out0, outputs], dim=2)                                                    # :56
+        """encoder.py:50-57 and :59: the backward direction runs on the sequences reversed over their own
+        lengths and its output is reversed back; the forward direction's output is zeroed behind every
+        sequence's end; both halves side by side."""
+        lengths = lengths.cpu().long()
+        keep = set_mask(lengths)
+        # the reference builds the mask with lengths[0] rows and multiplies a [T, B, H] tensor with it (:51,
+        # :55), so the longest sequence must fill the tensor
+        assert keep.shape[0] == input.shape[0], "the longest sequence must fill the tensor"
+        backward_dir = self.layer2(_RevertVarlen.apply(input, lengths))[0]
+        forward_dir = self.layer1(input)[0] * keep.unsqueeze(-1).type_as(input)
+        return torch.cat([forward_dir, _RevertVarlen.apply(backward_dir, lengths)], dim=2)
