@@ -143,8 +143,9 @@ def gpu_run(steps, warmup):
 def pmc_probe():
     """Workload for `rocprofv3 --pmc FETCH_SIZE` / `--pmc WRITE_SIZE` runs: a plain copy of
     known size (calibrates the counters: pd_copy_kernel moves 1 GiB in and 1 GiB out per
-    launch) followed by two steady-state steps of the benchmark stage, so the per-dispatch
-    counter values of the convolution kernels cover exactly the launch mix of the timed region."""
+    launch) followed by steady-state steps of the benchmark stage, so the per-dispatch counter values of
+    the convolution kernels cover exactly the launch mix of the timed region, and by the optimizer kernel
+    on the VGG16-sized parameter set.  The same workload serves the MFMA-utilisation counters."""
     import ctypes
     import torch
     from pipedream_amd import _cabi
@@ -156,6 +157,8 @@ def pmc_probe():
     torch.cuda.synchronize()
     del src, dst
     gpu_run(steps=2, warmup=1)
+    # and the fused stash + SGD kernel on the VGG16-sized parameter set of `optimizer_hbm`
+    optimizer_bandwidth()
     print("pmc probe done")
 
 
