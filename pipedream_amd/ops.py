@@ -425,8 +425,13 @@ def set_conv_algorithm(name):
     _CONV_ALGO = name
 
 
-def _use_winograd(c, k):
+def _use_winograd(c, k, h, w):
+    """Whether a convolution with c input and k output channels on h x w images takes the Winograd kernel:
+    channel counts it supports, an image it can address with 32-bit offsets (the limits its entry point
+    checks), and, unless forced, enough channels for it to pay."""
     if _CONV_ALGO == "direct" or not _cabi.lib().pd_conv3x3_winograd_supported(c, k):
+        return False
+    if h * w * max(c, k) >= 1 << 29 or c * 16 * 64 * 4 >= 1 << 31:
         return False
     return _CONV_ALGO == "winograd" or (c >= 16 and k >= 32)
 
@@ -458,7 +463,7 @@ def conv3x3_forward(x, w, bias=None, relu=False):
         _check(bias, "bias")
         if bias.numel() != k or not bias.is_contiguous():
             raise ValueError("conv3x3: bias must be a contiguous vector of K=%d" % k)
-    if _use_winograd(c, k):
+    if _use_winograd(c, k, h, wd):
         return _winograd_conv(x, w, bias, None, None, n, h, wd, c, k, relu, False)
     y = torch.empty((n, k, h, wd), dtype=torch.float32, device=x.device, memory_format=torch.channels_last)
     with _timed("conv3x3_fwd_kernel" if c > 8 else "conv3x3_fwd_kernel_smallc", 18.0 * c * k * n * h * wd):
@@ -476,7 +481,7 @@ def conv3x3_forward_pool(x, w, bias=None, relu=False):
     k, cw = _filter_dims(w)
     if cw != c:
         raise ValueError("conv3x3: input has %d channels, filter expects %d" % (c, cw))
-    if not (_use_winograd(c, k) and h >= 2 and wd >= 2):
+    if not (_use_winograd(c, k, h, wd) and h >= 2 and wd >= 2):
         return maxpool2x2_idx(conv3x3_forward(x, w, bias, relu))
     if bias is not None:
         _check(bias, "bias")
@@ -515,7 +520,7 @@ def conv3x3_input_grad(dy, w, relu_out=None, x_rectified=None):
     kw, c = _filter_dims(w)
     if kw != k:
         raise ValueError("conv3x3_input_grad: dy has %d channels, filter has %d outputs" % (k, kw))
-    if _use_winograd(k, c):
+    if _use_winograd(k, c, h, wd):
         return _winograd_conv(dy, w, None, relu_out, x_rectified, n, h, wd, k, c, False, True)
     lib = _cabi.lib()
     # rotated filter: logical [C, K, 3, 3] in channels_last order = memory [C][3][3][K]
@@ -541,7 +546,8 @@ def conv3x3_weight_grad(x, dy, with_bias=True, relu_out=None):
         raise ValueError("conv3x3_weight_grad: x %s and dy %s disagree" % (tuple(x.shape), tuple(dy.shape)))
     lib = _cabi.lib()
     nbytes = ctypes.c_uint64()
-    if relu_out is None and _CONV_ALGO != "direct" and lib.pd_conv3x3_winograd_wgrad_supported(c, k):
+    if (relu_out is None and _CONV_ALGO != "direct" and lib.pd_conv3x3_winograd_wgrad_supported(c, k)
+            and wd * max(c, k) < 1 << 28):
         lib.pd_conv3x3_winograd_wgrad_workspace_bytes(c, k, ctypes.byref(nbytes))
         ws = torch.empty(nbytes.value, dtype=torch.uint8, device=x.device)
         dw = torch.empty((k, c, 3, 3), dtype=torch.float32, device=x.device, memory_format=torch.channels_last)

@@ -56,3 +56,24 @@ def test_product_refuses_cpu_tensors():
     model = torch.nn.Linear(4, 4)
     with pytest.raises(RuntimeError, match="no CPU fallback"):
         sgd.SGDWithWeightStashing([model], list(model.parameters()), None, 1.0, 2, lr=0.1)
+
+
+def test_convolution_algorithm_choice_is_host_logic():
+    """Which kernel a 3x3 convolution takes is decided on the host from shapes alone: Winograd for channel
+    counts it supports and that pay, the direct kernels otherwise -- including images the Winograd kernels
+    cannot address with 32-bit offsets."""
+    from pipedream_amd import ops
+    assert ops._use_winograd(64, 64, 224, 224)
+    assert ops._use_winograd(128, 128, 112, 112)
+    assert not ops._use_winograd(3, 64, 224, 224)          # few channels: the dense-tap kernels
+    assert not ops._use_winograd(20, 70, 17, 33)           # K % 4 != 0
+    assert not ops._use_winograd(64, 64, 4096, 4096)       # H*W*C beyond the kernel's offset range
+    try:
+        ops.set_conv_algorithm("winograd")
+        assert ops._use_winograd(8, 4, 9, 9) and not ops._use_winograd(64, 64, 4096, 4096)
+        ops.set_conv_algorithm("direct")
+        assert not ops._use_winograd(64, 64, 224, 224)
+        with pytest.raises(ValueError):
+            ops.set_conv_algorithm("fft")
+    finally:
+        ops.set_conv_algorithm("auto")
