@@ -189,7 +189,7 @@ def optimizer_bandwidth():
             "achieved_GBps": 20.0 * n / sec / 1e9, "peak_GBps": 8000.0, "frac": 20.0 * n / sec / 1e9 / 8000.0}
 
 
-def cpu_baseline(timed_steps=2):
+def cpu_baseline(timed_steps=6):
     """The CPU oracle (torch.nn modules, state_dict-copy weight stashing, torch.optim.SGD)
     on the same workload: 1 warm-up + `timed_steps` steady-state steps at batch 64."""
     import torch
