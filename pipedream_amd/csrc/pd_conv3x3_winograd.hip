@@ -416,9 +416,38 @@ __global__ __launch_bounds__(WG_THREADS, 1) void winograd_fwd_kernel(const WinoA
                     if ((e & 3) == 3) __builtin_amdgcn_sched_barrier(0);
                 }
             };
+            // Output mask (the ReLU backward of the layer that produced this convolution's input): the thread
+            // that stores pixel rows prow + 2 it of column pcol, channels k4..k4+3 fetches their mask values
+            // while its wave has nothing else to do -- the waves with gh = 1 during the first phase, the others
+            // during the second -- eight loads in flight, and keeps one bit per element ("mask > 0").  Inside
+            // the store loop each load would be a full round trip to memory.
+            constexpr int NV = 256 * (WG_BN / 4) / WG_THREADS;
+            const int k4 = (tid & 15) * 4, pcol = (tid >> 4) & 15, prow = tid >> 8;
+            const uint32_t out_bytes = (uint32_t)a.H * a.W * a.K * 4;
+            const bool col_ok = w.x0 + pcol < a.W && k0 + k4 < a.K;
+            const uint32_t obase = (uint32_t)(((w.y0 + prow) * a.W + w.x0 + pcol) * a.K + k0 + k4) * 4;
+            const int row_stride = 2 * a.W * a.K * 4;
+            uint32_t mbits = 0;
+            auto fetch_mask = [&]() {
+                const __amdgpu_buffer_rsrc_t omr =
+                    __builtin_amdgcn_make_buffer_rsrc((void*)(a.out_mask + oimg), 0, out_bytes, 0x00020000);
+                float4_t mk[NV];
+#pragma unroll
+                for (int it = 0; it < NV; ++it) {
+                    const uint32_t voff = (col_ok && w.y0 + prow + 2 * it < a.H) ? obase : 0x80000000u;
+                    mk[it] = __builtin_bit_cast(
+                        float4_t, __builtin_amdgcn_raw_buffer_load_b128(omr, voff, it * row_stride, 2));
+                }
+#pragma unroll
+                for (int it = 0; it < NV; ++it)
+#pragma unroll
+                    for (int c = 0; c < 4; ++c) mbits |= (mk[it][c] > 0.f ? 1u : 0u) << (it * 4 + c);
+            };
+            if (!POOL && a.out_mask && gh == 1) fetch_mask();
             if (gh == 0) out_rows(false);
             __syncthreads();
             if (gh == 1) out_rows(true);
+            else if (!POOL && a.out_mask) fetch_mask();
             __syncthreads();
             if constexpr (POOL) {
                 // 2x2 max pooling of the tile (bias and ReLU first), written with one index byte per element
@@ -473,24 +502,17 @@ __global__ __launch_bounds__(WG_THREADS, 1) void winograd_fwd_kernel(const WinoA
                     __builtin_amdgcn_raw_buffer_store_b32(packed, pir, ok ? eoff : 0x80000000u, 0, 0);
                 }
             } else {
-                // bias, ReLU, output mask and the NHWC stores.  Thread -> pixel column (tid >> 4) & 15, channels
-                // k4..k4+3, pixel rows (tid >> 8) + 2 it: one base offset, a scalar stride per row pair.  Pixels
-                // outside the image get an offset beyond the buffer's size: such a store is dropped.
-                constexpr int NV = 256 * (WG_BN / 4) / WG_THREADS;
-                const int k4 = (tid & 15) * 4, pcol = (tid >> 4) & 15, prow = tid >> 8;
+                // bias, ReLU, output mask (bits fetched above) and the NHWC stores.  Thread -> pixel column
+                // (tid >> 4) & 15, channels k4..k4+3, pixel rows (tid >> 8) + 2 it: one base offset, a scalar
+                // stride per row pair.  Pixels outside the image get an offset beyond the buffer's size: such a
+                // store is dropped.
                 float4_t b4 = {0.f, 0.f, 0.f, 0.f};
                 if (a.bias) {
     #pragma unroll
                     for (int c = 0; c < 4; ++c) b4[c] = k0 + k4 + c < a.K ? a.bias[k0 + k4 + c] : 0.f;
                 }
-                const uint32_t out_bytes = (uint32_t)a.H * a.W * a.K * 4;
                 const __amdgpu_buffer_rsrc_t yr =
                     __builtin_amdgcn_make_buffer_rsrc((void*)(a.y + oimg), 0, out_bytes, 0x00020000);
-                const __amdgpu_buffer_rsrc_t omr = __builtin_amdgcn_make_buffer_rsrc(
-                    (void*)((a.out_mask ? a.out_mask : a.y) + oimg), 0, out_bytes, 0x00020000);
-                const bool col_ok = w.x0 + pcol < a.W && k0 + k4 < a.K;
-                const uint32_t obase = (uint32_t)(((w.y0 + prow) * a.W + w.x0 + pcol) * a.K + k0 + k4) * 4;
-                const int row_stride = 2 * a.W * a.K * 4;
                 const float* src = stg + (prow * WG_PIX + pcol) * WG_OP + k4;
     #pragma unroll
                 for (int it = 0; it < NV; ++it) {
@@ -501,10 +523,8 @@ __global__ __launch_bounds__(WG_THREADS, 1) void winograd_fwd_kernel(const WinoA
                         for (int c = 0; c < 4; ++c) v[c] = v[c] > 0.f ? v[c] : 0.f;
                     }
                     if (a.out_mask) {
-                        const float4_t mk = __builtin_bit_cast(
-                            float4_t, __builtin_amdgcn_raw_buffer_load_b128(omr, voff, it * row_stride, 2));
     #pragma unroll
-                        for (int c = 0; c < 4; ++c) v[c] = mk[c] > 0.f ? v[c] : 0.f;
+                        for (int c = 0; c < 4; ++c) v[c] = (mbits >> (it * 4 + c)) & 1u ? v[c] : 0.f;
                     }
                     typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
                     __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(u32x4, v), yr, voff, it * row_stride, 2);
