@@ -1288,16 +1288,17 @@ __global__ __launch_bounds__(256) void reduce_partials_kernel(const float* __res
     __shared__ float red[4][64];
     const int lane = threadIdx.x % 64, w = threadIdx.x / 64;
     const int i = blockIdx.x * 64 + lane;
-    float s0 = 0.f, s1 = 0.f;
+    // eight independent sums per lane: eight loads in flight instead of a chain of round trips (the order
+    // of the additions is fixed, so the result is reproducible)
+    float t[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
     if (i < n) {
         int b = w;
-        for (; b + 4 < n_part; b += 8) {
-            s0 += part[(size_t)b * n + i];
-            s1 += part[(size_t)(b + 4) * n + i];
-        }
-        if (b < n_part) s0 += part[(size_t)b * n + i];
+        for (; b + 28 < n_part; b += 32)
+#pragma unroll
+            for (int u = 0; u < 8; ++u) t[u] += part[(size_t)(b + 4 * u) * n + i];
+        for (; b < n_part; b += 4) t[0] += part[(size_t)b * n + i];
     }
-    red[w][lane] = s0 + s1;
+    red[w][lane] = ((t[0] + t[1]) + (t[2] + t[3])) + ((t[4] + t[5]) + (t[6] + t[7]));
     __syncthreads();
     if (w == 0 && i < n) out[i] = (red[0][lane] + red[1][lane]) + (red[2][lane] + red[3][lane]);
 }
