@@ -38,12 +38,25 @@ __global__ __launch_bounds__(LSTM_THREADS) void lstm_cell_fwd_kernel(float* __re
     float4_t gf = *(const float4_t*)(g + H + j);
     float4_t gg = *(const float4_t*)(g + 2 * H + j);
     float4_t go = *(const float4_t*)(g + 3 * H + j);
-    for (int s = 0; s < n_rec; ++s) {   // split-k partial sums of h_{t-1} W_hh^T, added in a fixed order
-        const float* r = rec + ((size_t)s * B + b) * 4 * H;
-        gi += *(const float4_t*)(r + j);
-        gf += *(const float4_t*)(r + H + j);
-        gg += *(const float4_t*)(r + 2 * H + j);
-        go += *(const float4_t*)(r + 3 * H + j);
+    // split-k partial sums of h_{t-1} W_hh^T, added in a fixed order, four partials (16 loads) in flight at
+    // a time: one at a time the loop is a chain of round trips to memory
+    for (int s0 = 0; s0 < n_rec; s0 += 4) {
+        float4_t p[4][4];
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+            const bool live = s0 + u < n_rec;
+            const float* r = rec + ((size_t)(live ? s0 + u : s0) * B + b) * 4 * H;
+#pragma unroll
+            for (int q = 0; q < 4; ++q) p[u][q] = *(const float4_t*)(r + q * H + j);
+            if (!live) {
+#pragma unroll
+                for (int q = 0; q < 4; ++q) p[u][q] = float4_t{0.f, 0.f, 0.f, 0.f};
+            }
+        }
+        gi += (p[0][0] + p[1][0]) + (p[2][0] + p[3][0]);
+        gf += (p[0][1] + p[1][1]) + (p[2][1] + p[3][1]);
+        gg += (p[0][2] + p[1][2]) + (p[2][2] + p[3][2]);
+        go += (p[0][3] + p[1][3]) + (p[2][3] + p[3][3]);
     }
     if (b_ih) {
         gi += *(const float4_t*)(b_ih + j) + *(const float4_t*)(b_hh + j);
@@ -95,8 +108,19 @@ __global__ __launch_bounds__(LSTM_THREADS) void lstm_cell_bwd_kernel(const float
     if (c_prev) cp = *(const float4_t*)(c_prev + o);
     const float4_t ct = *(const float4_t*)(c + o);
     float4_t dh = *(const float4_t*)(dy + o);
-    if (dh_rec)
-        for (int s = 0; s < n_rec; ++s) dh += *(const float4_t*)(dh_rec + (size_t)s * B * H + o);
+    if (dh_rec) {
+        // the split-k partial sums of dgates W_hh, eight loads in flight at a time, added in a fixed order
+        for (int s0 = 0; s0 < n_rec; s0 += 8) {
+            float4_t p[8];
+#pragma unroll
+            for (int u = 0; u < 8; ++u) {
+                const bool live = s0 + u < n_rec;
+                p[u] = *(const float4_t*)(dh_rec + (size_t)(live ? s0 + u : s0) * B * H + o);
+                if (!live) p[u] = float4_t{0.f, 0.f, 0.f, 0.f};
+            }
+            dh += ((p[0] + p[1]) + (p[2] + p[3])) + ((p[4] + p[5]) + (p[6] + p[7]));
+        }
+    }
     float4_t dc = {0.f, 0.f, 0.f, 0.f};
     if (!first_step) dc = *(const float4_t*)(dc_io + o);
     float4_t di, df, dg, dO, dcp;
