@@ -475,8 +475,20 @@ __global__ __launch_bounds__(256) void splitk_reduce_kernel(const float* __restr
     if (id >= (long long)M * n4) return;
     const int row = (int)(id / n4), col = (int)(id % n4) * 4;
     const size_t per = (size_t)M * N;
-    float4_t v = *(const float4_t*)(partials + (size_t)row * N + col);
-    for (int s = 1; s < splits; ++s) v += *(const float4_t*)(partials + s * per + (size_t)row * N + col);
+    // eight partials in flight at a time (one at a time the loop is a chain of round trips to memory),
+    // added in a fixed order
+    const float* src = partials + (size_t)row * N + col;
+    float4_t v = {0.f, 0.f, 0.f, 0.f};
+    for (int s0 = 0; s0 < splits; s0 += 8) {
+        float4_t p[8];
+#pragma unroll
+        for (int u = 0; u < 8; ++u) {
+            const bool live = s0 + u < splits;
+            p[u] = *(const float4_t*)(src + (size_t)(live ? s0 + u : s0) * per);
+            if (!live) p[u] = float4_t{0.f, 0.f, 0.f, 0.f};
+        }
+        v += ((p[0] + p[1]) + (p[2] + p[3])) + ((p[4] + p[5]) + (p[6] + p[7]));
+    }
     if (bias) v += *(const float4_t*)(bias + col);
     float* p = C + (size_t)row * ldc + col;
     if (beta != 0.f) v += beta * *(const float4_t*)p;
