@@ -328,19 +328,25 @@ __device__ __forceinline__ void smallc_store_tile(const float16_t (&acc)[2][2], 
     const int K = KT ? KT : K_rt;
     const int rows_left = H - y0 - wave * (64 / TW);                   // wave-uniform
     const int cols_left = W - x0 - 4 * h;
+    uint32_t lane_off[2];
 #pragma unroll
     for (int j = 0; j < 2; ++j) {
         const int k = k0 + j * 32 + idx;
-        const uint32_t lane_off = k < K ? (uint32_t)((y0 * W + x0 + 4 * h) * K + k) * 4 : 0x80000000u;
+        lane_off[j] = k < K ? (uint32_t)((y0 * W + x0 + 4 * h) * K + k) * 4 : 0x80000000u;
+    }
+    // the two 128-byte halves of a pixel's 64 channels are stored back to back
 #pragma unroll
-        for (int i = 0; i < 2; ++i)
+    for (int i = 0; i < 2; ++i)
 #pragma unroll
-            for (int e = 0; e < 16; ++e) {
-                const int qq = i * 32 + 8 * (e / 4) + (e % 4);
-                const int r_rel = qq / TW, c_rel = qq % TW;              // compile-time
+        for (int e = 0; e < 16; ++e) {
+            const int qq = i * 32 + 8 * (e / 4) + (e % 4);
+            const int r_rel = qq / TW, c_rel = qq % TW;              // compile-time
+            const bool inside = FULL || (r_rel < rows_left && c_rel < cols_left);
+#pragma unroll
+            for (int j = 0; j < 2; ++j) {
                 float v = acc[i][j][e] + bv[j];
                 if (relu) v = v > 0.f ? v : 0.f;
-                const uint32_t voff = (FULL || (r_rel < rows_left && c_rel < cols_left)) ? lane_off : 0x80000000u;
+                const uint32_t voff = inside ? lane_off[j] : 0x80000000u;
                 if (KT) {
                     const int soff = (wave * (64 / TW) + r_rel) * W * (KT * 4);
                     __builtin_amdgcn_raw_buffer_store_b32(__builtin_bit_cast(uint32_t, v), yr, voff + c_rel * (KT * 4),
@@ -350,7 +356,7 @@ __device__ __forceinline__ void smallc_store_tile(const float16_t (&acc)[2][2], 
                     __builtin_amdgcn_raw_buffer_store_b32(__builtin_bit_cast(uint32_t, v), yr, voff, soff, 0);
                 }
             }
-    }
+        }
 }
 
 // Forward for very few input channels (9*C <= 32: the first VGG layer, C = 3).  The whole
