@@ -313,47 +313,49 @@ __global__ __launch_bounds__(CONV_THREADS, 2) void conv3x3_fwd_kernel(const Conv
 }
 
 // Epilogue of the few-channel forward kernels: the 2 x 2 accumulator tiles of a wave (32 pixels x 32
-// channels each) to y, 64 dword stores per lane (lanes 0-31 = 32 consecutive channels of one pixel: 128-byte
-// runs).  Accumulator element e of tile i is pixel q = (wave*2 + i)*32 + 8*(e/4) + 4h + e%4 of the block's TH x
-// TW pixels, row q / TW, column q % TW (the column part 4h + e%4 < 8 never carries into the row).  One
-// per-lane byte offset; the pixel's row goes into a scalar offset, its column too -- or, when the channel
-// count is a compile-time constant (KT != 0), into the instruction's offset field.  Pixels and channels
-// outside the tensor get an offset beyond the buffer, which drops the store; FULL = the tile lies inside
-// the image, no per-pixel test.
+// channels each) to y.  Accumulator element e of tile i is pixel q = (wave*2 + i)*32 + 8*(e/4) + 4h + e%4 of
+// the block's TH x TW pixels (h = lane / 32), row q / TW, column q % TW (the column part 4h + e%4 < 8 never
+// carries into the row), channel j*32 + lane % 32.  The upper half of the j = 0 register is exchanged with
+// the lower half of the j = 1 register (one v_permlane32_swap), after which a register holds all 64
+// channels of one pixel: every store instruction writes one 256-byte run, and the pixel (h = 0 or 1) is the
+// same for the whole wave, so its row and column go into a scalar offset -- or, when the channel count is
+// a compile-time constant (KT != 0), the column into the instruction's offset field.  Channels outside
+// the tensor get an offset beyond the buffer, which drops the store; pixels outside the image are skipped
+// (wave-uniform); FULL = the tile lies inside the image, no per-pixel test.
 template <int TW, int KT, bool FULL>
 __device__ __forceinline__ void smallc_store_tile(const float16_t (&acc)[2][2], const __amdgpu_buffer_rsrc_t yr,
-                                                  const float (&bv)[2], int y0, int x0, int k0, int H, int W,
-                                                  int K_rt, bool relu, int wave, int idx, int h) {
+                                                  float bias_lane, int y0, int x0, int k0, int H, int W,
+                                                  int K_rt, bool relu, int wave, int lane) {
     static_assert(TW == 8 || TW == 16 || TW == 32, "tile widths the pixel mapping assumes");
     const int K = KT ? KT : K_rt;
     const int rows_left = H - y0 - wave * (64 / TW);                   // wave-uniform
-    const int cols_left = W - x0 - 4 * h;
-    uint32_t lane_off[2];
-#pragma unroll
-    for (int j = 0; j < 2; ++j) {
-        const int k = k0 + j * 32 + idx;
-        lane_off[j] = k < K ? (uint32_t)((y0 * W + x0 + 4 * h) * K + k) * 4 : 0x80000000u;
-    }
-    // the two 128-byte halves of a pixel's 64 channels are stored back to back
+    const int cols_left = W - x0;
+    const int k = k0 + lane;                                           // after the exchange: 64 channels a pixel
+    const uint32_t lane_off = k < K ? (uint32_t)((y0 * W + x0) * K + k) * 4 : 0x80000000u;
 #pragma unroll
     for (int i = 0; i < 2; ++i)
 #pragma unroll
         for (int e = 0; e < 16; ++e) {
+            // (copies first: a bit cast applied to a vector element expression reads the vector's first element)
+            const float lo = acc[i][0][e], hi = acc[i][1][e];
+            const auto sw = __builtin_amdgcn_permlane32_swap(__builtin_bit_cast(uint32_t, lo),
+                                                             __builtin_bit_cast(uint32_t, hi), false, false);
             const int qq = i * 32 + 8 * (e / 4) + (e % 4);
-            const int r_rel = qq / TW, c_rel = qq % TW;              // compile-time
-            const bool inside = FULL || (r_rel < rows_left && c_rel < cols_left);
+            const int r_rel = qq / TW;                               // compile-time
 #pragma unroll
-            for (int j = 0; j < 2; ++j) {
-                float v = acc[i][j][e] + bv[j];
+            for (int hh = 0; hh < 2; ++hh) {                         // the pixels of the two lane halves
+                const int c_rel = qq % TW + 4 * hh;                  // compile-time
+                if (!FULL && !(r_rel < rows_left && c_rel < cols_left)) continue;
+                const uint32_t bits = sw[hh];                        // (a copy first, as above)
+                float v = __builtin_bit_cast(float, bits) + bias_lane;
                 if (relu) v = v > 0.f ? v : 0.f;
-                const uint32_t voff = inside ? lane_off[j] : 0x80000000u;
                 if (KT) {
                     const int soff = (wave * (64 / TW) + r_rel) * W * (KT * 4);
-                    __builtin_amdgcn_raw_buffer_store_b32(__builtin_bit_cast(uint32_t, v), yr, voff + c_rel * (KT * 4),
-                                                          soff, 0);
+                    __builtin_amdgcn_raw_buffer_store_b32(__builtin_bit_cast(uint32_t, v), yr,
+                                                          lane_off + c_rel * (KT * 4), soff, 0);
                 } else {
                     const int soff = ((wave * (64 / TW) + r_rel) * W + c_rel) * (K * 4);
-                    __builtin_amdgcn_raw_buffer_store_b32(__builtin_bit_cast(uint32_t, v), yr, voff, soff, 0);
+                    __builtin_amdgcn_raw_buffer_store_b32(__builtin_bit_cast(uint32_t, v), yr, lane_off, soff, 0);
                 }
             }
         }
@@ -488,13 +490,11 @@ __global__ __launch_bounds__(CONV_THREADS, 2) void conv3x3_fwd_smallc_kernel(con
     const uint32_t img_bytes = (uint32_t)a.H * a.W * a.K * 4;
     const __amdgpu_buffer_rsrc_t yr = __builtin_amdgcn_make_buffer_rsrc(
         (void*)(a.y + (size_t)n * a.H * a.W * a.K), 0, img_bytes, 0x00020000);
-    float bv[2];
-#pragma unroll
-    for (int j = 0; j < 2; ++j) bv[j] = (a.bias && k0 + j * 32 + idx < a.K) ? a.bias[k0 + j * 32 + idx] : 0.f;
+    const float bv = (a.bias && k0 + lane < a.K) ? a.bias[k0 + lane] : 0.f;
     if (y0 + TH <= a.H && x0 + TW <= a.W)           // block-uniform
-        smallc_store_tile<TW, 0, true>(acc, yr, bv, y0, x0, k0, a.H, a.W, a.K, a.relu, wave, idx, h);
+        smallc_store_tile<TW, 0, true>(acc, yr, bv, y0, x0, k0, a.H, a.W, a.K, a.relu, wave, lane);
     else
-        smallc_store_tile<TW, 0, false>(acc, yr, bv, y0, x0, k0, a.H, a.W, a.K, a.relu, wave, idx, h);
+        smallc_store_tile<TW, 0, false>(acc, yr, bv, y0, x0, k0, a.H, a.W, a.K, a.relu, wave, lane);
 }
 
 // The same kernel for a layer with a single block of output channels (K <= 64), as a persistent loop: a
@@ -622,7 +622,7 @@ __global__ __launch_bounds__(CONV_THREADS, 4) void conv3x3_fwd_smallc_persist_ke
         const int q = (wave * 2 + i) * 32 + idx;
         pbase[i] = ((q / TW) * HW_ + (q % TW)) * 4;
     }
-    const float bv[2] = {a.bias ? a.bias[idx] : 0.f, a.bias ? a.bias[32 + idx] : 0.f};
+    const float bv = a.bias ? a.bias[lane] : 0.f;
     const uint32_t y_img_bytes = (uint32_t)a.H * a.W * KT * 4;
     const float16_t zero16 = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
     __syncthreads();
@@ -658,9 +658,9 @@ __global__ __launch_bounds__(CONV_THREADS, 4) void conv3x3_fwd_smallc_persist_ke
         const __amdgpu_buffer_rsrc_t yr = __builtin_amdgcn_make_buffer_rsrc(
             (void*)(a.y + (size_t)p.n * a.H * a.W * KT), 0, y_img_bytes, 0x00020000);
         if (p.y0 + TH <= a.H && p.x0 + TW <= a.W)
-            smallc_store_tile<TW, KT, true>(acc, yr, bv, p.y0, p.x0, 0, a.H, a.W, KT, a.relu, wave, idx, h);
+            smallc_store_tile<TW, KT, true>(acc, yr, bv, p.y0, p.x0, 0, a.H, a.W, KT, a.relu, wave, lane);
         else
-            smallc_store_tile<TW, KT, false>(acc, yr, bv, p.y0, p.x0, 0, a.H, a.W, KT, a.relu, wave, idx, h);
+            smallc_store_tile<TW, KT, false>(acc, yr, bv, p.y0, p.x0, 0, a.H, a.W, KT, a.relu, wave, lane);
         __syncthreads();
     }
 }
