@@ -77,3 +77,58 @@ def test_convolution_algorithm_choice_is_host_logic():
             ops.set_conv_algorithm("fft")
     finally:
         ops.set_conv_algorithm("auto")
+
+
+def test_argument_validation_of_the_sequence_and_pooling_entry_points():
+    """Bad arguments are rejected on the host, before any launch: these calls need no GPU."""
+    lib = _cabi.lib()
+    p = ctypes.c_void_p(4096)      # any non-null, 16-byte aligned address: never dereferenced
+    odd = ctypes.c_void_p(4100)
+    E = _cabi.PipedreamAmdError
+    # label smoothing: empty shapes, NULL pointers, ld < V, non-positive divisor
+    with pytest.raises(E, match="empty"):
+        lib.pd_label_smoothing_fwd_f32(p, p, p, p, p, 0, 10, 10, 0, 0.1, 1.0, None)
+    with pytest.raises(E, match="NULL"):
+        lib.pd_label_smoothing_fwd_f32(p, None, p, p, p, 4, 10, 10, 0, 0.1, 1.0, None)
+    with pytest.raises(E, match="ld < V"):
+        lib.pd_label_smoothing_fwd_f32(p, p, p, p, p, 4, 10, 8, 0, 0.1, 1.0, None)
+    with pytest.raises(E, match="divisor"):
+        lib.pd_label_smoothing_bwd_f32(p, p, p, p, p, 4, 10, 10, 10, 0, 0.1, 0.0, None)
+    with pytest.raises(E, match="leading dimension"):
+        lib.pd_label_smoothing_bwd_f32(p, p, p, p, p, 4, 10, 10, 9, 0, 0.1, 1.0, None)
+    # revert_varlen / length mask: nothing to do is fine; in-place reversal, odd sizes and pitches are not
+    lib.pd_revert_varlen(None, None, None, 0, 5, 64, 64, 64, None)
+    with pytest.raises(E, match="in place"):
+        lib.pd_revert_varlen(p, p, p, 3, 2, 64, 64, 64, None)
+    with pytest.raises(E, match="pitch"):
+        lib.pd_revert_varlen(p, ctypes.c_void_p(8192), p, 3, 2, 64, 32, 64, None)
+    with pytest.raises(E, match="2-byte"):
+        lib.pd_length_mask_apply(p, p, p, 3, 2, 7, 7, 7, None)
+    with pytest.raises(E, match="NULL"):
+        lib.pd_length_mask_apply(p, p, None, 3, 2, 64, 64, 64, None)
+    with pytest.raises(E, match="65535"):
+        lib.pd_revert_varlen(p, ctypes.c_void_p(8192), p, 70000, 2, 64, 64, 64, None)
+    # the host-side mask builder works on host memory
+    lengths = (ctypes.c_int64 * 3)(3, 2, 1)
+    mask = (ctypes.c_uint8 * 9)()
+    lib.pd_set_mask_u8(ctypes.cast(lengths, ctypes.c_void_p), 3, 3, ctypes.cast(mask, ctypes.c_void_p))
+    assert list(mask) == [1, 1, 1, 1, 1, 0, 1, 0, 0]
+    with pytest.raises(E, match="NULL"):
+        lib.pd_set_mask_u8(None, 3, 3, ctypes.cast(mask, ctypes.c_void_p))
+    # pooling with index bytes: channel multiple of 4, alignment, NULL
+    with pytest.raises(E, match="multiple of 4"):
+        lib.pd_maxpool2x2_fwd_idx_nhwc_f32(p, p, p, 1, 4, 4, 6, 0, None)
+    with pytest.raises(E, match="aligned"):
+        lib.pd_maxpool2x2_fwd_idx_nhwc_f32(odd, p, p, 1, 4, 4, 8, 0, None)
+    with pytest.raises(E, match="NULL"):
+        lib.pd_maxpool2x2_bwd_idx_nhwc_f32(p, p, None, 1, 4, 4, 8, 0, None)
+    lib.pd_maxpool2x2_fwd_idx_nhwc_f32(None, None, None, 1, 1, 3, 8, 0, None)      # no window: nothing to do
+    # convolution with the pooling epilogue: shapes and pointers
+    with pytest.raises(E, match="2x2 window"):
+        lib.pd_conv3x3_winograd_fwd_pool_nhwc_f32(p, p, None, p, p, 1, 1, 8, 16, 32, 1, None)
+    with pytest.raises(E, match="NULL"):
+        lib.pd_conv3x3_winograd_fwd_pool_nhwc_f32(p, p, None, None, p, 1, 8, 8, 16, 32, 1, None)
+    with pytest.raises(E, match="C % 8"):
+        lib.pd_conv3x3_winograd_fwd_pool_nhwc_f32(p, p, None, p, p, 1, 8, 8, 12, 32, 1, None)
+    with pytest.raises(E, match="too large"):
+        lib.pd_conv3x3_winograd_fwd_nhwc_f32(p, p, None, None, None, p, 1, 4096, 4096, 64, 64, 0, None)
