@@ -177,6 +177,24 @@ def test_maxpool_with_index_bytes_bit_exact(shape, relu):
         assert torch.equal((b & 4) != 0, picked > 0) and int((b >> 3).max()) == 0
 
 
+def test_maxpool_with_index_bytes_propagates_nan_like_torch():
+    """A NaN in a window wins (torch's max_pool2d rule) and receives the window's gradient."""
+    g = torch.Generator().manual_seed(4)
+    x = torch.randn(2, 8, 6, 6, generator=g)
+    x[0, 1, 2, 3] = float("nan")
+    x[1, 5, 5, 5] = float("nan")
+    x[1, 5, 4, 4] = float("nan")          # two NaNs in one window: the first in scan order is picked
+    xr = x.clone().requires_grad_(True)
+    y_ref = F.max_pool2d(xr, 2, 2)
+    dy = torch.randn(y_ref.shape, generator=g)
+    y_ref.backward(dy)
+    y, idx = ops.maxpool2x2_idx(x.cuda().contiguous(memory_format=torch.channels_last))
+    assert torch.equal(torch.isnan(y.cpu()), torch.isnan(y_ref.detach()))
+    assert torch.equal(torch.nan_to_num(y.cpu(), nan=7.0), torch.nan_to_num(y_ref.detach(), nan=7.0))
+    dx = ops.maxpool2x2_idx_backward(dy.cuda(), idx, 6, 6)
+    assert torch.equal(dx.cpu(), xr.grad)
+
+
 @pytest.mark.parametrize("B,C", [(64, 10), (64, 1000), (7, 32320), (1, 3)])
 def test_cross_entropy_vs_torch(B, C):
     g = torch.Generator().manual_seed(2)
