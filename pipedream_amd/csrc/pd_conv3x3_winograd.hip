@@ -858,7 +858,7 @@ __global__ __launch_bounds__(WW_THREADS, 1) void winograd_wgrad_kernel(const Win
                 }
             load_dy(dp, d_left > 0);           // strip q+1
             next_d();
-            if (gh == 0) {
+            if (gh == 0 && wn == 0) {          // the waves that write the bias gradient at the end
 #pragma unroll
                 for (int j = 0; j < 4; ++j) db_acc += rr[1][0][j] + rr[1][1][j];
             }
