@@ -672,7 +672,7 @@ struct WinoWgradArgs {
     int c_blocks, n_pairs, ranks;
 };
 
-struct StripPos { int n, y0, x0; };
+struct StripPos { int n, y0, x0, row; };      // row = n * H + y0, the strip's first output row counted over all images
 
 // Strips are numbered down the image first (row pair fastest), then across, then over images: a block's
 // consecutive strips share two of their four input rows, which the second one finds in cache.
@@ -684,14 +684,17 @@ __device__ __forceinline__ StripPos strip_decode(const WinoWgradArgs& a, int s) 
     const int tx = rem / a.sy;
     p.x0 = tx * (2 * WW_TILES);
     p.y0 = 2 * (rem - tx * a.sy);
+    p.row = p.n * a.H + p.y0;
     return p;
 }
 __device__ __forceinline__ void strip_next(const WinoWgradArgs& a, StripPos& p) {
     p.y0 += 2;
+    p.row += 2;
     if (p.y0 >= a.H) {
+        p.row -= p.y0;
         p.y0 = 0;
         p.x0 += 2 * WW_TILES;
-        if (p.x0 >= a.W) { p.x0 = 0; ++p.n; }
+        if (p.x0 >= a.W) { p.x0 = 0; ++p.n; p.row += a.H; }
     }
 }
 
@@ -736,14 +739,16 @@ __global__ __launch_bounds__(WW_THREADS, 1) void winograd_wgrad_kernel(const Win
         raw_dst[j] = ((prow[j] & 3) * WW_PATCH_W + (live[j] ? ppx : 0)) * 64 + pcg * 4;
     }
     float4_t rawr[3];
+    const int row_floats_x = a.W * a.C;
     auto load_raw = [&](const StripPos& p, bool valid) {
         const uint32_t strip_off = (uint32_t)(p.x0 * a.C) * 4;
 #pragma unroll
         for (int j = 0; j < 3; ++j) {
             const int gy = p.y0 - 1 + prow[j];
             const bool row_ok = valid && gy >= 0 && gy < a.H && (j < 2 || wave < 4);
-            const float* base = a.x + ((size_t)(row_ok ? p.n : 0) * a.H + (row_ok ? gy : 0)) * a.W * a.C + cb * 64;
-            const uint32_t bytes = row_ok ? (uint32_t)(a.W * a.C - cb * 64) * 4 : 0u;
+            // a row outside the image gets an empty descriptor, whose base address is never used
+            const float* base = a.x + (int64_t)(p.row - 1 + prow[j]) * row_floats_x + cb * 64;
+            const uint32_t bytes = row_ok ? (uint32_t)(row_floats_x - cb * 64) * 4 : 0u;
             const __amdgpu_buffer_rsrc_t r = __builtin_amdgcn_make_buffer_rsrc((void*)base, 0, bytes, 0x00020000);
             rawr[j] = __builtin_bit_cast(float4_t, __builtin_amdgcn_raw_buffer_load_b128(r, xoff[j] + strip_off, 0, 0));
         }
@@ -791,8 +796,7 @@ __global__ __launch_bounds__(WW_THREADS, 1) void winograd_wgrad_kernel(const Win
 #pragma unroll
         for (int r = 0; r < 2; ++r) {
             const bool row_ok = valid && p.y0 + r < a.H;
-            const float* base =
-                a.dy + (row_ok ? (((size_t)p.n * a.H + p.y0 + r) * a.W + p.x0) * a.K : (size_t)0);
+            const float* base = a.dy + (int64_t)((p.row + r) * a.W + p.x0) * a.K;
             const uint32_t bytes = row_ok ? (uint32_t)((a.W - p.x0) * a.K) * 4 : 0u;
             const __amdgpu_buffer_rsrc_t rs = __builtin_amdgcn_make_buffer_rsrc((void*)base, 0, bytes, 0x00020000);
 #pragma unroll
@@ -1047,6 +1051,8 @@ extern "C" int pd_conv3x3_winograd_wgrad_nhwc_f32(const float* x, const float* d
     PD_REQUIRE(N > 0 && H > 0 && W > 0 && C > 0 && K > 0, PD_ESHAPE, "%s: dimensions must be positive", who);
     PD_REQUIRE(wino_wgrad_shape_ok(C, K), PD_ESHAPE, "%s: unsupported channel counts C=%d K=%d", who, C, K);
     PD_REQUIRE((long)W * (C > K ? C : K) < (1L << 28), PD_ESHAPE, "%s: image row too large", who);
+    // the kernel counts pixels over all images in 32 bits, a few strips past the last one included
+    PD_REQUIRE(((long)N * H + 2L * H + 8) * W < (1L << 31), PD_ESHAPE, "%s: too many pixels", who);
     PD_REQUIRE(x && dy && dw && workspace, PD_EINVAL, "%s: NULL pointer", who);
     PD_REQUIRE(pd_aligned(x, 16) && pd_aligned(dy, 16) && pd_aligned(workspace, 16), PD_EINVAL,
                "%s: tensors must be 16-byte aligned", who);

@@ -547,7 +547,7 @@ def conv3x3_weight_grad(x, dy, with_bias=True, relu_out=None):
     lib = _cabi.lib()
     nbytes = ctypes.c_uint64()
     if (relu_out is None and _CONV_ALGO != "direct" and lib.pd_conv3x3_winograd_wgrad_supported(c, k)
-            and wd * max(c, k) < 1 << 28):
+            and wd * max(c, k) < 1 << 28 and (n * h + 2 * h + 8) * wd < 1 << 31):
         lib.pd_conv3x3_winograd_wgrad_workspace_bytes(c, k, ctypes.byref(nbytes))
         ws = torch.empty(nbytes.value, dtype=torch.uint8, device=x.device)
         dw = torch.empty((k, c, 3, 3), dtype=torch.float32, device=x.device, memory_format=torch.channels_last)
