@@ -739,17 +739,26 @@ __global__ __launch_bounds__(WW_THREADS, 1) void winograd_wgrad_kernel(const Win
         raw_dst[j] = ((prow[j] & 3) * WW_PATCH_W + (live[j] ? ppx : 0)) * 64 + pcg * 4;
     }
     float4_t rawr[3];
-    const int row_floats_x = a.W * a.C;
+    // row descriptors, kept cheap in scalar instructions: per patch row a loop-invariant 64-bit base (row -1 +
+    // prow of image 0) to which the strip's running row index times the row pitch is added; a row outside
+    // the image (one unsigned comparison) or of a strip past the end gets size 0, and then its base is unused
+    const uint32_t row_pitch_x = (uint32_t)(a.W * a.C) * 4;
+    const uint32_t row_bytes_x = (uint32_t)(a.W * a.C - cb * 64) * 4;
+    const char* xrow0[3];
+#pragma unroll
+    for (int j = 0; j < 3; ++j) xrow0[j] = (const char*)(a.x + cb * 64) + (int64_t)(prow[j] - 1) * row_pitch_x;
+    const bool third_row_live = wave < 4;      // the third round of pieces covers the patch's last row only
     auto load_raw = [&](const StripPos& p, bool valid) {
         const uint32_t strip_off = (uint32_t)(p.x0 * a.C) * 4;
+        const uint32_t live_bytes = valid ? row_bytes_x : 0u;
+        const uint64_t strip_row = (uint64_t)(uint32_t)p.row * row_pitch_x;
 #pragma unroll
         for (int j = 0; j < 3; ++j) {
-            const int gy = p.y0 - 1 + prow[j];
-            const bool row_ok = valid && gy >= 0 && gy < a.H && (j < 2 || wave < 4);
-            // a row outside the image gets an empty descriptor, whose base address is never used
-            const float* base = a.x + (int64_t)(p.row - 1 + prow[j]) * row_floats_x + cb * 64;
-            const uint32_t bytes = row_ok ? (uint32_t)(row_floats_x - cb * 64) * 4 : 0u;
-            const __amdgpu_buffer_rsrc_t r = __builtin_amdgcn_make_buffer_rsrc((void*)base, 0, bytes, 0x00020000);
+            const uint32_t gy = (uint32_t)(p.y0 - 1 + prow[j]);
+            const uint32_t row_bytes = (j < 2 || third_row_live) ? live_bytes : 0u;
+            const uint32_t bytes = gy < (uint32_t)a.H ? row_bytes : 0u;
+            const __amdgpu_buffer_rsrc_t r =
+                __builtin_amdgcn_make_buffer_rsrc((void*)(xrow0[j] + strip_row), 0, bytes, 0x00020000);
             rawr[j] = __builtin_bit_cast(float4_t, __builtin_amdgcn_raw_buffer_load_b128(r, xoff[j] + strip_off, 0, 0));
         }
     };
@@ -792,13 +801,16 @@ __global__ __launch_bounds__(WW_THREADS, 1) void winograd_wgrad_kernel(const Win
 #pragma unroll
         for (int b = 0; b < 2; ++b) dyoff[j][b] = (uint32_t)((4 * j + 2 * h + b) * a.K + kb * 64 + wm * 32 + cl) * 4;
     float dyr[2][2][4];                        // [row a][column b][j]
+    const uint32_t row_pitch_dy = (uint32_t)(a.W * a.K) * 4;
     auto load_dy = [&](const StripPos& p, bool valid) {
+        const uint32_t live_bytes = valid ? (uint32_t)((a.W - p.x0) * a.K) * 4 : 0u;
+        const char* row0 = (const char*)a.dy + (uint64_t)(uint32_t)(p.row * a.W + p.x0) * (uint32_t)(a.K * 4);
 #pragma unroll
         for (int r = 0; r < 2; ++r) {
-            const bool row_ok = valid && p.y0 + r < a.H;
-            const float* base = a.dy + (int64_t)((p.row + r) * a.W + p.x0) * a.K;
-            const uint32_t bytes = row_ok ? (uint32_t)((a.W - p.x0) * a.K) * 4 : 0u;
-            const __amdgpu_buffer_rsrc_t rs = __builtin_amdgcn_make_buffer_rsrc((void*)base, 0, bytes, 0x00020000);
+            // the strip's first row always lies in the image, its second may not (odd H)
+            const uint32_t bytes = (r == 0 || p.y0 + 1 < a.H) ? live_bytes : 0u;
+            const __amdgpu_buffer_rsrc_t rs =
+                __builtin_amdgcn_make_buffer_rsrc((void*)(row0 + (r ? row_pitch_dy : 0u)), 0, bytes, 0x00020000);
 #pragma unroll
             for (int b = 0; b < 2; ++b)
 #pragma unroll
@@ -807,6 +819,7 @@ __global__ __launch_bounds__(WW_THREADS, 1) void winograd_wgrad_kernel(const Win
         }
     };
     float rr[2][2][4];                         // rows 2gh, 2gh+1 of A dY (signs of row 3 left out): [ii][b][j]
+    const float rr_c0 = gh ? -1.f : 0.f, rr_c1 = gh ? 0.f : 1.f;
 
     float16_t acc[WG_GW];
 #pragma unroll
@@ -857,15 +870,13 @@ __global__ __launch_bounds__(WW_THREADS, 1) void winograd_wgrad_kernel(const Win
             for (int b = 0; b < 2; ++b)
 #pragma unroll
                 for (int j = 0; j < 4; ++j) {
-                    rr[0][b][j] = gh ? dyr[0][b][j] - dyr[1][b][j] : dyr[0][b][j];
-                    rr[1][b][j] = gh ? dyr[1][b][j] : dyr[0][b][j] + dyr[1][b][j];
+                    // rows (0, 0+1) for the first GEMM half, (0-1, 1) for the second: one fma each with the
+                    // wave's constants instead of computing both forms and selecting
+                    rr[0][b][j] = __builtin_fmaf(rr_c0, dyr[1][b][j], dyr[0][b][j]);
+                    rr[1][b][j] = __builtin_fmaf(rr_c1, dyr[0][b][j], dyr[1][b][j]);
                 }
             load_dy(dp, d_left > 0);           // strip q+1
             next_d();
-            if (gh == 0 && wn == 0) {          // the waves that write the bias gradient at the end
-#pragma unroll
-                for (int j = 0; j < 4; ++j) db_acc += rr[1][0][j] + rr[1][1][j];
-            }
             __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
             for (int gp = 0; gp < WG_GW / 2; ++gp) {
@@ -876,6 +887,12 @@ __global__ __launch_bounds__(WW_THREADS, 1) void winograd_wgrad_kernel(const Win
                 for (int j = 0; j < 4; ++j) {
                     a0[j] = (gp & 1) ? rr[ii][0][j] - rr[ii][1][j] : rr[ii][0][j];
                     a1[j] = (gp & 1) ? rr[ii][1][j] : rr[ii][0][j] + rr[ii][1][j];
+                }
+                // the waves that write the bias gradient at the end: their a1 is now the sum of dY over a
+                // tile's four pixels
+                if (gp == 2 && gh == 0 && wn == 0) {
+#pragma unroll
+                    for (int j = 0; j < 4; ++j) db_acc += a1[j];
                 }
 #pragma unroll
                 for (int k = 0; k < 8; ++k) {
