@@ -406,11 +406,16 @@ __global__ __launch_bounds__(WG_THREADS, 1) void winograd_fwd_kernel(const WinoA
                     const float part[4] = {s0[0] + s0[1] + s0[2], s0[1] - s0[2] - s0[3], s1[0] + s1[1] + s1[2],
                                            s1[1] - s1[2] - s1[3]};
                     // (each staging element belongs to one lane of one wave per phase: plain read-add-write)
-                    float prev[4];
+                    if (add) {
+                        float prev[4];
 #pragma unroll
-                    for (int i = 0; i < 4; ++i) prev[i] = add ? stg_lane[stg_index(e, i)] : 0.f;
+                        for (int i = 0; i < 4; ++i) prev[i] = stg_lane[stg_index(e, i)];
 #pragma unroll
-                    for (int i = 0; i < 4; ++i) stg_lane[stg_index(e, i)] = prev[i] + part[i];
+                        for (int i = 0; i < 4; ++i) stg_lane[stg_index(e, i)] = prev[i] + part[i];
+                    } else {                   // (not 0 + part: that addition would be kept, for the sign of zero)
+#pragma unroll
+                        for (int i = 0; i < 4; ++i) stg_lane[stg_index(e, i)] = part[i];
+                    }
                     // four rows at a time may overlap (their chains of additions and LDS round trips are
                     // independent); more would need more registers than a wave has left here
                     if ((e & 3) == 3) __builtin_amdgcn_sched_barrier(0);
