@@ -267,6 +267,35 @@ def test_convolution_with_pooling_in_its_epilogue_equals_the_two_layers(N, C, K,
         torch.testing.assert_close(pb.grad, pc.grad, rtol=1e-5, atol=1e-5 * float(pc.grad.abs().max()))
 
 
+def _wgrad_shapes(count, seed):
+    rng = np.random.RandomState(seed)
+    shapes = [(4, 64, 64, 97, 131),      # several strips per block, images change inside a block's range
+              (1, 64, 64, 1, 1), (2, 128, 64, 1, 37), (3, 64, 128, 29, 1), (1, 256, 64, 5, 16)]
+    for _ in range(count):
+        shapes.append((int(rng.randint(1, 6)), int(rng.choice([64, 128])), int(rng.choice([64, 128, 256])),
+                       int(rng.randint(1, 51)), int(rng.randint(1, 51))))
+    return shapes
+
+
+@pytest.mark.parametrize("N,C,K,H,W", _wgrad_shapes(10, seed=7))
+def test_winograd_weight_gradient_on_ragged_images(N, C, K, H, W, conv_algorithm):
+    """The Winograd weight-gradient kernel alone (channel counts it takes, no ReLU mask) on image sizes that
+    leave half strips at the right and bottom edges, single rows and columns, and strip ranges that cross
+    from one image into the next: weight and bias gradients against torch in fp64."""
+    if conv_algorithm != "winograd":
+        pytest.skip("covers the Winograd kernel")
+    g = torch.Generator().manual_seed(H * 100 + W)
+    x = torch.randn(N, C, H, W, generator=g)
+    dy = torch.randn(N, K, H, W, generator=g)
+    wd = torch.zeros(K, C, 3, 3, dtype=torch.float64, requires_grad=True)
+    bd = torch.zeros(K, dtype=torch.float64, requires_grad=True)
+    F.conv2d(x.double(), wd, bd, padding=1).backward(dy.double())
+    dw, db = ops.conv3x3_weight_grad(_nhwc(x), _nhwc(dy))
+    R = N * H * W
+    torch.testing.assert_close(dw.cpu().double(), wd.grad, rtol=1e-5, atol=4e-7 * math.sqrt(R) * 4)
+    torch.testing.assert_close(db.cpu().double(), bd.grad, rtol=1e-5, atol=4e-7 * math.sqrt(R) * 4)
+
+
 def test_winograd_impulse_response_and_brute_force():
     # the Winograd path on shapes it accepts: (a) brute-force direct convolution of a small case with
     # random (asymmetric) filters; (b) a unit impulse must return the flipped filter taps around it
