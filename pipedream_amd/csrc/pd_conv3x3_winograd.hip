@@ -211,13 +211,16 @@ __global__ __launch_bounds__(WG_THREADS, 1) void winograd_fwd_kernel(const WinoA
                     float4_t, __builtin_amdgcn_raw_buffer_load_b128(mr, loff[j], chunk * (WG_CC * 4), 0));
         }
     };
-    auto store_raw = [&](int stage, int j) {
+    auto store_raw_at = [&](float* dst, int j) {
         float4_t v = rawr[j];
         if (MASK) {
 #pragma unroll
             for (int c = 0; c < 4; ++c) v[c] = rawm[MASK ? j : 0][c] > 0.f ? v[c] : 0.f;
         }
-        if (j == 0 || second_piece) *(float4_t*)(lds + WG_RAW_OFF + stage * WG_RAW_STAGE + raw_dst[j]) = v;
+        if (j == 0 || second_piece) *(float4_t*)dst = v;
+    };
+    auto store_raw = [&](int stage, int j) {
+        store_raw_at(lds + WG_RAW_OFF + stage * WG_RAW_STAGE + raw_dst[j], j);
     };
 
     // ---- stage 2 role: tile tt, channel half cg and row ti of B^T d, which is  Ra + sgn * Rb  of two
@@ -238,6 +241,11 @@ __global__ __launch_bounds__(WG_THREADS, 1) void winograd_fwd_kernel(const WinoA
         dc[s & 1][0] = *(const float4_t*)(rs + src_a + o);
         dc[s & 1][1] = *(const float4_t*)(rs + src_b + o);
     };
+    auto read_col_at = [&](const float* ra, const float* rb, int s) {   // the same through per-lane pointers
+        const int o = (((s & 1) * WG_HALO) * WG_RAW_PITCH + (s >> 1)) * 4;
+        dc[s & 1][0] = *(const float4_t*)(ra + o);
+        dc[s & 1][1] = *(const float4_t*)(rb + o);
+    };
     auto transform_col = [&](int s) { t[s] = dc[s & 1][0] + sgn * dc[s & 1][1]; };
     float4_t vout;
     auto transform_out = [&](int m) {
@@ -249,6 +257,7 @@ __global__ __launch_bounds__(WG_THREADS, 1) void winograd_fwd_kernel(const WinoA
     auto store_out = [&](float* vst, int m) {
         *(float4_t*)(vst + (ti * 4 + m) * (2 * WG_FRAG) + twm * WG_FRAG + lane * 4) = vout;
     };
+    auto store_out_at = [&](float* pv, int m) { *(float4_t*)(pv + m * (2 * WG_FRAG)) = vout; };
 
     // ---- stage 3 role: wave (gh, wm, wn) owns GEMMs gh*8..+7 of tiles wm*32..+31 x channels wn*32..+31
     const int gh = wave >> 2, wm = (wave >> 1) & 1, wn = wave & 1;
@@ -314,15 +323,20 @@ __global__ __launch_bounds__(WG_THREADS, 1) void winograd_fwd_kernel(const WinoA
     // section, which then requests the first fragments and patch column of the next step while its own
     // MFMAs (operands already in registers) run.  The reduction index of MFMA j pairs channel j (lanes
     // 0-31) with channel 4+j (lanes 32-63).
+    // The LDS stages alternate with the parity of the step.  Every per-lane address that depends on it is a
+    // pointer carried through the loop and moved to the other stage once per step, after its last use in the
+    // step (one vector addition each, instead of rebuilding index * 4 + stage offset for every use).
     int q = 0;                                 // step of stage 3
+    int dv = WG_V_STAGE, dr = WG_RAW_STAGE;    // signed distances to the other stage, flipped every step
+    const float* pa = lds + a_lane;                                            // A fragments: stage q & 1
+    float* pv = lds + WG_V_STAGE + ti * 4 * (2 * WG_FRAG) + twm * WG_FRAG + lane * 4;   // stage 2 output: (q+1) & 1
+    const float* pra = lds + WG_RAW_OFF + WG_RAW_STAGE + src_a;                // patch rows: (q+1) & 1
+    const float* prb = lds + WG_RAW_OFF + WG_RAW_STAGE + src_b;
+    float* pw0 = lds + WG_RAW_OFF + raw_dst[0];                                // stage 1 output: q & 1
+    float* pw1 = lds + WG_RAW_OFF + raw_dst[1];
     for (int m_i = 0; m_i < n_my; ++m_i) {
     zero_acc();
     for (int m_cc = 0; m_cc < a.n_chunks; ++m_cc, ++q) {
-        const float* vs = lds + (q & 1) * WG_V_STAGE + a_lane;
-        const float* vs_next = lds + ((q + 1) & 1) * WG_V_STAGE + a_lane;
-        float* vn = lds + ((q + 1) & 1) * WG_V_STAGE;
-        const float* rs = lds + WG_RAW_OFF + ((q + 1) & 1) * WG_RAW_STAGE;   // step q+1, transformed now
-        const float* rs_next = lds + WG_RAW_OFF + (q & 1) * WG_RAW_STAGE;    // step q+2, stored in section 1
         const int ustep = u_kb * a.n_chunks + u_cc;
 #pragma unroll
         for (int gp = 0; gp < WG_GW / 2; ++gp) {
@@ -336,31 +350,37 @@ __global__ __launch_bounds__(WG_THREADS, 1) void winograd_fwd_kernel(const WinoA
                     acc[g1] = __builtin_amdgcn_mfma_f32_32x32x2f32(af[cur][1][j], uf[g1][j], acc[g1], 0, 0, 0);
                 if (k == 0) {
                     if (gp < 3) {              // A fragments of the next section
-                        af[cur ^ 1][0] = *(const float4_t*)(vs + (g0 + 2) * (2 * WG_FRAG));
-                        af[cur ^ 1][1] = *(const float4_t*)(vs + (g1 + 2) * (2 * WG_FRAG));
+                        af[cur ^ 1][0] = *(const float4_t*)(pa + (g0 + 2) * (2 * WG_FRAG));
+                        af[cur ^ 1][1] = *(const float4_t*)(pa + (g1 + 2) * (2 * WG_FRAG));
                     } else {
-                        store_out(vn, 3);
+                        store_out_at(pv, 3);
                         __syncthreads();       // stage 2 of step q+1 and stage 1 of step q+2 are in LDS
-                        af[0][0] = *(const float4_t*)(vs_next);
-                        af[0][1] = *(const float4_t*)(vs_next + (2 * WG_FRAG));
-                        read_col(rs_next, 0);
+                        af[0][0] = *(const float4_t*)(pa);         // (pa, pra, prb moved on in section 2)
+                        af[0][1] = *(const float4_t*)(pa + (2 * WG_FRAG));
+                        read_col_at(pra, prb, 0);
                     }
                 }
                 // stage 2 of step q+1: columns 0..3 of the patch, then the four output vectors
-                if (gp == 0 && k == 1) read_col(rs, 1);
+                if (gp == 0 && k == 1) read_col_at(pra, prb, 1);
                 if (gp == 0 && k == 3) transform_col(0);
-                if (gp == 0 && k == 4) read_col(rs, 2);
+                if (gp == 0 && k == 4) read_col_at(pra, prb, 2);
                 if (gp == 0 && k == 6) transform_col(1);
-                if (gp == 1 && k == 1) read_col(rs, 3);
+                if (gp == 1 && k == 1) read_col_at(pra, prb, 3);
                 if (gp == 1 && k == 3) transform_col(2);
                 if (gp == 1 && k == 6) transform_col(3);
                 if (gp == 2 && (k == 1 || k == 3 || k == 5)) transform_out(k >> 1);
-                if (gp == 2 && (k == 2 || k == 4 || k == 6)) store_out(vn, (k >> 1) - 1);
+                if (gp == 2 && (k == 2 || k == 4 || k == 6)) store_out_at(pv, (k >> 1) - 1);
                 if (gp == 2 && k == 7) transform_out(3);
                 // stage 1: the registers hold step q+2 (requested a step ago); then request step q+3
-                if (gp == 1 && k == 2) store_raw(q & 1, 0);
-                if (gp == 1 && k == 4) store_raw(q & 1, 1);
+                if (gp == 1 && k == 2) store_raw_at(pw0, 0);
+                if (gp == 1 && k == 4) store_raw_at(pw1, 1);
                 if (gp == 1 && k == 5) load_raw(l_cc);
+                // the pointers move to the other stage after their last use of the step
+                if (gp == 1 && k == 7) { pra -= dr; prb -= dr; }
+                if (gp == 2 && k == 2) pw0 += dr;
+                if (gp == 2 && k == 4) pw1 += dr;
+                if (gp == 2 && k == 6) pa += dv;
+                if (gp == 3 && k == 1) pv -= dv;
                 if (k == 7) {                  // the filter fragments of this pair, for step q+1
                     uf[g0] = load_u(ustep, g0);
                     uf[g1] = load_u(ustep, g1);
@@ -370,6 +390,8 @@ __global__ __launch_bounds__(WG_THREADS, 1) void winograd_fwd_kernel(const WinoA
         }
         advance_l();
         advance_u();
+        dv = -dv;
+        dr = -dr;
     }
         {
             // ---- epilogue of item m_i.  Each wave applies A^T . A to its two rows of M (lane-local);
