@@ -132,3 +132,10 @@ def test_argument_validation_of_the_sequence_and_pooling_entry_points():
         lib.pd_conv3x3_winograd_fwd_pool_nhwc_f32(p, p, None, p, p, 1, 8, 8, 12, 32, 1, None)
     with pytest.raises(E, match="too large"):
         lib.pd_conv3x3_winograd_fwd_nhwc_f32(p, p, None, None, None, p, 1, 4096, 4096, 64, 64, 0, None)
+    # Winograd weight gradient: channel counts, a batch whose pixels overflow its 32-bit row counter, workspace
+    with pytest.raises(E, match="unsupported channel counts"):
+        lib.pd_conv3x3_winograd_wgrad_nhwc_f32(p, p, p, p, p, 1 << 30, 1, 8, 8, 48, 64, None)
+    with pytest.raises(E, match="too many pixels"):
+        lib.pd_conv3x3_winograd_wgrad_nhwc_f32(p, p, p, p, p, 1 << 30, 70000, 224, 224, 64, 64, None)
+    with pytest.raises(E, match="workspace too small"):
+        lib.pd_conv3x3_winograd_wgrad_nhwc_f32(p, p, p, p, p, 1024, 1, 8, 8, 64, 64, None)
