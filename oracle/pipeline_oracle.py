@@ -12,6 +12,14 @@ Stage compute is the installed torch library on CPU (``torch.nn`` modules +
 contract is the reference's: a forward-received fp32 tensor becomes a leaf that
 requires grad (runtime/communication.py:595-596), what is sent is detached (:699), and
 backward pops the oldest in-flight minibatch (runtime/runtime.py:571).
+
+How ``run_pipeline`` is pinned (tests/test_oracle_pipeline_pin.py, tests/test_pipeline_mlp.py): its
+event order against the closed form of the 1F1B loop; its numbers, bit for bit, (i) with all
+warm-up depths 0 against the unsplit ``nn.Sequential`` under the library's ``torch.optim.SGD`` /
+``Adam``, and (ii) with depths S-1-s against a loop written from the definition of weight stashing
+(one ``deepcopy`` of a stage per version, forward and backward of minibatch k through copy
+``max(0, k - W)``); mutants of this function (dropped ``detach``, wrong version, LIFO, missing
+leaf, perturbed hand-off gradient) fail those pins.
 """
 import collections
 
