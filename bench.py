@@ -74,9 +74,9 @@ class Downstream(object):
         self.i = 0
 
     def after_forward(self):
-        self.fabric.queue("out0", 1, False).popleft()
-        self.fabric.queue("target", 1, False).popleft()
-        self.fabric.queue("out0", 0, True).append(self.grads[self.i % len(self.grads)])
+        self.fabric.take("out0", 1, False)
+        self.fabric.take("target", 1, False)
+        self.fabric.put("out0", 0, True, self.grads[self.i % len(self.grads)])
         self.i += 1
 
 

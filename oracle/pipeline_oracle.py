@@ -45,13 +45,16 @@ class StageOracle(object):
         self.bwd_versions = []
 
 
-def run_pipeline(stage_modules, criterion, make_optimizer, batches, warmups=None, on_loss=None):
+def run_pipeline(stage_modules, criterion, make_optimizer, batches, warmups=None, on_loss=None, lr_schedule=None):
     """Run ``len(batches)`` minibatches through the stages with 1F1B + weight stashing.
 
     ``stage_modules``: CPU modules, stage 0 first; ``make_optimizer(stage_index, module,
     num_versions)`` returns a ``StashingOptimizerOracle``; ``batches``: list of
     ``(input, target)``; ``warmups``: warm-up depth per stage (default: straight pipeline,
-    S-1-s).  Returns (losses in minibatch order, list of StageOracle)."""
+    S-1-s); ``lr_schedule(stage_index, i)``: learning rate written into every param group after
+    the i-th steady-state forward of a stage, as ``adjust_learning_rate`` is called at
+    main_with_runtime.py:368 (warm-up forwards do not touch it).
+    Returns (losses in minibatch order, list of StageOracle)."""
     S = len(stage_modules)
     n = len(batches)
     if warmups is None:
@@ -99,6 +102,9 @@ def run_pipeline(stage_modules, criterion, make_optimizer, batches, warmups=None
                         st.in_flight.append((x, out))
                         fwd_q[s + 1].append(out.detach())
                         tgt_q[s + 1].append(target)
+                    if lr_schedule is not None and k >= min(st.warmup, n):
+                        for group in st.optimizer.param_groups:
+                            group["lr"] = lr_schedule(s, k - min(st.warmup, n))
                 else:
                     opt = st.optimizer
                     opt.zero_grad()

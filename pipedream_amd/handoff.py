@@ -1,20 +1,42 @@
-"""Device-buffer hand-off of activations and gradients between co-resident stages.
+"""Device-buffer hand-off of activations, gradients and acknowledgements between co-resident stages.
 
-On one GPU the stages of a pipeline live in one process, so the transport of the
-reference's ``CommunicationHandler`` (helper threads + ``torch.distributed`` send/recv,
-runtime/communication.py:610-712) collapses to passing the device tensor itself.  What
-is kept is its queue contract (runtime/communication.py:583-608):
+On one GPU the stages of a pipeline live in one process, so the transport of the reference's
+``CommunicationHandler`` (helper threads + ``torch.distributed`` send/recv,
+runtime/communication.py:610-712) collapses to passing the device tensor itself.  What is kept is
+its queue contract (runtime/communication.py:583-608):
 
 * one FIFO per tensor name, receiver and direction;
-* a tensor received in the forward direction becomes a gradient-requiring leaf when it
-  is fp32 (:595-596);
-* what is sent is detached from the sender's autograd graph (:699) -- without the copy,
-  because neither side writes into a hand-off buffer afterwards.
+* a tensor received in the forward direction becomes a gradient-requiring leaf when it is fp32
+  (:595-596);
+* what is sent is detached from the sender's autograd graph (:699) -- without the copy, because
+  neither side writes into a hand-off buffer afterwards;
+* in a forward-only run an ``ack`` travels in the backward direction as the clock that keeps a stage
+  from running ahead of its consumer (runtime/communication.py:193-211, runtime/runtime.py:629-653).
 
-All stages launch on torch's current stream, so queue order is execution order and no
-events are needed.
+Added to it: every parcel carries the minibatch number it belongs to (the receiver checks that it
+takes them in order) and a ``premasked`` flag, the producer's statement about who applies the backward
+pass of the ReLU that ends the producing stage (see ``StageRuntime``).
+
+All stages launch on torch's current stream, so queue order is execution order and no events are
+needed.
 """
 import collections
+
+import torch
+
+ACK = "ack"
+
+Parcel = collections.namedtuple("Parcel", "tensor seq premasked")
+
+
+class HandoffContractError(RuntimeError):
+    """Producer and consumer of a hand-off disagree about the gradient they exchange."""
+
+
+def becomes_leaf(tensor):
+    """A received tensor of this kind takes part in the consumer's backward pass and gets a gradient
+    sent back (runtime/communication.py:595)."""
+    return torch.is_tensor(tensor) and tensor.dtype == torch.float32
 
 
 class HandoffFabric(object):
@@ -27,12 +49,21 @@ class HandoffFabric(object):
     def queue(self, tensor_name, receiver_rank, backward):
         return self.queues[(tensor_name, receiver_rank, bool(backward))]
 
+    def put(self, tensor_name, receiver_rank, backward, tensor, seq=None, premasked=False):
+        """Queue ``tensor`` for ``receiver_rank``; also the way a test or a benchmark plays a neighbour
+        stage that is not there."""
+        self.bytes_sent += tensor.element_size() * tensor.nelement()
+        self.queue(tensor_name, receiver_rank, backward).append(Parcel(tensor.detach(), seq, bool(premasked)))
+
+    def take(self, tensor_name, receiver_rank, backward):
+        return self.queue(tensor_name, receiver_rank, backward).popleft()
+
 
 _FABRICS = {}
 
 
 def fabric_for(key):
-    """Stages created with the same ``(master_addr, master_port)`` share a fabric."""
+    """Stages created with the same key (``(master_addr, master_port)``) share a fabric."""
     if key not in _FABRICS:
         _FABRICS[key] = HandoffFabric()
     return _FABRICS[key]
@@ -43,78 +74,55 @@ def reset_fabrics():
 
 
 class DeviceHandoff(object):
-    """Per-stage endpoint with the ``recv`` / ``send`` signature of the reference's
-    ``CommunicationHandler`` (runtime/communication.py:583-608)."""
+    """One stage's end of the fabric.  ``inbound`` / ``outbound`` map a tensor name to the rank it comes
+    from / goes to in the forward direction; gradients and acknowledgements take the same routes
+    backwards."""
 
-    def __init__(self, master_addr, master_port, rank, local_rank, num_ranks_in_server, world_size, fp16,
-                 backend):
+    def __init__(self, fabric_key, rank, inbound, outbound, ack_to=None):
         self.rank = rank
-        self.local_rank = local_rank
-        self.world_size = world_size
-        self.backend = backend
-        self.fabric = fabric_for((master_addr, master_port))
+        self.fabric = fabric_for(fabric_key)
+        self.inbound = dict(inbound)
+        self.outbound = dict(outbound)
+        self.forward_only = False
+        self._ack = None
+        self._ack_to = ack_to          # rank of the previous stage, None for the first
 
-    def initialize(self, receive_ranks, send_ranks, tensor_tags, target_tensor_names, training_tensor_dtypes,
-                   rank_in_stage, num_ranks_in_stage, ranks_in_previous_stage, ranks_in_next_stage):
-        self.receive_ranks = receive_ranks
-        self.send_ranks = send_ranks
-        self.tensor_tags = tensor_tags
-        self.target_tensor_names = target_tensor_names
-        self.training_tensor_dtypes = training_tensor_dtypes
-        self.rank_in_stage = rank_in_stage
-        self.num_ranks_in_stage = num_ranks_in_stage
-        self.ranks_in_previous_stage = ranks_in_previous_stage
-        self.ranks_in_next_stage = ranks_in_next_stage
-        # Targets travel with the activations from stage to stage; the reference adds them
-        # to the (shared) rank tables here too (runtime/communication.py:165-200).
-        for name in target_tensor_names:
-            if len(ranks_in_previous_stage) > 0:
-                receive_ranks[name] = ranks_in_previous_stage
-            if len(ranks_in_next_stage) > 0:
-                send_ranks[name] = ranks_in_next_stage
-        for name, ranks in list(receive_ranks.items()) + list(send_ranks.items()):
-            if len(ranks) != 1:
-                raise NotImplementedError(
-                    "tensor %r is exchanged with %d ranks; replicated stages need more than one GPU"
-                    % (name, len(ranks)))
-
-    # helper threads do not exist here; the calls are kept so callers need not change
-    def set_tensor_shapes(self, tensor_shapes):
-        self.tensor_shapes = tensor_shapes
-
-    def start_helper_threads(self, num_iterations, forward_only):
+    def begin_run(self, forward_only):
+        """Start of a ``train`` / ``eval`` run.  Whatever still waits for this stage in the backward
+        direction is left over from an earlier run (its senders act only on what this stage hands them in
+        the current one) and is dropped; the forward direction may already hold the first minibatches of
+        an upstream stage that started earlier and is kept."""
         self.forward_only = forward_only
-
-    def increment_messaging_index(self, sending):
-        pass
+        for (name, receiver, backward), q in self.fabric.queues.items():
+            if receiver == self.rank and backward:
+                q.clear()
 
     def wait(self):
-        pass
+        """The reference joins its helper threads here (runtime/communication.py:357-367); device
+        tensors handed over in-process are complete when queued."""
 
-    # ---------------------------------------------------------------------------------
-    def _recv_queue(self, tensor_name, backward):
-        return self.fabric.queue(tensor_name, self.rank, backward)
+    def ready(self, names, backward):
+        return all(len(self.fabric.queue(n, self.rank, backward)) > 0 for n in names)
 
-    def can_recv(self, tensor_name, backward=False):
-        return len(self._recv_queue(tensor_name, backward)) > 0
-
-    def recv(self, tensor_name, forward_minibatch_id, backward_minibatch_id, backward=False):
-        q = self._recv_queue(tensor_name, backward)
+    def take(self, tensor_name, seq, backward):
+        q = self.fabric.queue(tensor_name, self.rank, backward)
         if not q:
             raise RuntimeError(
                 "stage rank %s: nothing queued for %r (%s); the schedule ran this stage before its "
                 "neighbour produced the tensor" % (self.rank, tensor_name, "backward" if backward else "forward"))
-        tensor = q.popleft()
-        if not backward:
-            import torch
-            if tensor.dtype == torch.float32:
-                tensor = tensor.requires_grad_()
-        return tensor
+        parcel = q.popleft()
+        if parcel.seq is not None and parcel.seq != seq:
+            raise RuntimeError("stage rank %s: %r of minibatch %s arrived where minibatch %s was due"
+                               % (self.rank, tensor_name, parcel.seq, seq))
+        if not backward and becomes_leaf(parcel.tensor):
+            parcel = parcel._replace(tensor=parcel.tensor.requires_grad_())
+        return parcel
 
-    def send(self, tensor_name, tensor, forward_minibatch_id, backward_minibatch_id, backward=False):
-        if backward:
-            dst = self.receive_ranks[tensor_name][0]
-        else:
-            dst = self.send_ranks[tensor_name][0]
-        self.fabric.bytes_sent += tensor.element_size() * tensor.nelement()
-        self.fabric.queue(tensor_name, dst, backward).append(tensor.detach())
+    def put(self, tensor_name, tensor, seq, backward, premasked=False):
+        receiver = self.inbound[tensor_name] if backward else self.outbound[tensor_name]
+        self.fabric.put(tensor_name, receiver, backward, tensor, seq, premasked)
+
+    def put_ack(self, seq):
+        if self._ack is None:
+            self._ack = torch.zeros(1, dtype=torch.int64, device="cuda")
+        self.fabric.put(ACK, self._ack_to, True, self._ack, seq)

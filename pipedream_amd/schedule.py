@@ -7,7 +7,8 @@ then ``n - W`` times [forward, adjust lr, zero_grad, load_old_params, backward,
 load_new_params, step], then ``W`` times the backward half.  In the reference every
 stage is its own process and simply blocks in a receive queue; here the loop is a
 generator that yields whenever its next receive would find the queue empty, and
-``run_pipeline`` round-robins the generators until all are finished.
+``run_pipeline`` round-robins the generators until all are finished.  ``stage_eval_loop`` is the
+forward-only counterpart (``validate()``, main_with_runtime.py:429-487) with the ``ack`` clock.
 """
 
 
@@ -54,6 +55,31 @@ def stage_train_loop(r, optimizer, num_minibatches, loader=None, lr_schedule=Non
     for _ in range(warmup):
         for blocked in backward_and_update():
             yield blocked
+    r.wait()
+
+
+def stage_eval_loop(r, num_minibatches, loader=None, on_forward=None, no_input_pipelining=False):
+    """Generator running one stage's forward-only schedule, the body of ``validate()`` in the
+    reference's caller (runtime/image_classification/main_with_runtime.py:429-487): ``W`` warm-up
+    forwards, then ``n - W`` times [forward, ack].  The ack is the clock: a stage takes its next
+    steady-state minibatch only after its consumer has acknowledged the oldest outstanding one.
+    Call it under ``torch.no_grad()`` as the reference does.  ``on_forward(i, r)`` is called after each
+    steady-state forward (where the reference reads ``r.output`` / ``r.loss``)."""
+    n = num_minibatches
+    r.eval(n)
+    r.set_loader(loader if (r.stage is None or r.stage == 0) else None)
+    warmup = 0 if no_input_pipelining else min(r.num_warmup_minibatches, n)
+    for i in range(n):
+        while not r.can_run_forward():
+            yield r
+        r.run_forward()
+        if i < warmup:
+            continue
+        if on_forward is not None:
+            on_forward(i - warmup, r)
+        while not r.can_run_ack():
+            yield r
+        r.run_ack()
     r.wait()
 
 

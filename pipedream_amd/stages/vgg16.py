@@ -74,7 +74,9 @@ class Stage0(torch.nn.Module):
 
 class Stage1(torch.nn.Module):
     """Stage 1 of the 4-way split.  Its last ReLU's backward is applied by ``Stage2`` (the first convolution
-    there masks its input gradient), so the gradient this stage receives must come from ``Stage2``."""
+    there masks its input gradient), so the gradient this stage receives must come from ``Stage2``:
+    ``premasked_output_grads`` states it, ``StageRuntime`` checks it on every hand-off."""
+    premasked_output_grads = (True,)
 
     def __init__(self):
         super(Stage1, self).__init__()
@@ -93,8 +95,11 @@ class Stage1(torch.nn.Module):
 
 
 class Stage2(torch.nn.Module):
-    """Stage 2 of the 4-way split.  Takes ``Stage1``'s rectified output; its last ReLU's backward is applied
-    by the pooling layer that opens ``Stage3``."""
+    """Stage 2 of the 4-way split.  Takes ``Stage1``'s rectified output and applies that ReLU's backward to
+    the gradient it hands back (``masks_input_grads``); its own last ReLU's backward is applied by the
+    pooling layer that opens ``Stage3`` (``premasked_output_grads``)."""
+    masks_input_grads = (True,)
+    premasked_output_grads = (True,)
 
     def __init__(self):
         super(Stage2, self).__init__()
@@ -114,6 +119,10 @@ class Stage2(torch.nn.Module):
 
 
 class Stage3(torch.nn.Module):
+    """Last stage of the 4-way split; its opening ReLU + MaxPool applies the backward of ``Stage2``'s last
+    ReLU (``masks_input_grads``)."""
+    masks_input_grads = (True,)
+
     def __init__(self, dropout=0.5, num_classes=1000):
         super(Stage3, self).__init__()
         self.layer1 = layers.MaxPool2d(2, 2, relu=True)

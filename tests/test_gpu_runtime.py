@@ -1,0 +1,325 @@
+"""``StageRuntime`` pieces beyond the plain training pipeline, on the GPU against the CPU oracle:
+
+* a time-varying learning rate written into ``param_groups`` every iteration
+  (runtime/image_classification/main_with_runtime.py:368, 532-563) reaches the fused kernels as a
+  per-launch scalar: 2-stage MLP pipeline under SGD and one stashed stage under Adam, parameters within
+  rel 1e-5 of the oracle that applies the same rates;
+* forward-only runs with the ``ack`` clock (runtime/runtime.py:351-368, 376-379, 629-653): at most one
+  minibatch is kept, acknowledgements arrive in order and bound how far a stage runs ahead, outputs equal
+  the oracle's ``eval()`` forward;
+* the boundary contract about who applies a stage's last ReLU to the gradient: a producer / consumer pair
+  that disagrees raises instead of training on wrong gradients."""
+import pytest
+import torch
+
+from oracle import pipeline_oracle, stash_oracle as so
+
+pytestmark = pytest.mark.gpu
+
+SGD_KW = dict(lr=0.01, momentum=0.9, weight_decay=1e-4)
+
+
+def _runtimes(model, conf, n_stages, depth_map=None):
+    from pipedream_amd import handoff, runtime
+    handoff.reset_fabrics()
+    out = []
+    for rank in range(n_stages):
+        out.append(runtime.StageRuntime(
+            model=model, distributed_backend="gloo", fp16=False, loss_scale=1.0,
+            training_tensor_shapes={}, eval_tensor_shapes={}, training_tensor_dtypes={},
+            inputs_module_destinations={"input": 0}, target_tensor_names={"target"},
+            configuration_maps={"module_to_stage_map": conf["module_to_stage_map"],
+                                "stage_to_rank_map": conf["stage_to_rank_map"], "stage_to_depth_map": depth_map},
+            master_addr="127.0.0.1", rank=rank, local_rank=0, num_ranks_in_server=n_stages, verbose_freq=0,
+            model_type=runtime.IMAGE_CLASSIFICATION))
+    return out
+
+
+def _mlp_pair(d_in=48, d_hidden=64, d_out=10):
+    """The 2-stage MLP of the small configuration at a reduced width, product and oracle twins with the same
+    initial weights."""
+    from oracle import models
+    from pipedream_amd.layers import CrossEntropyLoss
+    from pipedream_amd.stages import mlp
+    torch.manual_seed(0)
+    ref = [models.MlpStage0(d_in, d_hidden), models.MlpStage1(d_hidden, d_out)]
+    model = mlp.model(CrossEntropyLoss(), d_in, d_hidden, d_out)
+    for (m, _, _), r in zip(model, ref):
+        m.load_state_dict(r.state_dict())
+    return model, ref
+
+
+def _batches(n, d_in=48, classes=10, batch=16, seed=3):
+    g = torch.Generator().manual_seed(seed)
+    return [(torch.randn(batch, d_in, generator=g), torch.randint(0, classes, (batch,), generator=g))
+            for _ in range(n)]
+
+
+def test_per_iteration_learning_rate_pipeline_sgd():
+    from pipedream_amd import lr_policy, schedule, sgd
+    from pipedream_amd.stages import mlp
+    n = 12
+    model, ref = _mlp_pair()
+    rts = _runtimes(model, mlp.conf(), 2)
+    opts = [sgd.SGDWithWeightStashing(r.modules(), r.master_parameters, r.model_parameters, 1.0,
+                                      num_versions=r.num_warmup_minibatches + 1, **SGD_KW) for r in rts]
+    batches = _batches(n)
+    # linear warm-up of the first epochs: a different rate at every step (main_with_runtime.py:545-546)
+    scheds = [lr_policy.schedule_for(r, base_lr=0.05, epoch=0, total_epochs=90, lr_policy="polynomial",
+                                     epoch_length=n, lr_warmup=True) for r in rts]
+    assert len({scheds[0](i) for i in range(n)}) == n
+    losses = []
+    seen_lr = [[], []]
+    loops = []
+    for s, (r, o) in enumerate(zip(rts, opts)):
+        def on_forward(i, rr, s=s, o=o):
+            seen_lr[s].append(o.param_groups[0]["lr"])
+            if s == 1:
+                losses.append(float(rr.loss.detach()))
+        loops.append(schedule.stage_train_loop(r, o, n, loader=batches if s == 0 else None,
+                                               lr_schedule=scheds[s], on_forward=on_forward))
+    schedule.run_pipeline(loops)
+    torch.cuda.synchronize()
+    assert seen_lr[1] == [scheds[1](i) for i in range(n)] and seen_lr[0] == [scheds[0](i) for i in range(n - 1)]
+
+    ref_losses, ref_st = pipeline_oracle.run_pipeline(
+        ref, torch.nn.CrossEntropyLoss(),
+        lambda s, m, nv: so.StashingOptimizerOracle("SGD", [m], m.parameters(), nv, **SGD_KW), batches,
+        lr_schedule=lambda s, i: so.adjust_learning_rate(0.05, 0, 90, "polynomial", i, n, lr_warmup=True))
+    assert [st.optimizer.versions() for st in ref_st] == [o.queue.versions() for o in opts]
+    for a, b in zip(losses, ref_losses):
+        assert abs(a - b) <= 1e-5 * abs(b) + 1e-6
+    for r, m in zip(rts, ref):
+        got = r.modules()[0].state_dict()
+        for k, v in m.state_dict().items():
+            torch.testing.assert_close(got[k].cpu(), v, rtol=1e-5, atol=1e-6, msg=k)
+    # the schedule mattered: a constant rate gives other parameters
+    assert seen_lr[1][0] != seen_lr[1][-1]
+
+
+def test_per_iteration_learning_rate_adam_stage():
+    """One stage under AdamWithWeightStashing, stash depth 3, the rate of the exponential-decay policy with
+    warm-up written into the param groups before every update."""
+    from oracle import models
+    from pipedream_amd import adam
+    from pipedream_amd.stages import mlp
+    torch.manual_seed(1)
+    ref = models.MlpStage0(40, 56)
+    mine = mlp.Stage0(40, 56)
+    mine.load_state_dict(ref.state_dict())
+    mine = mine.cuda()
+    kw = dict(lr=1e-3, betas=(0.9, 0.999), weight_decay=1e-4)
+    W, nv, n = 2, 3, 10
+    opt = adam.AdamWithWeightStashing([mine], list(mine.parameters()), None, 1.0, nv, **kw)
+    ora = so.StashingOptimizerOracle("Adam", [ref], ref.parameters(), nv, **kw)
+    g = torch.Generator().manual_seed(2)
+    xs = [torch.randn(8, 40, generator=g) for _ in range(n)]
+    gs = [torch.randn(8, 56, generator=g) * 1e-2 for _ in range(n)]
+    rate = lambda i: so.adjust_learning_rate(5e-3, 0, 10, "exponential_decay", i, n, lr_warmup=(i < 5)) * (0.5 if i >= 5 else 1)
+    pend_ref, pend = [], []
+    updates = 0
+    for kind, k in so.one_f_one_b(n, W):
+        if kind == "F":
+            pend_ref.append(ref(xs[k]))
+            pend.append(mine(xs[k].cuda()))
+            continue
+        for o in (ora, opt):
+            for group in o.param_groups:
+                group["lr"] = rate(updates)
+            o.zero_grad()
+            o.load_old_params()
+        pend_ref.pop(0).backward(gs[k])
+        pend.pop(0).backward(gs[k].cuda())
+        for o in (ora, opt):
+            o.load_new_params()
+            o.step()
+        updates += 1
+        assert opt.queue.versions() == ora.versions()
+    got = mine.state_dict()
+    for key, v in ref.state_dict().items():
+        # Adam divides by sqrt(v): an entry whose gradient is within rounding of zero moves by up to lr
+        # whatever the implementation, hence the absolute term of 0.05 lr
+        torch.testing.assert_close(got[key].cpu(), v, rtol=1e-5, atol=0.05 * 5e-3, msg=key)
+        assert float((got[key].cpu() - v).norm() / v.norm()) < 1e-5
+
+
+class _Tail(torch.nn.Module):
+    def __init__(self, d_in, d_out):
+        super(_Tail, self).__init__()
+        from pipedream_amd import layers
+        self.drop = layers.Dropout(0.5)
+        self.fc = layers.Linear(d_in, d_out)
+
+    def forward(self, x):
+        return self.fc(self.drop(x))
+
+
+def test_forward_only_run_with_ack_clock():
+    """Three stages (warm-up depths 2/1/0), 9 minibatches, under no_grad: the loop of validate()
+    (main_with_runtime.py:455-461)."""
+    from pipedream_amd import handoff, layers, schedule
+    from pipedream_amd.layers import CrossEntropyLoss
+    n = 9
+    torch.manual_seed(5)
+    ref = [torch.nn.Sequential(torch.nn.Linear(24, 32), torch.nn.ReLU()),
+           torch.nn.Sequential(torch.nn.Linear(32, 32), torch.nn.ReLU()),
+           torch.nn.Sequential(torch.nn.Dropout(0.5), torch.nn.Linear(32, 6))]
+    s0 = torch.nn.Sequential(layers.Linear(24, 32, relu=True))
+    s1 = torch.nn.Sequential(layers.Linear(32, 32, relu=True))
+    s2 = _Tail(32, 6)
+    s0[0].load_state_dict(ref[0][0].state_dict())
+    s1[0].load_state_dict(ref[1][0].state_dict())
+    s2.fc.load_state_dict(ref[2][1].state_dict())
+    model = [(s0, ["input0"], ["out0"]), (s1, ["out0"], ["out1"]), (s2, ["out1"], ["out2"]),
+             (CrossEntropyLoss(), ["out2"], ["loss"])]
+    conf = {"module_to_stage_map": [0, 1, 2, 2], "stage_to_rank_map": {"0": [0], "1": [1], "2": [2]}}
+    rts = _runtimes(model, conf, 3)
+    assert [r.num_warmup_minibatches for r in rts] == [2, 1, 0]
+    batches = _batches(n, d_in=24, classes=6)
+    outputs, losses = [], []
+    acks = [[] for _ in rts]
+    ahead = [0, 0, 0]
+    for s, r in enumerate(rts):
+        fwd, ack = r.run_forward, r.run_ack
+
+        def run_forward(fwd=fwd, r=r, s=s):
+            fwd()
+            assert len(r.tensors) == 1                      # runtime.py:376-379: nothing is kept for a backward
+            ahead[s] = max(ahead[s], r.forward_minibatch_id - r.backward_minibatch_id)
+
+        def run_ack(ack=ack, r=r, s=s):
+            acks[s].append(r.backward_minibatch_id)
+            ack()
+
+        r.run_forward, r.run_ack = run_forward, run_ack
+
+    def on_last(i, rr):
+        outputs.append(rr.output.detach().cpu())
+        losses.append(float(rr.loss))
+        assert not rr.output.requires_grad
+
+    with torch.no_grad():
+        schedule.run_pipeline([schedule.stage_eval_loop(r, n, loader=batches if s == 0 else None,
+                                                        on_forward=on_last if s == 2 else None)
+                               for s, r in enumerate(rts)])
+    torch.cuda.synchronize()
+    # every stage acknowledged n - W minibatches, in order, and never ran further ahead than W + 1
+    assert acks == [list(range(n - 2)), list(range(n - 1)), list(range(n))]
+    assert ahead == [3, 2, 1]
+    assert all(not m.training for r in rts for m in r.modules())
+    # values: the oracle's modules in eval() mode (dropout is the identity)
+    for m in ref:
+        m.eval()
+    crit = torch.nn.CrossEntropyLoss()
+    with torch.no_grad():
+        for (x, y), out, loss in zip(batches, outputs, losses):
+            want = ref[2](ref[1](ref[0](x)))
+            torch.testing.assert_close(out, want, rtol=1e-5, atol=1e-6)
+            assert abs(loss - float(crit(want, y))) <= 1e-5 * abs(float(crit(want, y))) + 1e-6
+    assert len(outputs) == n
+    # a training run right after it starts clean: stale acknowledgements are dropped, gradients flow again
+    fabric = rts[0].comm_handler.fabric
+    rts[0].train(1)
+    assert len(fabric.queue(handoff.ACK, 0, True)) == 0
+
+
+def _tiny_image_batches(n):
+    g = torch.Generator().manual_seed(0)
+    return [(torch.randn(1, 3, 16, 16, generator=g), torch.randint(0, 4, (1,), generator=g)) for _ in range(n)]
+
+
+class _PlainConsumer(torch.nn.Module):
+    """Takes a rectified activation but leaves the producer's ReLU backward to the producer."""
+
+    def __init__(self, channels):
+        super(_PlainConsumer, self).__init__()
+        from pipedream_amd import layers
+        self.conv = layers.Conv2d(channels, 8)
+
+    def forward(self, x):
+        return self.conv(x).mean(dim=(2, 3))
+
+
+def test_mismatched_relu_contract_raises():
+    from pipedream_amd import handoff
+    from pipedream_amd.layers import CrossEntropyLoss
+    from pipedream_amd.stages import vgg16
+    conf = {"module_to_stage_map": [0, 1, 2, 2], "stage_to_rank_map": {"0": [0], "1": [1], "2": [2]}}
+    # Stage1 leaves its last ReLU's backward to its consumer; this consumer does not apply it
+    model = [(vgg16.Stage0(), ["input0"], ["out0"]), (vgg16.Stage1(), ["out0"], ["out1"]),
+             (_PlainConsumer(256), ["out1"], ["out2"]), (CrossEntropyLoss(), ["out2"], ["loss"])]
+    rts = _runtimes(model, conf, 3)
+    for r in rts:
+        r.train(1)
+    rts[0].set_loader(_tiny_image_batches(1))
+    rts[0].run_forward()
+    rts[1].run_forward()
+    with pytest.raises(handoff.HandoffContractError, match="masks_input_grads"):
+        rts[2].run_forward()
+    # the producer also refuses a plain gradient that reaches it some other way (a replay driver, a peer
+    # that skipped the forward check)
+    fabric = rts[1].comm_handler.fabric
+    fabric.put("out1", 1, True, torch.zeros(1, 256, 4, 4, device="cuda"), seq=0, premasked=False)
+    with pytest.raises(handoff.HandoffContractError, match="premasked_output_grads"):
+        rts[1].run_backward()
+    # the other way round: Stage2 masks the gradient it returns, Stage0's output is not rectified
+    model = [(vgg16.Stage0(), ["input0"], ["out0"]), (vgg16.Stage2(), ["out0"], ["out1"]),
+             (CrossEntropyLoss(), ["out1"], ["loss"])]
+    rts = _runtimes(model, {"module_to_stage_map": [0, 1, 1], "stage_to_rank_map": {"0": [0], "1": [1]}}, 2)
+    for r in rts:
+        r.train(1)
+    rts[0].set_loader(_tiny_image_batches(1))
+    rts[0].run_forward()
+    with pytest.raises(handoff.HandoffContractError):
+        rts[1].run_forward()
+
+
+def test_matched_relu_contract_trains():
+    """The real Stage1 -> Stage2 pair passes the check in both directions and hands back the gradient of a
+    plain ReLU network: compared with torch autograd on the oracle's twins."""
+    from oracle import models
+    from pipedream_amd.layers import CrossEntropyLoss
+    from pipedream_amd.stages import vgg16
+    conf = {"module_to_stage_map": [0, 1, 2, 2], "stage_to_rank_map": {"0": [0], "1": [1], "2": [2]}}
+
+    class Head(torch.nn.Module):
+        masks_input_grads = (True,)
+
+        def __init__(self):
+            super(Head, self).__init__()
+            self.body = vgg16.Stage2()
+
+        def forward(self, x):
+            # Stage2 leaves its last ReLU's backward to whatever follows it; a second ReLU is the identity
+            # on the rectified output and applies exactly that mask to the gradient
+            return torch.relu(self.body(x)).mean(dim=(2, 3))
+
+    torch.manual_seed(0)
+    head = Head()
+    model = [(vgg16.Stage0(), ["input0"], ["out0"]), (vgg16.Stage1(), ["out0"], ["out1"]),
+             (head, ["out1"], ["out2"]), (CrossEntropyLoss(), ["out2"], ["loss"])]
+    ref = [models.VggStage0(), models.VggStage1(), models.VggStage2()]
+    for (m, _, _), r in zip(model[:2], ref[:2]):
+        m.load_state_dict(r.state_dict())
+    head.body.load_state_dict(ref[2].state_dict())
+    rts = _runtimes(model, conf, 3)
+    g = torch.Generator().manual_seed(0)
+    x = torch.randn(2, 3, 16, 16, generator=g)
+    y = torch.randint(0, 512, (2,), generator=g)
+    for r in rts:
+        r.train(1)
+    rts[0].set_loader([(x, y)])
+    for r in rts:
+        r.run_forward()
+    for r in reversed(rts):
+        r.run_backward()
+    torch.cuda.synchronize()
+    loss = torch.nn.functional.cross_entropy(ref[2](ref[1](ref[0](x))).mean(dim=(2, 3)), y)
+    loss.backward()
+    assert abs(float(rts[2].loss) - float(loss)) <= 1e-5 * float(loss)
+    for r, m in zip(rts, ref):
+        mod = r.modules()[0]
+        mod = mod.body if isinstance(mod, Head) else mod
+        for (k, p), (_, q) in zip(mod.named_parameters(), m.named_parameters()):
+            err = float((p.grad.cpu() - q.grad).norm() / q.grad.norm())
+            assert err < 1e-4, (k, err)

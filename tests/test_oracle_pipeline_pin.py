@@ -164,6 +164,35 @@ def test_stashing_is_not_a_no_op_here():
     assert a[0][:1] == b[0][:1] and a[0][3:] != b[0][3:]
 
 
+def test_lr_schedule_hook_equals_unsplit_model_with_per_step_lr():
+    """The oracle's learning-rate hook against the unsplit model whose ``param_group['lr']`` is written
+    before every step (main_with_runtime.py:368, 562-563)."""
+    lrs = [0.01 * (1 + i) for i in range(10)]
+    stages = _stages(2)
+    losses, _ = pipeline_oracle.run_pipeline(stages, torch.nn.CrossEntropyLoss(), _make_opt("SGD", SGD_KW),
+                                             _batches(10), warmups=[0, 0], lr_schedule=lambda s, i: lrs[i])
+    ref = _stages(2)
+    model = torch.nn.Sequential(*ref)
+    opt = torch.optim.SGD(model.parameters(), **SGD_KW)
+    crit = torch.nn.CrossEntropyLoss()
+    ref_losses = []
+    for i, (x, y) in enumerate(_batches(10)):
+        loss = crit(model(x), y)
+        for g in opt.param_groups:
+            g["lr"] = lrs[i]
+        opt.zero_grad()
+        loss.backward()
+        opt.step()
+        ref_losses.append(float(loss.detach()))
+    _assert_same((losses, [m.state_dict() for m in stages]), (ref_losses, [m.state_dict() for m in ref]))
+    # with a warm-up depth the first W forwards leave the rate alone: stage 0 applies lrs[i] to its i-th update
+    seen = []
+    stages = _stages(2)
+    pipeline_oracle.run_pipeline(stages, torch.nn.CrossEntropyLoss(), _make_opt("SGD", SGD_KW), _batches(6),
+                                 lr_schedule=lambda s, i: seen.append((s, i)) or lrs[i])
+    assert [i for s, i in seen if s == 0] == list(range(5)) and [i for s, i in seen if s == 1] == list(range(6))
+
+
 def _mutant(old, new):
     src = textwrap.dedent(inspect.getsource(pipeline_oracle.run_pipeline))
     assert src.count(old) == 1, old
