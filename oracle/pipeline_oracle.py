@@ -45,7 +45,8 @@ class StageOracle(object):
         self.bwd_versions = []
 
 
-def run_pipeline(stage_modules, criterion, make_optimizer, batches, warmups=None, on_loss=None, lr_schedule=None):
+def run_pipeline(stage_modules, criterion, make_optimizer, batches, warmups=None, on_loss=None, lr_schedule=None,
+                 observer=None):
     """Run ``len(batches)`` minibatches through the stages with 1F1B + weight stashing.
 
     ``stage_modules``: CPU modules, stage 0 first; ``make_optimizer(stage_index, module,
@@ -53,7 +54,10 @@ def run_pipeline(stage_modules, criterion, make_optimizer, batches, warmups=None
     ``(input, target)``; ``warmups``: warm-up depth per stage (default: straight pipeline,
     S-1-s); ``lr_schedule(stage_index, i)``: learning rate written into every param group after
     the i-th steady-state forward of a stage, as ``adjust_learning_rate`` is called at
-    main_with_runtime.py:368 (warm-up forwards do not touch it).
+    main_with_runtime.py:368 (warm-up forwards do not touch it); ``observer(kind, s, k, **tensors)``
+    is shown every pass without taking part in it: ``("F", x, target, out)`` after a forward pass (``out``
+    is the loss on the last stage) and ``("B", grad_out, grad_in, stage)`` after a backward pass and its
+    update (``grad_out`` None on the last stage, ``grad_in`` None on the first).
     Returns (losses in minibatch order, list of StageOracle)."""
     S = len(stage_modules)
     n = len(batches)
@@ -102,6 +106,8 @@ def run_pipeline(stage_modules, criterion, make_optimizer, batches, warmups=None
                         st.in_flight.append((x, out))
                         fwd_q[s + 1].append(out.detach())
                         tgt_q[s + 1].append(target)
+                    if observer is not None:
+                        observer("F", s, k, x=x, target=target, out=st.in_flight[-1][1])
                     if lr_schedule is not None and k >= min(st.warmup, n):
                         for group in st.optimizer.param_groups:
                             group["lr"] = lr_schedule(s, k - min(st.warmup, n))
@@ -111,14 +117,18 @@ def run_pipeline(stage_modules, criterion, make_optimizer, batches, warmups=None
                     opt.load_old_params()
                     st.bwd_versions.append(opt.current_version if opt.num_versions > 1 else opt.latest_version)
                     x, out = st.in_flight.popleft()
+                    grad_out = None
                     if st.is_last:
                         (out * st.loss_scale).backward()
                     else:
-                        torch.autograd.backward((out,), grad_tensors=(bwd_q[s].popleft(),))
+                        grad_out = bwd_q[s].popleft()
+                        torch.autograd.backward((out,), grad_tensors=(grad_out,))
                     if s > 0:
                         bwd_q[s - 1].append(x.grad)
                     opt.load_new_params()
                     opt.step()
+                    if observer is not None:
+                        observer("B", s, k, grad_out=grad_out, grad_in=x.grad if s > 0 else None, stage=st)
         if not progressed:
             raise RuntimeError("oracle pipeline deadlocked")
     return [losses[k] for k in range(n)], stages

@@ -48,7 +48,7 @@ def make_stages(mask_fn, seed=0):
             models.VggStage3(dropout=0.5, masks=mask_fn)]
 
 
-def run_oracle(dtype=torch.float32):
+def run_oracle(dtype=torch.float32, observer=None):
     masks = dropout_masks()
     count = {"layer13": 0, "layer16": 0}
 
@@ -64,7 +64,8 @@ def run_oracle(dtype=torch.float32):
     try:
         losses, st = pipeline_oracle.run_pipeline(
             stages, torch.nn.CrossEntropyLoss(),
-            lambda s, m, nv: so.StashingOptimizerOracle("SGD", [m], m.parameters(), nv, **SGD_KW), batches)
+            lambda s, m, nv: so.StashingOptimizerOracle("SGD", [m], m.parameters(), nv, **SGD_KW), batches,
+            observer=observer)
     finally:
         pipeline_oracle.LEAF_DTYPES = old
     return losses, stages, st
