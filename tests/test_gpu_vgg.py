@@ -420,3 +420,166 @@ def test_full_size_conv_properties(conv_algorithm):
         dw_w, _ = (ops.set_conv_algorithm("winograd"), ops.conv3x3_weight_grad(x, dy))[1]
         dw_d, _ = (ops.set_conv_algorithm("direct"), ops.conv3x3_weight_grad(x, dy))[1]
         assert float((dw_w - dw_d).abs().max()) <= 1e-5 * float(dw_d.abs().max())
+
+
+# ----------------------------------------------------------------------------------------------------------
+# The front stage at the benchmark's size, layer by layer
+# ----------------------------------------------------------------------------------------------------------
+def _windows(h, w, size=24):
+    """Top-left corner, bottom-right corner and an interior window of an h x w image (even-aligned)."""
+    c = (h // 2 - size // 2) // 2 * 2
+    return [(0, size, 0, size), (h - size, h, w - size, w), (c, c + size, c + 2, c + 2 + size)]
+
+
+def _crop_with_halo(t, n, win, halo):
+    """Image n of the NCHW tensor, window ``win`` grown by ``halo`` pixels, zero-filled outside the image
+    (what the convolution's padding supplies there), fp64 on the CPU."""
+    h0, h1, w0, w1 = win
+    H, W = t.shape[2], t.shape[3]
+    out = torch.zeros(t.shape[1], h1 - h0 + 2 * halo, w1 - w0 + 2 * halo, dtype=torch.float64)
+    a0, a1, b0, b1 = max(h0 - halo, 0), min(h1 + halo, H), max(w0 - halo, 0), min(w1 + halo, W)
+    out[:, a0 - (h0 - halo):a1 - (h0 - halo), b0 - (w0 - halo):b1 - (w0 - halo)] = t[n, :, a0:a1, b0:b1].double().cpu()
+    return out
+
+
+def _weight_grad_fp64(x, dz, chunk=4):
+    """dw[k,c,r,s] = sum over images and pixels of dz[n,k,h,w] * x[n,c,h+r-1,w+s-1], and db[k] = sum dz, as
+    fp64 matrix products over all of the batch (the definition, no convolution routine)."""
+    N, C, H, W = x.shape
+    K = dz.shape[1]
+    dw = torch.zeros(K, C, 3, 3, dtype=torch.float64, device=x.device)
+    db = torch.zeros(K, dtype=torch.float64, device=x.device)
+    for n0 in range(0, N, chunk):
+        xs = torch.nn.functional.pad(x[n0:n0 + chunk].double().permute(0, 2, 3, 1), (0, 0, 1, 1, 1, 1))   # N,H+2,W+2,C
+        g = dz[n0:n0 + chunk].double().permute(0, 2, 3, 1).reshape(-1, K)
+        db += g.sum(0)
+        for r in range(3):
+            for s in range(3):
+                dw[:, :, r, s] += g.t() @ xs[:, r:r + H, s:s + W, :].reshape(-1, C)
+    return dw, db
+
+
+def test_front_stage_full_size_every_layer_against_fp64():
+    """conv1_1 .. pool2 at batch 64, 224x224 -- the kernels and launch shapes of the headline benchmark
+    (Winograd forward with the pooling epilogue, the masked input-gradient launches, the few-channel forward
+    and weight-gradient kernels, pooling backward from index bytes) -- one forward and one backward pass.
+
+    Convolution is local, so windows of the first and the last image (two corners that see the zero padding
+    and an interior one, all channels) of every layer's output and input gradient are compared with fp64
+    ``conv2d`` on the matching crop of that layer's actual operands; the weight and bias gradients of all
+    four layers are compared in full with their definition evaluated in fp64.  Where a ReLU or pooling
+    decision enters, the index bytes the forward kernel wrote are checked against the fp64 pre-activations
+    (every decision whose margin exceeds rounding must agree), and the gradient checks then use the
+    product's decisions, so they are exact statements about linear maps.  rel 1e-5 throughout."""
+    import torch.nn.functional as F
+    from pipedream_amd import ops
+    from pipedream_amd.stages import vgg16
+    torch.manual_seed(0)
+    stage = vgg16.FrontStage().cuda()
+    gen = torch.Generator(device="cuda").manual_seed(1)
+    N = 64
+    x = torch.randn(N, 3, 224, 224, device="cuda", generator=gen).contiguous(memory_format=torch.channels_last)
+    dy = (torch.randn(N, 128, 56, 56, device="cuda", generator=gen) * 1e-3).contiguous(memory_format=torch.channels_last)
+
+    a1 = stage.layer2(x)
+    a2 = stage.layer6(stage.layer4(a1))
+    a3 = stage.layer7(a2)
+    a4 = stage.layer11(stage.layer9(a3))
+    for t in (a1, a2, a3):
+        t.retain_grad()
+    assert a1.shape == (N, 64, 224, 224) and a2.shape == (N, 64, 112, 112) and a4.shape == (N, 128, 56, 56)
+    assert torch.equal(a4, stage(x).detach())            # the stage's own forward is this chain, bit for bit
+    idx4, idx9 = a2.grad_fn.saved_tensors[2], a4.grad_fn.saved_tensors[2]
+    a4.backward(dy)
+    torch.cuda.synchronize()
+
+    tol = 1e-5
+    worst = {}
+
+    def close(what, got, want):
+        got = got.detach()
+        err = float((got.double().cpu() - want).norm() / want.norm())
+        worst[what] = max(worst.get(what, 0.0), err)
+        assert err <= tol, (what, err)
+        assert float((got.double().cpu() - want).abs().max()) <= 10 * tol * float(want.abs().max()), what
+
+    # ---- forward, layer by layer on the layer's actual input ----
+    def forward_layer(name, layer, inp, out, idx):
+        w64, b64 = layer.weight.detach().double().cpu(), layer.bias.detach().double().cpu()
+        H, W = inp.shape[2], inp.shape[3]
+        undecided = total = 0
+        for n in (0, N - 1):
+            for win in _windows(H, W):
+                h0, h1, w0, w1 = win
+                z = F.conv2d(_crop_with_halo(inp, n, win, 1)[None], w64, b64)[0]
+                ref = torch.relu(z)
+                if idx is None:
+                    close(name + " output", out[n, :, h0:h1, w0:w1], ref)
+                    continue
+                pooled, arg = F.max_pool2d(ref[None], 2, 2, return_indices=True)
+                close(name + " pooled output", out[n, :, h0 // 2:h1 // 2, w0 // 2:w1 // 2], pooled[0])
+                # index bytes: bits 0-1 the window position of the maximum, bit 2 "the maximum is positive"
+                got = idx[n, :, h0 // 2:h1 // 2, w0 // 2:w1 // 2].cpu().long()
+                arg = arg[0]
+                pos = (arg // (w1 - w0)) % 2 * 2 + (arg % (w1 - w0)) % 2
+                win4 = z.reshape(z.shape[0], (h1 - h0) // 2, 2, (w1 - w0) // 2, 2).permute(0, 1, 3, 2, 4).reshape(
+                    z.shape[0], (h1 - h0) // 2, (w1 - w0) // 2, 4)
+                top = torch.topk(win4, 2, dim=-1).values
+                margin = 1e-4 * float(z.std())
+                positive = top[..., 0] > 0
+                assert torch.equal((got >> 2)[top[..., 0].abs() > margin] == 1, positive[top[..., 0].abs() > margin])
+                decided = positive & (top[..., 0] - top[..., 1] > margin) & (top[..., 0] > margin)
+                assert torch.equal((got & 3)[decided], pos[decided]), name
+                total += positive.numel()
+                undecided += int((positive & ~decided).sum())
+        assert undecided <= 1e-3 * max(total, 1), (name, undecided, total)
+
+    forward_layer("conv1_1", stage.layer2, x, a1, None)
+    forward_layer("conv1_2", stage.layer4, a1, a2, idx4)
+    forward_layer("conv2_1", stage.layer7, a2, a3, None)
+    forward_layer("conv2_2", stage.layer9, a3, a4, idx9)
+
+    # the fused convolution + pooling kernel against the two kernels it replaces, at full size
+    y_plain, idx_plain = ops.maxpool2x2_idx(ops.conv3x3_forward(a3.detach(), stage.layer9.weight.detach(),
+                                                                stage.layer9.bias.detach(), relu=True))
+    assert torch.equal(y_plain, a4.detach()) and torch.equal(idx_plain, idx9)
+    del y_plain, idx_plain
+
+    # ---- backward: gradient of each layer's pre-activation, with the product's decisions ----
+    dz9 = ops.maxpool2x2_idx_backward(dy, idx9, 112, 112, relu_mask=True)
+    dz7 = a3.grad                     # conv2_2 masked it with conv2_1's ReLU as it stored it (input_rectified)
+    dz4 = ops.maxpool2x2_idx_backward(a2.grad, idx4, 224, 224, relu_mask=True)
+    dz2 = a1.grad
+    # pooling backward moves values, no arithmetic: each gradient lands on the position its byte names
+    for dz, g, idx in ((dz9, dy, idx9), (dz4, a2.grad, idx4)):
+        n_, c_, h_, w_ = dz.shape
+        parts = dz.reshape(n_, c_, h_ // 2, 2, w_ // 2, 2)
+        assert torch.equal(parts.sum(dim=(3, 5)), torch.where((idx & 4) != 0, g, torch.zeros_like(g)))
+        assert int((parts != 0).sum(dim=(3, 5)).max()) <= 1
+        hit = parts.permute(0, 1, 2, 4, 3, 5).reshape(n_, c_, h_ // 2, w_ // 2, 4).gather(-1, (idx & 3).long()[..., None])[..., 0]
+        assert torch.equal(hit, parts.sum(dim=(3, 5)))
+
+    def input_grad(name, layer, dz, got, mask_by):
+        """``got`` (the gradient the layer handed to its producer) against conv_transpose of dz on crops."""
+        w64 = layer.weight.detach().double().cpu()
+        H, W = dz.shape[2], dz.shape[3]
+        for n in (0, N - 1):
+            for win in _windows(H, W):
+                h0, h1, w0, w1 = win
+                # dx = conv2d(dz, w rotated by 180 degrees with in/out channels swapped), padding 1
+                ref = F.conv2d(_crop_with_halo(dz, n, win, 1)[None], w64.flip(2, 3).transpose(0, 1))[0]
+                if mask_by is not None:
+                    ref = ref * (mask_by[n, :, h0:h1, w0:w1] > 0).double().cpu()
+                close(name + " input gradient", got[n, :, h0:h1, w0:w1], ref)
+
+    input_grad("conv2_2", stage.layer9, dz9, a3.grad, a3.detach())
+    # conv2_1 hands its input gradient to pool1, i.e. a2.grad, unmasked (the pooling backward masks it)
+    input_grad("conv2_1", stage.layer7, dz7, a2.grad, None)
+    input_grad("conv1_2", stage.layer4, dz4, a1.grad, a1.detach())
+
+    for name, layer, inp, dz in (("conv2_2", stage.layer9, a3.detach(), dz9), ("conv2_1", stage.layer7, a2.detach(), dz7),
+                                 ("conv1_2", stage.layer4, a1.detach(), dz4), ("conv1_1", stage.layer2, x, dz2)):
+        dw, db = _weight_grad_fp64(inp, dz)
+        close(name + " weight gradient", layer.weight.grad, dw.cpu())
+        close(name + " bias gradient", layer.bias.grad, db.cpu())
+    print("front stage at full size, worst rel-L2 per check:", {k: "%.1e" % v for k, v in worst.items()})
