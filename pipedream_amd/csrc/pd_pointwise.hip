@@ -246,7 +246,8 @@ __device__ __forceinline__ float wave_sum(float v) {
 }
 
 // One block per row: row max and log-sum-exp via wave shuffles + an LDS exchange between
-// the 4 waves.  row_loss[b] = lse - x[target] (0 for ignored rows), lse[b] kept for backward.
+// the 4 waves.  row_loss[b] = lse - x[target] (0 for ignored rows, NaN for a target outside [0, C)),
+// lse[b] kept for backward.
 __global__ __launch_bounds__(PW_THREADS) void xent_fwd_kernel(const float* __restrict__ logits,
                                                               const int64_t* __restrict__ target,
                                                               float* __restrict__ row_loss, float* __restrict__ lse,
@@ -272,7 +273,8 @@ __global__ __launch_bounds__(PW_THREADS) void xent_fwd_kernel(const float* __res
         float l = m + logf(tot);
         lse[b] = l;
         int64_t t = target[b];
-        row_loss[b] = (t == ignore_index) ? 0.f : l - x[t];
+        // a label outside [0, C) that is not the ignore index poisons the loss instead of reading out of bounds
+        row_loss[b] = (t == ignore_index) ? 0.f : ((t >= 0 && t < C) ? l - x[t] : NAN);
     }
 }
 

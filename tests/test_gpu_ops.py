@@ -212,6 +212,27 @@ def test_cross_entropy_vs_torch(B, C):
         assert not d[1].any()
 
 
+@pytest.mark.parametrize("bad", [-1, 10, 1 << 40])
+def test_cross_entropy_target_out_of_range_gives_nan_loss(bad):
+    """A label outside [0, C) that is not the ignore index: the loss is NaN (no read outside the row), the
+    other rows' log-sum-exp values and the backward kernel run as usual."""
+    g = torch.Generator().manual_seed(4)
+    x = torch.randn(6, 10, generator=g)
+    t = torch.randint(0, 10, (6,), generator=g)
+    t[3] = bad
+    loss, (lse, count) = ops.cross_entropy_forward(x.cuda(), t.cuda())
+    assert torch.isnan(loss).item()
+    torch.testing.assert_close(lse.cpu(), torch.logsumexp(x, dim=1), rtol=1e-5, atol=1e-6)
+    d = ops.cross_entropy_backward(x.cuda(), t.cuda(), lse, count, torch.tensor(1.0).cuda())
+    torch.cuda.synchronize()
+    # rows with valid labels get their usual gradient; the bad row gets softmax / count (no one-hot entry)
+    keep = [i for i in range(6) if i != 3]
+    xr = x[keep].clone().requires_grad_(True)
+    (F.cross_entropy(xr, t[keep], reduction="sum") / 6).backward()
+    torch.testing.assert_close(d.cpu()[keep], xr.grad, rtol=1e-5, atol=1e-7)
+    torch.testing.assert_close(d.cpu()[3], torch.softmax(x[3], 0) / 6, rtol=1e-5, atol=1e-7)
+
+
 def test_linear_layer_matches_torch_nn():
     torch.manual_seed(3)
     ref = torch.nn.Linear(37, 21)
