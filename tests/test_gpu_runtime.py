@@ -316,7 +316,7 @@ def test_matched_relu_contract_trains():
     torch.cuda.synchronize()
     loss = torch.nn.functional.cross_entropy(ref[2](ref[1](ref[0](x))).mean(dim=(2, 3)), y)
     loss.backward()
-    assert abs(float(rts[2].loss.detach()) - float(loss)) <= 1e-5 * float(loss)
+    assert abs(float(rts[2].loss.detach()) - float(loss.detach())) <= 1e-5 * float(loss.detach())
     for r, m in zip(rts, ref):
         mod = r.modules()[0]
         mod = mod.body if isinstance(mod, Head) else mod
