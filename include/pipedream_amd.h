@@ -250,6 +250,17 @@ int pd_conv3x3_wgrad_workspace_bytes(int N, int H, int W, int C, int K, uint64_t
 int pd_conv3x3_wgrad_nhwc_f32(const float* x, const float* dy, const float* relu_out, float* dw, float* dbias,
                               void* workspace, uint64_t workspace_bytes,
                               int N, int H, int W, int C, int K, void* stream);
+/* pd_conv3x3_wgrad_nhwc_f32 for callers that cannot allocate device memory (code under HIP graph
+ * capture, tight serving loops, harnesses that forbid hipMalloc); it has no counterpart in the reference.
+ * Same arguments without the workspace, same results bit for bit: the partial sums go to a fixed array
+ * of PD_CONV3X3_WGRAD_NOALLOC_MAX_WORKSPACE bytes in device memory that every GPU the library runs on
+ * holds until the process ends.  The call allocates and frees nothing.  A shape whose
+ * pd_conv3x3_wgrad_workspace_bytes() exceeds that size is refused with PD_ESHAPE (the few-channel first
+ * layer fits at any batch size; 64-channel layers up to about 100k pixels per call).  All calls on one
+ * GPU share the array: calls that overlap on one GPU (different streams or threads) race. */
+#define PD_CONV3X3_WGRAD_NOALLOC_MAX_WORKSPACE (16u << 20)
+int pd_conv3x3_wgrad_noalloc_nhwc_f32(const float* x, const float* dy, const float* relu_out, float* dw,
+                                      float* dbias, int N, int H, int W, int C, int K, void* stream);
 
 /* torch.nn.LSTM cell (gnmt_large/gpus=4/stage0.py:14-19), gate order i,f,g,o.
  * Forward, one time step: gates[B][4H] holds x W_ih^T on entry, to which the n_rec split-k

@@ -87,6 +87,7 @@ SIGNATURES = {
     "pd_conv3x3_winograd_wgrad_workspace_bytes": (_i, [_i, _i, ctypes.POINTER(_u64)], True),
     "pd_conv3x3_winograd_wgrad_nhwc_f32": (_i, [_vp, _vp, _vp, _vp, _vp, _u64, _i, _i, _i, _i, _i, _vp], True),
     "pd_conv3x3_wgrad_nhwc_f32": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _u64, _i, _i, _i, _i, _i, _vp], True),
+    "pd_conv3x3_wgrad_noalloc_nhwc_f32": (_i, [_vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _vp], True),
     "pd_lstm_cell_fwd_f32": (_i, [_vp, _vp, _i, _vp, _vp, _vp, _vp, _vp, _i, _i, _vp], True),
     "pd_lstm_cell_bwd_f32": (_i, [_vp, _vp, _vp, _vp, _vp, _i, _vp, _vp, _i, _i, _i, _vp], True),
     "pd_add_f32": (_i, [_vp, _vp, _vp, _u64, _vp], True),

@@ -27,6 +27,8 @@
 //   tiles, stage dY and the X halo tile in LDS, and write per-block partial sums that a
 //   second kernel reduces in a fixed order (deterministic, no atomics).  The bias
 //   gradient falls out of the same dY tile.
+#include <mutex>
+
 #include "pd_internal.h"
 
 typedef float float4_t __attribute__((ext_vector_type(4)));
@@ -1438,17 +1440,11 @@ extern "C" int pd_conv3x3_wgrad_workspace_bytes(int N, int H, int W, int C, int 
     return PD_OK;
 }
 
-extern "C" int pd_conv3x3_wgrad_nhwc_f32(const float* x, const float* dy, const float* relu_out, float* dw,
-                                         float* dbias, void* workspace, uint64_t workspace_bytes, int N, int H, int W,
-                                         int C, int K, void* stream) {
-    int rc = check_dims("pd_conv3x3_wgrad_nhwc_f32", N, H, W, C, K);
-    if (rc != PD_OK) return rc;
-    PD_REQUIRE(x && dy && dw && workspace, PD_EINVAL, "pd_conv3x3_wgrad_nhwc_f32: NULL pointer");
-    uint64_t need = 0;
-    pd_conv3x3_wgrad_workspace_bytes(N, H, W, C, K, &need);
-    PD_REQUIRE(workspace_bytes >= need, PD_EINVAL, "pd_conv3x3_wgrad_nhwc_f32: workspace too small (%llu < %llu)",
-               (unsigned long long)workspace_bytes, (unsigned long long)need);
-    PD_REQUIRE(pd_aligned(workspace, 16), PD_EINVAL, "pd_conv3x3_wgrad_nhwc_f32: workspace must be 16-byte aligned");
+// The launches behind both weight-gradient entry points; ``workspace`` holds at least
+// pd_conv3x3_wgrad_workspace_bytes() bytes, every one of which the first launch writes before the
+// reduction reads it (nothing has to be cleared).
+static int wgrad_launch(const float* x, const float* dy, const float* relu_out, float* dw, float* dbias,
+                        void* workspace, int N, int H, int W, int C, int K, void* stream) {
     WgradArgs a;
     a.x = x; a.dy = dy; a.mask = relu_out;
     a.N = N; a.H = H; a.W = W; a.C = C; a.K = K;
@@ -1486,4 +1482,63 @@ extern "C" int pd_conv3x3_wgrad_nhwc_f32(const float* x, const float* dy, const 
         PD_CHECK_LAUNCH("pd_conv3x3_wgrad_nhwc_f32(reduce bias)");
     }
     return PD_OK;
+}
+
+extern "C" int pd_conv3x3_wgrad_nhwc_f32(const float* x, const float* dy, const float* relu_out, float* dw,
+                                         float* dbias, void* workspace, uint64_t workspace_bytes, int N, int H, int W,
+                                         int C, int K, void* stream) {
+    int rc = check_dims("pd_conv3x3_wgrad_nhwc_f32", N, H, W, C, K);
+    if (rc != PD_OK) return rc;
+    PD_REQUIRE(x && dy && dw && workspace, PD_EINVAL, "pd_conv3x3_wgrad_nhwc_f32: NULL pointer");
+    uint64_t need = 0;
+    pd_conv3x3_wgrad_workspace_bytes(N, H, W, C, K, &need);
+    PD_REQUIRE(workspace_bytes >= need, PD_EINVAL, "pd_conv3x3_wgrad_nhwc_f32: workspace too small (%llu < %llu)",
+               (unsigned long long)workspace_bytes, (unsigned long long)need);
+    PD_REQUIRE(pd_aligned(workspace, 16), PD_EINVAL, "pd_conv3x3_wgrad_nhwc_f32: workspace must be 16-byte aligned");
+    return wgrad_launch(x, dy, relu_out, dw, dbias, workspace, N, H, W, C, K, stream);
+}
+
+// ---- the same weight gradient for callers that cannot allocate ----------------------------------------
+// The partial sums go to a fixed array in device memory instead of a caller's workspace.  Each GPU the
+// library runs on holds its own copy of the array, at its own address, until the process ends.  In host
+// code the array's name is only a handle for hipGetSymbolAddress; the address it returns for the current
+// device is what kernels and copies get.
+constexpr uint64_t WGRAD_SCRATCH_BYTES = PD_CONV3X3_WGRAD_NOALLOC_MAX_WORKSPACE;
+static __device__ __align__(256) unsigned char scratch[WGRAD_SCRATCH_BYTES];
+
+constexpr int WGRAD_SCRATCH_MAX_DEVICES = 64;
+static std::mutex g_scratch_mutex;
+static void* g_scratch_ptr[WGRAD_SCRATCH_MAX_DEVICES];   // per device, filled on the first call there
+
+static int scratch_of_current_device(const char* who, void** out) {
+    int dev = -1;
+    PD_HIP(hipGetDevice(&dev));
+    PD_REQUIRE(dev >= 0 && dev < WGRAD_SCRATCH_MAX_DEVICES, PD_EINVAL, "%s: device ordinal %d not supported", who, dev);
+    std::lock_guard<std::mutex> lock(g_scratch_mutex);
+    if (!g_scratch_ptr[dev]) {
+        void* p = nullptr;
+        PD_HIP(hipGetSymbolAddress(&p, HIP_SYMBOL(scratch)));
+        PD_REQUIRE(p != nullptr && pd_aligned(p, 256), PD_EINVAL, "%s: no device address for the scratch array", who);
+        g_scratch_ptr[dev] = p;
+    }
+    *out = g_scratch_ptr[dev];
+    return PD_OK;
+}
+
+extern "C" int pd_conv3x3_wgrad_noalloc_nhwc_f32(const float* x, const float* dy, const float* relu_out, float* dw,
+                                                 float* dbias, int N, int H, int W, int C, int K, void* stream) {
+    const char* who = "pd_conv3x3_wgrad_noalloc_nhwc_f32";
+    int rc = check_dims(who, N, H, W, C, K);
+    if (rc != PD_OK) return rc;
+    PD_REQUIRE(x && dy && dw, PD_EINVAL, "%s: NULL pointer", who);
+    uint64_t need = 0;
+    pd_conv3x3_wgrad_workspace_bytes(N, H, W, C, K, &need);
+    PD_REQUIRE(need <= WGRAD_SCRATCH_BYTES, PD_ESHAPE,
+               "%s: this shape needs %llu bytes of partial sums, the built-in scratch array holds %llu; use "
+               "pd_conv3x3_wgrad_nhwc_f32 with a workspace", who, (unsigned long long)need,
+               (unsigned long long)WGRAD_SCRATCH_BYTES);
+    void* ws = nullptr;
+    rc = scratch_of_current_device(who, &ws);
+    if (rc != PD_OK) return rc;
+    return wgrad_launch(x, dy, relu_out, dw, dbias, ws, N, H, W, C, K, stream);
 }
