@@ -13,9 +13,16 @@ MFMA fp32 3x3 convolution by Winograd F(2x2, 3x3) (`winograd_fwd_kernel`, used f
 and input gradient): algorithmic flop of its launches in the timed region (those of the
 direct convolution, 2*9*C*K per output pixel) / their summed duration, both measured with
 HIP events around every launch on the launch stream.  The kernel issues 16/36 of those
-multiplications to the MFMA units; `executed` is the rate it actually executes.
+multiplications to the MFMA units: `roofline.achieved` / `roofline.frac` are the rate it actually
+executes against the MFMA fp32 peak (never above 1), `roofline.direct_equivalent` is the rate a direct
+convolution would need for the same launch time.  `roofline.traffic` is read from the tracked summary of
+the rocprofv3 --pmc runs under profiles/ and is refused if that summary is about another kernel.
 `cpu_baseline` times the CPU oracle (torch.nn on the host cores) on a bounded sample of
 the same workload.
+
+`--workload vgg16_pipeline | gnmt | gnmt_criterion | transformer` print the same kind of line for the
+other configurations (full VGG16 as four co-resident stages; the LSTM stage; the GNMT classifier +
+criterion; the 2BW transformer stage), each with its own CPU baseline sample.
 """
 import argparse
 import json
@@ -30,9 +37,23 @@ BATCH = 64
 STASH_DEPTH = 4
 SGD_KW = dict(lr=0.01, momentum=0.9, weight_decay=5e-4)
 PEAK_FP32_MFMA_TFLOPS = 157.3
-# HBM bytes per launch of the dominant kernel, from the rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE
-# runs summarised under profiles/ (None until measured for the current kernel).
-MEASURED_TRAFFIC_BYTES = 1.126e9
+# HBM bytes per launch of the dominant kernel: written next to the summary of the rocprofv3 --pmc
+# FETCH_SIZE / WRITE_SIZE runs it comes from
+TRAFFIC_SUMMARY = os.path.join(ROOT, "profiles", "winograd_fwd_vgg16_front_stage_bs64_pmc_traffic.json")
+
+
+def measured_traffic(kernel):
+    """HBM bytes per launch of ``kernel`` from the tracked counter summary, None if there is none; a summary
+    that is about another kernel is an error, not a number to print."""
+    if not os.path.isfile(TRAFFIC_SUMMARY):
+        return None
+    with open(TRAFFIC_SUMMARY) as f:
+        rec = json.load(f)
+    if rec["kernel"] != kernel:
+        sys.exit("bench.py: %s holds the HBM traffic of %r, the timed kernel is %r; profile the current kernel "
+                 "again (bench.py --pmc-probe under rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE) or remove the file"
+                 % (TRAFFIC_SUMMARY, rec["kernel"], kernel))
+    return float(rec["traffic_bytes_per_launch"])
 
 
 def build_stage():
@@ -332,8 +353,180 @@ def gnmt_criterion_run(steps, warmup):
                                          "smoothing 0.1, no padding rows, fp32, Adam, 1 weight version")
 
 
+def vgg16_pipeline_run(steps, warmup):
+    """Full VGG16 (13 convolutions + 3 Linear layers) as the reference's four stages co-resident on the GPU,
+    stash depths 4/3/2/1, batch 64 fp32, device-buffer hand-off, SGD momentum 0.9.  The pipeline is filled
+    (3/2/1/0 forwards in flight), then one step = one minibatch through the steady state: every stage runs
+    one forward, one backward and one stashed update, last stage first, so each stage finds its neighbour's
+    gradient of the same minibatch and its producer's activation of the next one already queued."""
+    import torch
+    from pipedream_amd import handoff, runtime, sgd
+    from pipedream_amd.layers import CrossEntropyLoss
+    from pipedream_amd.stages import vgg16
+    handoff.reset_fabrics()
+    torch.manual_seed(0)
+    model = vgg16.model(CrossEntropyLoss(), dropout=0.5)
+    conf = vgg16.conf()
+    shapes = {"input0": (BATCH, 3, 224, 224), "target": (BATCH,)}
+    dtypes = {"input0": torch.float32, "target": torch.int64}
+    stages = []
+    for rank in range(4):
+        r = runtime.StageRuntime(
+            model=model, distributed_backend="gloo", fp16=False, loss_scale=1.0,
+            training_tensor_shapes=shapes, eval_tensor_shapes=dict(shapes), training_tensor_dtypes=dtypes,
+            inputs_module_destinations={"input": 0}, target_tensor_names={"target"},
+            configuration_maps={"module_to_stage_map": conf["module_to_stage_map"],
+                                "stage_to_rank_map": conf["stage_to_rank_map"], "stage_to_depth_map": None},
+            master_addr="127.0.0.1", rank=rank, local_rank=0, num_ranks_in_server=4, verbose_freq=0,
+            model_type=runtime.IMAGE_CLASSIFICATION)
+        opt = sgd.SGDWithWeightStashing(r.modules(), r.master_parameters, r.model_parameters, 1.0,
+                                        num_versions=r.num_warmup_minibatches + 1, **SGD_KW)
+        stages.append((r, opt))
+    g = torch.Generator().manual_seed(0)
+    images = [torch.randn(BATCH, 3, 224, 224, generator=g).cuda().contiguous(memory_format=torch.channels_last)
+              for _ in range(2)]
+    targets = [torch.randint(0, 1000, (BATCH,), generator=g).cuda() for _ in range(2)]
+
+    def loader():
+        i = 0
+        while True:
+            yield images[i % 2], targets[i % 2]
+            i += 1
+
+    total = warmup + steps + 4 + 3
+    for i, (r, _) in enumerate(stages):
+        r.train(total)
+        r.set_loader(loader() if i == 0 else None)
+    for r, _ in stages:                                  # fill: 3 / 2 / 1 / 0 forwards in flight
+        for _ in range(r.num_warmup_minibatches):
+            r.run_forward()
+
+    def step():
+        for r, opt in reversed(stages):
+            assert r.can_run_forward()
+            r.run_forward()
+            opt.zero_grad()
+            opt.load_old_params()
+            assert r.can_run_backward()
+            r.run_backward()
+            opt.load_new_params()
+            opt.step()
+
+    elapsed, stats = _run_steps(step, steps, warmup)
+    done = warmup + steps + min(steps, 4)
+    assert [o.latest_version.version for _, o in stages] == [done] * 4
+    assert stages[0][1].queue.versions() == [done - 3 + i for i in range(4)]
+    return elapsed, stats, BATCH, "f32", ("Full VGG16 as 4 co-resident stages (reference split conv1_1-conv1_2 / ..conv3_1 / "
+                                           "..conv5_1 / rest + 3 FC), batch 64, fp32, stash depths 4/3/2/1, SGD momentum "
+                                           "0.9, steady-state 1F1B, device-buffer hand-off")
+
+
+# ---- CPU baselines of the other configurations: the oracle on a bounded sample ------------------------
+
+def _time_cpu(step, timed, unit_per_step, sample):
+    import torch
+    step()
+    t0 = time.perf_counter()
+    for _ in range(timed):
+        step()
+    sec = (time.perf_counter() - t0) / timed
+    return {"value": unit_per_step / sec, "unit": "samples/s", "cores": torch.get_num_threads(), "kind": "port",
+            "sample": sample % {"timed": timed, "sec": sec}}
+
+
+def cpu_vgg16_pipeline():
+    """The oracle's 4-stage pipeline (torch.nn stages, state_dict-copy stashing, torch.optim.SGD) at batch 8:
+    samples/s of a CPU convolution hardly depend on the batch size, and a batch-64 minibatch is 5.9 TFLOP."""
+    import torch
+    from oracle import models, pipeline_oracle, stash_oracle
+    torch.manual_seed(0)
+    batch, n = 16, 6
+    stages = [models.VggStage0(), models.VggStage1(), models.VggStage2(), models.VggStage3(dropout=0.5)]
+    g = torch.Generator().manual_seed(0)
+    batches = [(torch.randn(batch, 3, 224, 224, generator=g), torch.randint(0, 1000, (batch,), generator=g))
+               for _ in range(n)]
+    t0 = time.perf_counter()
+    pipeline_oracle.run_pipeline(stages, torch.nn.CrossEntropyLoss(),
+                                 lambda s, m, nv: stash_oracle.StashingOptimizerOracle("SGD", [m], m.parameters(), nv, **SGD_KW),
+                                 batches)
+    sec = (time.perf_counter() - t0) / n
+    return {"value": batch / sec, "unit": "samples/s", "cores": torch.get_num_threads(), "kind": "port",
+            "sample": "%d minibatches of batch %d through the 4-stage oracle pipeline incl. fill and drain (%.1f s per "
+                      "minibatch)" % (n, batch, sec)}
+
+
+def cpu_gnmt():
+    import torch
+    from oracle import models, stash_oracle
+    torch.manual_seed(0)
+    m = models.GnmtStage0(dropout=0.0)
+    opt = stash_oracle.StashingOptimizerOracle("Adam", [m], m.parameters(), 3, lr=1e-3, betas=(0.9, 0.999))
+    ids = torch.randint(0, 32320, (50, 128))
+    dy = torch.randn(50, 128, 1024) * 1e-2
+    pend = [m(ids) for _ in range(2)]
+
+    def step():
+        pend.append(m(ids))
+        opt.zero_grad()
+        opt.load_old_params()
+        pend.pop(0).backward(dy)
+        opt.load_new_params()
+        opt.step()
+
+    return _time_cpu(step, 6, 128, "%(timed)d steady-state steps at seq 50 x batch 128 after 1 warm-up step (%(sec).1f s/step)")
+
+
+def cpu_gnmt_criterion():
+    import torch
+    from oracle import seq2seq_oracle, stash_oracle
+    torch.manual_seed(0)
+    m = torch.nn.Linear(1024, 32320)
+    opt = stash_oracle.StashingOptimizerOracle("Adam", [m], m.parameters(), 1, lr=1e-3, betas=(0.9, 0.999))
+    x = torch.randn(50, 128, 1024, requires_grad=True)
+    tgt = torch.randint(1, 32320, (50 * 128,))
+
+    def step():
+        loss = seq2seq_oracle.label_smoothing(m(x), tgt, 0, 0.1)
+        opt.zero_grad()
+        opt.load_old_params()
+        x.grad = None
+        loss.backward()
+        opt.load_new_params()
+        opt.step()
+
+    return _time_cpu(step, 3, 128, "%(timed)d steps on seq 50 x batch 128 after 1 warm-up step (%(sec).1f s/step)")
+
+
+def cpu_transformer():
+    import torch
+    from oracle import models, stash_oracle
+    torch.manual_seed(0)
+    m = models.TransformerStage0()
+    opt = stash_oracle.StashingOptimizerOracle("Adam", [m], m.parameters(), 2, update_interval=4, lr=1e-3,
+                                               betas=(0.9, 0.999))
+    x = torch.randn(8, 512, 1024)
+    dy = (torch.randn(8, 512, 1024) * 0.05).bfloat16()
+    pend = [m(x)]
+
+    def step():
+        pend.append(m(x))
+        opt.zero_grad()
+        opt.load_old_params()
+        pend.pop(0).backward(dy)
+        opt.load_new_params()
+        opt.step()
+
+    return _time_cpu(step, 7, 8, "%(timed)d micro-batches of 8 x 512 tokens (two Adam updates among them) after 1 warm-up "
+                                 "micro-batch (%(sec).1f s each), torch's bf16 CPU kernels")
+
+
+CPU_BASELINES = {"vgg16_pipeline": cpu_vgg16_pipeline, "gnmt": cpu_gnmt, "gnmt_criterion": cpu_gnmt_criterion,
+                 "transformer": cpu_transformer}
+
+
 def secondary(args):
-    run, kernel, peak, bound = {"gnmt": (gnmt_run, "gemm_f32", PEAK_FP32_MFMA_TFLOPS, "mfma"),
+    run, kernel, peak, bound = {"vgg16_pipeline": (vgg16_pipeline_run, "conv3x3_winograd_kernel", PEAK_FP32_MFMA_TFLOPS, "mfma"),
+                                "gnmt": (gnmt_run, "gemm_f32", PEAK_FP32_MFMA_TFLOPS, "mfma"),
                                 "gnmt_criterion": (gnmt_criterion_run, "label_smoothing_bwd", 8000.0, "hbm"),
                                 "transformer": (transformer_run, "gemm_bf16", 2500.0, "mfma")}[args.workload]
     elapsed, stats, batch, dtype, desc = run(args.steps, args.warmup)
@@ -343,6 +536,11 @@ def secondary(args):
         for name in ("label_smoothing_fwd", "label_smoothing_bwd"):
             stats[name]["GB/s"] = round(stats[name].pop("TFLOP/s") * 1e3, 1)
         k["TFLOP/s"] = stats[kernel]["GB/s"]
+    extra = {}
+    if kernel == "conv3x3_winograd_kernel":
+        # the Winograd kernel executes 16/36 of the direct convolution's multiplications
+        extra = {"direct_equivalent": k["TFLOP/s"]}
+        k["TFLOP/s"] = k["TFLOP/s"] * 16.0 / 36.0
     out = {
         "metric": "samples/sec per stage (fwd+bwd+stashed update)", "value": batch * args.steps / elapsed,
         "unit": "samples/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
@@ -352,9 +550,11 @@ def secondary(args):
         "roofline": {"bound": bound, "achieved": k["TFLOP/s"], "peak": peak,
                      "unit": "GB/s" if bound == "hbm" else "TFLOP/s",
                      "frac": k["TFLOP/s"] / peak, "traffic": None, "kernel": kernel, "launches": k["launches"],
-                     "avg_us": k["avg_us"]},
+                     "avg_us": k["avg_us"], **extra},
         "kernels": stats,
     }
+    if not args.no_cpu_baseline:
+        out["cpu_baseline"] = CPU_BASELINES[args.workload]()
     print(json.dumps(out))
 
 
@@ -364,10 +564,10 @@ def main():
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--no-cpu-baseline", action="store_true")
-    ap.add_argument("--workload", default="vgg16_front", choices=["vgg16_front", "gnmt", "gnmt_criterion", "transformer"],
+    ap.add_argument("--workload", default="vgg16_front", choices=["vgg16_front", "vgg16_pipeline", "gnmt", "gnmt_criterion", "transformer"],
                     help="vgg16_front (default) is the headline configuration; the others print the same kind of "
-                         "line for the LSTM stage, the GNMT classifier + criterion and the transformer stage "
-                         "(no CPU baseline)")
+                         "line for the full VGG16 as four co-resident stages, the LSTM stage, the GNMT classifier + "
+                         "criterion and the transformer stage")
     ap.add_argument("--pmc-probe", action="store_true",
                     help="run the counter-calibration copy and two benchmark steps, print no JSON")
     ap.add_argument("--traffic-bytes", type=float, default=None,
@@ -389,7 +589,11 @@ def main():
     elapsed, stats, _ = gpu_run(args.steps, args.warmup)
     wino = "conv3x3_winograd_kernel" in stats
     conv = stats["conv3x3_winograd_kernel" if wino else "conv3x3_fwd_kernel"]
-    achieved = conv["rate"] / 1e12
+    kernel = "winograd_fwd_kernel" if wino else "conv3x3_fwd_kernel"
+    direct = conv["rate"] / 1e12
+    # what the MFMA units execute: 16 multiplies per 2x2 outputs and channel pair instead of 36
+    executed = direct * (16.0 / 36.0 if wino else 1.0)
+    traffic = args.traffic_bytes if args.traffic_bytes is not None else measured_traffic(kernel)
     out = {
         "metric": "samples/sec per stage (fwd+bwd+stashed update), VGG16 bs64; optimizer HBM GB/s",
         "value": BATCH * args.steps / elapsed,
@@ -406,16 +610,15 @@ def main():
         "config": {"workload": "VGG16 stage 0 (conv1_1..pool2), batch 64, fp32, stash depth 4, SGD momentum 0.9, "
                                "1F1B with 4 minibatches in flight",
                    "global_batch": BATCH, "parallelism": "1 stage on 1 GPU"},
-        "roofline": {"bound": "mfma", "achieved": achieved, "peak": PEAK_FP32_MFMA_TFLOPS, "unit": "TFLOP/s",
-                     "frac": achieved / PEAK_FP32_MFMA_TFLOPS,
-                     "traffic": args.traffic_bytes if args.traffic_bytes is not None else MEASURED_TRAFFIC_BYTES,
-                     "kernel": ("winograd_fwd_kernel (F(2x2,3x3); forward + input gradient)" if wino
-                                else "conv3x3_fwd_kernel<.,.,16> (forward + input gradient)"),
+        "roofline": {"bound": "mfma", "achieved": executed, "peak": PEAK_FP32_MFMA_TFLOPS, "unit": "TFLOP/s",
+                     "frac": executed / PEAK_FP32_MFMA_TFLOPS, "traffic": traffic,
+                     "kernel": kernel + (" (F(2x2,3x3); forward + input gradient)" if wino
+                                         else "<.,.,16> (forward + input gradient)"),
                      "launches": conv["launches"], "avg_us": conv["avg_us"],
-                     "flop_per_launch": conv["work_per_launch"],
-                     # what the MFMA units execute: 16 multiplies per 2x2 outputs instead of 36
-                     "executed": achieved * (16.0 / 36.0 if wino else 1.0),
-                     "executed_frac": achieved * (16.0 / 36.0 if wino else 1.0) / PEAK_FP32_MFMA_TFLOPS},
+                     "flop_per_launch": conv["work_per_launch"] * (16.0 / 36.0 if wino else 1.0),
+                     "direct_flop_per_launch": conv["work_per_launch"],
+                     # the rate a direct convolution (2*9*C*K flop per output pixel) would need for this time
+                     "direct_equivalent": direct},
         "kernels": {k: {"launches": v["launches"], "avg_us": round(v["avg_us"], 1),
                         "TFLOP/s": round(v["rate"] / 1e12, 2)} for k, v in stats.items()},
         "optimizer_hbm": optimizer_bandwidth(),
