@@ -178,36 +178,45 @@ def pmc_probe():
     torch.cuda.synchronize()
     del src, dst
     gpu_run(steps=2, warmup=1)
-    # and the fused stash + SGD kernel on the VGG16-sized parameter set of `optimizer_hbm`
-    optimizer_bandwidth()
+    # and the fused stash + SGD kernel on the VGG16 parameter set of `optimizer_hbm`
+    optimizer_bandwidth("SGD")
     print("pmc probe done")
 
 
-def optimizer_bandwidth():
-    """Fused stash+SGD step on a VGG16-sized flat parameter set (138 357 544 fp32 values,
-    20 algorithmic bytes each), timed with HIP events on the launch stream."""
+def optimizer_bandwidth(kind="SGD"):
+    """The fused stash + optimizer step as the product runs it: SGDWithWeightStashing (or the Adam wrapper)
+    over the parameters of all four VGG16 stages (138 357 544 fp32 values in 32 tensors) with two weight
+    versions, so every step reads the live ring slot and writes the other one.  20 (SGD) / 28 (Adam)
+    algorithmic bytes per parameter; timed with HIP events on the launch stream over 20 steps."""
     import torch
-    from pipedream_amd import _cabi
-    n = 138357544
-    t = [torch.randn(n, device="cuda") for _ in range(3)]
-    out = torch.empty(n, device="cuda")
-    d = (_cabi.TensorDesc * 1)()
-    d[0].grad, d[0].p_in, d[0].p_out = t[0].data_ptr(), t[1].data_ptr(), out.data_ptr()
-    d[0].state0, d[0].state1, d[0].bf16_out, d[0].n = t[2].data_ptr(), None, None, n
-    lib, s = _cabi.lib(), _cabi.stream_ptr()
-    run = lambda: lib.pd_sgd_step(d, 1, 0.01, 0.9, 0.0, 5e-4, 0, 0, 1.0, 1.0, s)
+    from pipedream_amd import adam, sgd
+    from pipedream_amd.layers import CrossEntropyLoss
+    from pipedream_amd.stages import vgg16
+    torch.manual_seed(0)
+    mods = [m.cuda() for m, _, _ in vgg16.model(CrossEntropyLoss())[:4]]
+    params = [p for m in mods for p in m.parameters()]
+    n = sum(p.numel() for p in params)
+    if kind == "SGD":
+        opt, bpp = sgd.SGDWithWeightStashing(mods, params, None, 1.0, 2, **SGD_KW), 20
+    else:
+        opt, bpp = adam.AdamWithWeightStashing(mods, params, None, 1.0, 2, lr=1e-3, betas=(0.9, 0.999)), 28
+    for p in params:
+        p.grad = torch.randn_like(p)
     for _ in range(3):
-        run()
+        opt.step()
     e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
     reps = 20
+    torch.cuda.synchronize()
     e0.record()
     for _ in range(reps):
-        run()
+        opt.step()
     e1.record()
     torch.cuda.synchronize()
     sec = e0.elapsed_time(e1) * 1e-3 / reps
-    return {"kernel": "pd_optim_kernel<SGD>", "params": n, "bytes_per_param": 20, "avg_us": sec * 1e6,
-            "achieved_GBps": 20.0 * n / sec / 1e9, "peak_GBps": 8000.0, "frac": 20.0 * n / sec / 1e9 / 8000.0}
+    assert opt.latest_version.version == reps + 3
+    return {"kernel": "pd_optim_kernel<%s>" % kind, "params": n, "tensors": len(params), "bytes_per_param": bpp,
+            "avg_us": sec * 1e6, "achieved_GBps": bpp * n / sec / 1e9, "peak_GBps": 8000.0,
+            "frac": bpp * n / sec / 1e9 / 8000.0}
 
 
 def cpu_baseline(timed_steps=6):
@@ -621,7 +630,8 @@ def main():
                      "direct_equivalent": direct},
         "kernels": {k: {"launches": v["launches"], "avg_us": round(v["avg_us"], 1),
                         "TFLOP/s": round(v["rate"] / 1e12, 2)} for k, v in stats.items()},
-        "optimizer_hbm": optimizer_bandwidth(),
+        "optimizer_hbm": optimizer_bandwidth("SGD"),
+        "optimizer_hbm_adam": optimizer_bandwidth("Adam"),
     }
     if not args.no_cpu_baseline:
         out["cpu_baseline"] = cpu_baseline()

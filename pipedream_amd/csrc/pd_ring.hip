@@ -104,7 +104,7 @@ extern "C" int pd_ring_push(pd_ring* ring, int64_t version, int* slot) {
 typedef float float4_t __attribute__((ext_vector_type(4)));
 
 constexpr int COPY_THREADS = 256;
-constexpr int COPY_UNROLL = 8;
+constexpr int COPY_UNROLL = 1;   // 4 KiB per block: 6.6 TB/s on a 553 MB copy; 32 KiB per block reached 4.5
 
 __global__ __launch_bounds__(COPY_THREADS) void pd_copy_kernel(float4_t* __restrict__ dst,
                                                                const float4_t* __restrict__ src,

@@ -17,7 +17,7 @@ import ctypes
 import torch
 
 from . import _cabi
-from .arena import WeightArena
+from .arena import WeightArena, staggered_empty
 
 
 class _FusedOptimizer(torch.optim.Optimizer):
@@ -39,7 +39,11 @@ class _FusedOptimizer(torch.optim.Optimizer):
         n = arena.master_bytes // 4
         device = arena.buffer.device
         # flat state buffers share the slot layout of the master section
-        self._flat_state = [torch.zeros(n, dtype=torch.float32, device=device) for _ in self._state_names]
+        # (start addresses staggered against the ring's slots, see arena.staggered_empty)
+        self._flat_state = []
+        for i, _ in enumerate(self._state_names):
+            buf = staggered_empty(4 * n, device, 2 + i)[1].view(torch.float32)
+            self._flat_state.append(buf.zero_())
         self._descs = (_cabi.TensorDesc * max(1, len(masters)))()
         self.bf16_copy = arena.bf16_image  # per-slot flat bf16 images of the master section, or None
 
