@@ -362,14 +362,16 @@ def gnmt_criterion_run(steps, warmup):
                                          "smoothing 0.1, no padding rows, fp32, Adam, 1 weight version")
 
 
-def vgg16_pipeline_run(steps, warmup):
+def vgg16_pipeline_run(steps, warmup, stage_streams=True):
     """Full VGG16 (13 convolutions + 3 Linear layers) as the reference's four stages co-resident on the GPU,
     stash depths 4/3/2/1, batch 64 fp32, device-buffer hand-off, SGD momentum 0.9.  The pipeline is filled
     (3/2/1/0 forwards in flight), then one step = one minibatch through the steady state: every stage runs
     one forward, one backward and one stashed update, last stage first, so each stage finds its neighbour's
-    gradient of the same minibatch and its producer's activation of the next one already queued."""
+    gradient of the same minibatch and its producer's activation of the next one already queued.  Each stage
+    launches on a stream of its own (the hand-off orders them with events), so kernels of different stages
+    can share the GPU."""
     import torch
-    from pipedream_amd import handoff, runtime, sgd
+    from pipedream_amd import handoff, runtime, schedule, sgd
     from pipedream_amd.layers import CrossEntropyLoss
     from pipedream_amd.stages import vgg16
     handoff.reset_fabrics()
@@ -406,20 +408,24 @@ def vgg16_pipeline_run(steps, warmup):
     for i, (r, _) in enumerate(stages):
         r.train(total)
         r.set_loader(loader() if i == 0 else None)
-    for r, _ in stages:                                  # fill: 3 / 2 / 1 / 0 forwards in flight
-        for _ in range(r.num_warmup_minibatches):
-            r.run_forward()
+    streams = schedule.stage_streams(4) if stage_streams else [torch.cuda.current_stream()] * 4
+    torch.cuda.synchronize()
+    for (r, _), stream in zip(stages, streams):          # fill: 3 / 2 / 1 / 0 forwards in flight
+        with torch.cuda.stream(stream):
+            for _ in range(r.num_warmup_minibatches):
+                r.run_forward()
 
     def step():
-        for r, opt in reversed(stages):
-            assert r.can_run_forward()
-            r.run_forward()
-            opt.zero_grad()
-            opt.load_old_params()
-            assert r.can_run_backward()
-            r.run_backward()
-            opt.load_new_params()
-            opt.step()
+        for (r, opt), stream in zip(reversed(stages), reversed(streams)):
+            with torch.cuda.stream(stream):
+                assert r.can_run_forward()
+                r.run_forward()
+                opt.zero_grad()
+                opt.load_old_params()
+                assert r.can_run_backward()
+                r.run_backward()
+                opt.load_new_params()
+                opt.step()
 
     elapsed, stats = _run_steps(step, steps, warmup)
     done = warmup + steps + min(steps, 4)
@@ -538,7 +544,11 @@ def secondary(args):
                                 "gnmt": (gnmt_run, "gemm_f32", PEAK_FP32_MFMA_TFLOPS, "mfma"),
                                 "gnmt_criterion": (gnmt_criterion_run, "label_smoothing_bwd", 8000.0, "hbm"),
                                 "transformer": (transformer_run, "gemm_bf16", 2500.0, "mfma")}[args.workload]
-    elapsed, stats, batch, dtype, desc = run(args.steps, args.warmup)
+    if args.workload == "vgg16_pipeline":
+        elapsed, stats, batch, dtype, desc = run(args.steps, args.warmup, stage_streams=not args.single_stream)
+        desc += ", one stream for all stages" if args.single_stream else ", one stream per stage"
+    else:
+        elapsed, stats, batch, dtype, desc = run(args.steps, args.warmup)
     k = dict(stats[kernel])
     if bound == "hbm":
         # the byte-moving kernels record algorithmic bytes as their work: the rate is in TB/s
@@ -577,6 +587,8 @@ def main():
                     help="vgg16_front (default) is the headline configuration; the others print the same kind of "
                          "line for the full VGG16 as four co-resident stages, the LSTM stage, the GNMT classifier + "
                          "criterion and the transformer stage")
+    ap.add_argument("--single-stream", action="store_true",
+                    help="vgg16_pipeline: launch all four stages on one stream instead of one stream per stage")
     ap.add_argument("--pmc-probe", action="store_true",
                     help="run the counter-calibration copy and two benchmark steps, print no JSON")
     ap.add_argument("--traffic-bytes", type=float, default=None,

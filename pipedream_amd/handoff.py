@@ -17,8 +17,11 @@ Added to it: every parcel carries the minibatch number it belongs to (the receiv
 takes them in order) and a ``premasked`` flag, the producer's statement about who applies the backward
 pass of the ReLU that ends the producing stage (see ``StageRuntime``).
 
-All stages launch on torch's current stream, so queue order is execution order and no events are
-needed.
+Stages may run on streams of their own (``schedule.stage_train_loop(..., stream=...)``): whoever queues a
+parcel records an event on the stream it is working on, whoever takes it makes its own stream wait for
+that event (and tells the caching allocator that the tensor is now in use there), so a consumer's kernels
+never start before the producer's have finished, whatever order the host issued them in.  On a single
+stream the wait is a no-op.
 """
 import collections
 
@@ -26,7 +29,7 @@ import torch
 
 ACK = "ack"
 
-Parcel = collections.namedtuple("Parcel", "tensor seq premasked")
+Parcel = collections.namedtuple("Parcel", "tensor seq premasked ready")
 
 
 class HandoffContractError(RuntimeError):
@@ -53,10 +56,20 @@ class HandoffFabric(object):
         """Queue ``tensor`` for ``receiver_rank``; also the way a test or a benchmark plays a neighbour
         stage that is not there."""
         self.bytes_sent += tensor.element_size() * tensor.nelement()
-        self.queue(tensor_name, receiver_rank, backward).append(Parcel(tensor.detach(), seq, bool(premasked)))
+        ready = None
+        if tensor.is_cuda:
+            ready = torch.cuda.Event()
+            ready.record()            # on the producer's current stream, behind the kernels that wrote the tensor
+        self.queue(tensor_name, receiver_rank, backward).append(Parcel(tensor.detach(), seq, bool(premasked), ready))
 
     def take(self, tensor_name, receiver_rank, backward):
-        return self.queue(tensor_name, receiver_rank, backward).popleft()
+        """The oldest parcel queued for ``receiver_rank``, safe to use on the caller's current stream."""
+        parcel = self.queue(tensor_name, receiver_rank, backward).popleft()
+        if parcel.ready is not None:
+            stream = torch.cuda.current_stream()
+            stream.wait_event(parcel.ready)
+            parcel.tensor.record_stream(stream)
+        return parcel
 
 
 _FABRICS = {}
@@ -110,7 +123,7 @@ class DeviceHandoff(object):
             raise RuntimeError(
                 "stage rank %s: nothing queued for %r (%s); the schedule ran this stage before its "
                 "neighbour produced the tensor" % (self.rank, tensor_name, "backward" if backward else "forward"))
-        parcel = q.popleft()
+        parcel = self.fabric.take(tensor_name, self.rank, backward)
         if parcel.seq is not None and parcel.seq != seq:
             raise RuntimeError("stage rank %s: %r of minibatch %s arrived where minibatch %s was due"
                                % (self.rank, tensor_name, parcel.seq, seq))

@@ -9,16 +9,36 @@ stage is its own process and simply blocks in a receive queue; here the loop is 
 generator that yields whenever its next receive would find the queue empty, and
 ``run_pipeline`` round-robins the generators until all are finished.  ``stage_eval_loop`` is the
 forward-only counterpart (``validate()``, main_with_runtime.py:429-487) with the ``ack`` clock.
+
+Each loop can be given a stream of its own (``stream=``, or ``stage_streams(n)`` for one per stage):
+everything the stage launches -- forward, backward, the stashed update -- then goes to that stream, the
+hand-off layer orders the stages with events, and the HBM-bound kernels of one stage (pooling backward,
+the optimizer, split-k reductions) can run beside the MFMA-bound kernels of another.  All streams have the
+default priority.
 """
+import contextlib
+
+import torch
+
+
+def stage_streams(num_stages):
+    """One stream per co-resident stage (default priority)."""
+    return [torch.cuda.Stream() for _ in range(num_stages)]
+
+
+def _on(stream):
+    return torch.cuda.stream(stream) if stream is not None else contextlib.nullcontext()
 
 
 def stage_train_loop(r, optimizer, num_minibatches, loader=None, lr_schedule=None, on_forward=None,
-                     no_input_pipelining=False):
+                     no_input_pipelining=False, stream=None):
     """Generator running one stage's 1F1B schedule.
 
     ``lr_schedule(step) -> lr`` is written into every param group each iteration, as
     ``adjust_learning_rate`` does (main_with_runtime.py:562-563).  ``on_forward(i, r)`` is
-    called after each steady-state forward (where the reference reads ``r.loss``)."""
+    called after each steady-state forward (where the reference reads ``r.loss``).  ``stream``: the
+    stream this stage's kernels are launched on (default: torch's current stream); it is made current
+    only around the stage's own calls, never across a ``yield``."""
     n = num_minibatches
     r.train(n)
     r.set_loader(loader if (r.stage is None or r.stage == 0) else None)
@@ -27,16 +47,18 @@ def stage_train_loop(r, optimizer, num_minibatches, loader=None, lr_schedule=Non
     def forward():
         while not r.can_run_forward():
             yield r
-        r.run_forward()
+        with _on(stream):
+            r.run_forward()
 
     def backward_and_update():
-        optimizer.zero_grad()
-        optimizer.load_old_params()
         while not r.can_run_backward():
             yield r
-        r.run_backward()
-        optimizer.load_new_params()
-        optimizer.step()
+        with _on(stream):
+            optimizer.zero_grad()
+            optimizer.load_old_params()
+            r.run_backward()
+            optimizer.load_new_params()
+            optimizer.step()
 
     for _ in range(warmup):
         for blocked in forward():
@@ -49,7 +71,8 @@ def stage_train_loop(r, optimizer, num_minibatches, loader=None, lr_schedule=Non
             for param_group in optimizer.param_groups:
                 param_group['lr'] = lr
         if on_forward is not None:
-            on_forward(i, r)
+            with _on(stream):
+                on_forward(i, r)
         for blocked in backward_and_update():
             yield blocked
     for _ in range(warmup):
@@ -58,7 +81,7 @@ def stage_train_loop(r, optimizer, num_minibatches, loader=None, lr_schedule=Non
     r.wait()
 
 
-def stage_eval_loop(r, num_minibatches, loader=None, on_forward=None, no_input_pipelining=False):
+def stage_eval_loop(r, num_minibatches, loader=None, on_forward=None, no_input_pipelining=False, stream=None):
     """Generator running one stage's forward-only schedule, the body of ``validate()`` in the
     reference's caller (runtime/image_classification/main_with_runtime.py:429-487): ``W`` warm-up
     forwards, then ``n - W`` times [forward, ack].  The ack is the clock: a stage takes its next
@@ -72,14 +95,17 @@ def stage_eval_loop(r, num_minibatches, loader=None, on_forward=None, no_input_p
     for i in range(n):
         while not r.can_run_forward():
             yield r
-        r.run_forward()
+        with _on(stream):
+            r.run_forward()
         if i < warmup:
             continue
         if on_forward is not None:
-            on_forward(i - warmup, r)
+            with _on(stream):
+                on_forward(i - warmup, r)
         while not r.can_run_ack():
             yield r
-        r.run_ack()
+        with _on(stream):
+            r.run_ack()
     r.wait()
 
 

@@ -166,9 +166,12 @@ def test_full_vgg16_four_stage_pipeline_matches_oracle(vgg_oracle):
 
     batches = nf.make_batches()
     losses = []
+    # every stage on a stream of its own, ordered by the hand-off's events
+    streams = schedule.stage_streams(4)
+    torch.cuda.synchronize()
     loops = [schedule.stage_train_loop(
         r, o, n, loader=batches if i == 0 else None,
-        on_forward=(lambda k, rr: losses.append(float(rr.loss.detach()))) if i == 3 else None)
+        on_forward=(lambda k, rr: losses.append(float(rr.loss.detach()))) if i == 3 else None, stream=streams[i])
         for i, (r, o) in enumerate(stages)]
     schedule.run_pipeline(loops)
     torch.cuda.synchronize()
@@ -497,7 +500,7 @@ def test_front_stage_full_size_every_layer_against_fp64():
     worst = {}
 
     def close(what, got, want):
-        got = got.detach()
+        got, want = got.detach(), want.detach()
         err = float((got.double().cpu() - want).norm() / want.norm())
         worst[what] = max(worst.get(what, 0.0), err)
         assert err <= tol, (what, err)

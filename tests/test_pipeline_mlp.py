@@ -66,11 +66,13 @@ def _build_product(num_minibatches=20):
     return stages
 
 
-def _run_product(n):
+def _run_product(n, per_stage_streams=False):
     """n minibatches through the two co-resident stages.  Returns losses, the version every
     forward/backward ran on, the final state_dicts and the ReLU masks of every forward."""
     from pipedream_amd import schedule
     stages = _build_product()
+    streams = schedule.stage_streams(len(stages)) if per_stage_streams else [None] * len(stages)
+    torch.cuda.synchronize()
     assert [r.num_warmup_minibatches for r, _ in stages] == [1, 0]
     assert [o.num_versions for _, o in stages] == [2, 1]
     batches = gold.make_batches()[:n]
@@ -95,7 +97,8 @@ def _run_product(n):
         r.run_forward, r.run_backward = fwd, bwd
         loops.append(schedule.stage_train_loop(
             r, opt, n, loader=batches if si == 0 else None,
-            on_forward=(lambda i, rr: losses.append(float(rr.loss.detach()))) if si == 1 else None))
+            on_forward=(lambda i, rr: losses.append(float(rr.loss.detach()))) if si == 1 else None,
+            stream=streams[si]))
     schedule.run_pipeline(loops)
     torch.cuda.synchronize()
     params = [{k: v.detach().cpu() for k, v in r.modules()[0].state_dict().items()} for r, _ in stages]
@@ -158,6 +161,20 @@ def test_product_matches_golden_and_oracle():
         for k, v in params[si].items():
             gv = GOLDEN["params"]["stage%d.%s" % (si, k)]
             assert abs(float(v.double().abs().sum()) - gv["abs_sum"]) <= 1e-4 * gv["abs_sum"] + 1e-6
+
+
+@pytest.mark.gpu
+def test_one_stream_per_stage_gives_the_same_bits():
+    """Each stage launching on a stream of its own, ordered by the hand-off's events: the same kernels on the
+    same operands in an order that respects every dependency, so losses, versions, masks and parameters
+    are identical, bit for bit, to the single-stream run."""
+    n = 12
+    one = _run_product(n)
+    many = _run_product(n, per_stage_streams=True)
+    assert one[0] == many[0] and one[1] == many[1]
+    for a, b in zip(one[2], many[2]):
+        assert a.keys() == b.keys() and all(torch.equal(a[k], b[k]) for k in a)
+    assert all(torch.equal(a, b) for a, b in zip(one[3], many[3]))
 
 
 @pytest.mark.gpu
