@@ -261,6 +261,18 @@ class WeightArena(object):
         self._lib.pd_copy(ctypes.c_void_p(self.slot_ptr(dst_slot)), ctypes.c_void_p(self.slot_ptr(src_slot)),
                           self.master_bytes, _cabi.stream_ptr(stream))
 
+    def refresh_bf16_image(self, slot=None):
+        """Re-cast the bf16 image of ``slot`` (default: the loaded one) from its fp32 masters.  The fused
+        optimizer step keeps the image current by itself; this is for the writes that bypass it (a foreign
+        ``state_dict`` copied into the parameters, ``get_params(clone=False)``, an in-place edit by the
+        caller)."""
+        if self.bf16_image is None:
+            return
+        slot = self.live_slot if slot is None else slot
+        self._lib.pd_cast_f32_to_bf16(ctypes.c_void_p(self.slot_ptr(slot)),
+                                      ctypes.c_void_p(self.bf16_image[slot].data_ptr()), self.master_bytes // 4,
+                                      _cabi.stream_ptr())
+
     def master_view(self, master_index, slot):
         return self.entries[master_index].views[slot]
 

@@ -164,6 +164,7 @@ class OptimizerWithWeightStashing(torch.optim.Optimizer):
             # live values -> storage of the oldest entry
             dst = self.arena.write_slot()
             self.arena.copy_masters(self.arena.live_slot, dst)
+            self.arena.refresh_bf16_image(dst)
             self.arena.store_others(dst)
             state_dicts = self.arena.state_dicts(dst)
         return state_dicts, self.latest_version
@@ -182,6 +183,8 @@ class OptimizerWithWeightStashing(torch.optim.Optimizer):
                         if "running_" in key or "mask" in key:
                             continue
                         cur[key].copy_(state_dict[key])
+            # the copy went into the loaded slot's fp32 masters; bf16-compute layers read its bf16 image
+            self.arena.refresh_bf16_image()
         self.current_version = version
 
     def load_old_params(self):

@@ -170,3 +170,28 @@ def test_unknown_optimizer_and_fp16_lists_fail_loudly():
         optimizer.OptimizerWithWeightStashing("RMSprop", [model], model.parameters(), None, 1.0, 2, lr=0.1)
     with pytest.raises(NotImplementedError):
         sgd.SGDWithWeightStashing([model], model.parameters(), list(model.parameters()), 1.0, 2, lr=0.1)
+
+
+def test_bf16_image_follows_writes_that_bypass_the_fused_step():
+    """With ``bf16_image=True`` every weight version has a bf16 copy that bf16-compute layers multiply with.
+    The fused step writes it; a foreign ``state_dict`` handed to ``set_params`` and ``get_params(clone=False)``
+    write fp32 masters without it and must re-cast the image of the slot they touched."""
+    import collections
+    from pipedream_amd import adam, ops
+    torch.manual_seed(0)
+    m = torch.nn.Linear(24, 16).cuda()
+    opt = adam.AdamWithWeightStashing([m], list(m.parameters()), None, 1.0, 2, bf16_image=True, lr=1e-2)
+    image = lambda p: ops.bf16_weight(p).float()
+    assert torch.equal(image(m.weight), m.weight.detach().bfloat16().float())
+    # a foreign state_dict (fresh tensors, not views of a ring slot)
+    foreign = collections.OrderedDict((k, torch.randn_like(v)) for k, v in m.state_dict().items())
+    opt.set_params([foreign], opt.latest_version)
+    torch.testing.assert_close(m.weight.detach(), foreign["weight"], rtol=0, atol=0)
+    assert torch.equal(image(m.weight), foreign["weight"].bfloat16().float())
+    assert torch.equal(image(m.bias), foreign["bias"].bfloat16().float())
+    # get_params(clone=False) copies the live values into the oldest entry's storage: its image follows
+    stash, _ = opt.get_params(clone=False)
+    slot = stash[0]._pd_slot
+    assert slot != opt.arena.live_slot
+    got = opt.arena.bf16_image[slot][:m.weight.numel()].view_as(m.weight).float()
+    assert torch.equal(got, foreign["weight"].bfloat16().float())
