@@ -121,3 +121,16 @@ def test_checkpoint_resume_matches_oracle_and_formats_interchange():
             torch.testing.assert_close(got[k].cpu(), v, rtol=1e-5, atol=1e-6)
     # after a resume the ring holds identical clones at version 0 + the new updates
     assert st_mine[0][1].queue.versions() == [3, 4]
+
+
+def test_checkpoint_holds_one_copy_of_every_tensor():
+    """The live parameters are views into the version ring and the momentum buffers views into one flat
+    buffer; what ``state_dict()`` hands to ``torch.save`` must not drag the ring's other slots along: the file
+    is about the size of the parameters plus the optimizer state."""
+    stages, _ = _product_segment(gold.make_batches()[:3])
+    buf = io.BytesIO()
+    torch.save([{"state_dict": r.state_dict(), "optimizer": o.state_dict()} for r, o in stages], buf)
+    n_params = sum(p.numel() for r, _ in stages for p in r.parameters())
+    assert stages[0][1].num_versions == 2                       # a ring with more than one slot is in play
+    expected = 2 * 4 * n_params                                 # parameters + momentum, fp32
+    assert expected <= buf.getbuffer().nbytes <= 1.02 * expected + (1 << 16)
