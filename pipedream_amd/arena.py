@@ -24,6 +24,12 @@ ALIGN = 256  # bytes; every entry and every slot starts on a 256-byte boundary
 
 STAGGER = 4096            # bytes between the start addresses of operand streams, modulo STAGGER_PERIOD
 STAGGER_PERIOD = 16384
+# Entries of at least BIG_ENTRY bytes start BIG_ENTRY_PHASE bytes past a STAGGER boundary of their slot: their
+# gradients come from the allocator on large power-of-two boundaries, and with the parameter streams a quarter
+# of a 4 KiB granule off that grid the fused step measured 0.81 (SGD) / 0.78 (Adam) of the HBM peak on VGG16's
+# 32 tensors instead of 0.78 / 0.72 with entries packed at 256-byte granularity.
+BIG_ENTRY = 1 << 20
+BIG_ENTRY_PHASE = 1024
 
 
 def _round_up(x, a):
@@ -131,6 +137,8 @@ class WeightArena(object):
                 # strided views cannot be re-homed; make the owner dense first
                 e.tensor.data = e.tensor.data.contiguous()
                 e.stride = tuple(e.tensor.stride())
+            if e.nbytes >= BIG_ENTRY:
+                off = _round_up(off - BIG_ENTRY_PHASE, STAGGER) + BIG_ENTRY_PHASE
             e.offset = off
             off = _round_up(off + e.nbytes, ALIGN)
             if e.master_index == self.num_master - 1:
@@ -139,7 +147,7 @@ class WeightArena(object):
         # The fused step streams a slot it reads, a slot it writes, the gradients and the optimizer state at
         # the same element offset.  HBM bandwidth drops by 5-8 % when those streams start at the same address
         # modulo 16 KiB, so consecutive slots are staggered by 4 KiB (and the optimizer's flat state buffers,
-        # ``staggered_like``, by 8 and 12 KiB).
+        # ``staggered_empty`` in fused_optim, by 8 and 12 KiB).
         self.slot_bytes = _round_up(max(off, ALIGN), STAGGER_PERIOD) + STAGGER
         self._raw_buffer, self.buffer = staggered_empty(self.num_versions * self.slot_bytes, device, 0)
         # padding between entries must stay finite: the fused step walks it too
