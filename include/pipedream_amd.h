@@ -110,6 +110,25 @@ int pd_sgd_step(const pd_tensor_desc* descs, int n_tensors,
                 int nesterov, int first_step,
                 double loss_scale, double update_interval, void* stream);
 
+/* The same two steps for 16-bit model parameters with fp32 masters -- the branch of
+ * OptimizerWithWeightStashing.step that runtime/optimizer.py:137-155 takes when model_parameters is given
+ * (apex.fp16_utils.model_grads_to_master_grads, the division by loss_scale, the base optimizer on the
+ * masters, master_params_to_model_params) as one launch: desc.grad points at the MODEL's gradient in
+ * grad_format (PD_F32, PD_BF16 or PD_F16; widened exactly), p_in / p_out / state are the fp32 masters
+ * and state, and desc.bf16_out receives the new parameters rounded to out_format (PD_BF16 or PD_F16):
+ * the 16-bit model copy, written straight into the version ring's slot. */
+#define PD_F32 0
+#define PD_BF16 1
+#define PD_F16 2
+int pd_sgd_step_mixed(const pd_tensor_desc* descs, int n_tensors,
+                      double lr, double momentum, double dampening, double weight_decay,
+                      int nesterov, int first_step, double loss_scale, double update_interval,
+                      int grad_format, int out_format, void* stream);
+int pd_adam_step_mixed(const pd_tensor_desc* descs, int n_tensors,
+                       double lr, double beta1, double beta2, double eps, double weight_decay,
+                       int64_t step, int eps_mode, double loss_scale, double update_interval,
+                       int grad_format, int out_format, void* stream);
+
 /* torch.optim.Adam maths (selected at runtime/adam.py:16):
  * eps_mode 0 = installed-torch form  p -= (lr/bc1) * m / (sqrt(v)/sqrt(bc2) + eps)
  * eps_mode 1 = PyTorch-1.1 form      p -= (lr*sqrt(bc2)/bc1) * m / (sqrt(v) + eps)

@@ -173,7 +173,13 @@ class StashingOptimizerOracle(object):
     """``OptimizerWithWeightStashing`` of the reference on CPU tensors."""
 
     def __init__(self, optim_name, modules, master_parameters, num_versions, macrobatch=False,
-                 update_interval=None, **optimizer_args):
+                 update_interval=None, model_parameters=None, loss_scale=1.0, **optimizer_args):
+        """``model_parameters`` / ``loss_scale``: the mixed-precision branch (runtime/optimizer.py:137-155), with
+        the two apex.fp16_utils routines it calls (third-party, absent here) restated from their published
+        behaviour: ``model_grads_to_master_grads`` copies every model gradient into the fp32 gradient of its
+        master, ``master_params_to_model_params`` copies every master into its (16-bit) model parameter."""
+        self.model_parameters = None if model_parameters is None else list(model_parameters)
+        self.loss_scale = loss_scale
         self.modules = list(modules)
         if macrobatch:
             num_versions = min(2, num_versions)
@@ -241,11 +247,21 @@ class StashingOptimizerOracle(object):
         if self.batch_counter % self.update_interval != self.update_interval - 1:
             self.batch_counter += 1
             return
+        if self.model_parameters is not None:
+            for model, master in zip(self.model_parameters, self._masters):      # model_grads_to_master_grads
+                master.grad = None if model.grad is None else model.grad.detach().float()
+            if self.loss_scale != 1.0:                                           # optimizer.py:143-145
+                for master in self._masters:
+                    if master.grad is not None:
+                        master.grad = master.grad / self.loss_scale
         for p, alias in zip(self._masters, self._aliases):
             if p.grad is not None:
                 p.grad.div_(self.update_interval)
             alias.grad = p.grad
         self.base_optimizer.step()
+        if self.model_parameters is not None:
+            for model, master in zip(self.model_parameters, self._masters):      # master_params_to_model_params
+                model.data.copy_(master.data)
         self.latest_version += 1
         if self.num_versions > 1:
             oldest = self.queue[0][0]

@@ -11,6 +11,8 @@ _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "libpipedream_amd.so")
 
 PD_OK = 0
+# element formats of the mixed-precision optimizer step (include/pipedream_amd.h)
+PD_F32, PD_BF16, PD_F16 = 0, 1, 2
 
 
 class PipedreamAmdError(RuntimeError):
@@ -62,6 +64,9 @@ SIGNATURES = {
     "pd_fill_zero": (_i, [_vp, _u64, _vp], True),
     "pd_sgd_step": (_i, [ctypes.POINTER(TensorDesc), _i, _d, _d, _d, _d, _i, _i, _d, _d, _vp], True),
     "pd_adam_step": (_i, [ctypes.POINTER(TensorDesc), _i, _d, _d, _d, _d, _d, _i64, _i, _d, _d, _vp], True),
+    "pd_sgd_step_mixed": (_i, [ctypes.POINTER(TensorDesc), _i, _d, _d, _d, _d, _i, _i, _d, _d, _i, _i, _vp], True),
+    "pd_adam_step_mixed": (_i, [ctypes.POINTER(TensorDesc), _i, _d, _d, _d, _d, _d, _i64, _i, _d, _d, _i, _i, _vp],
+                           True),
     "pd_gemm_f32": (_i, [_i, _i, _i, _i, _i, _vp, _i, _vp, _i, _f, _vp, _i, _vp, _i, _vp], True),
     "pd_gemm_splitk_f32": (_i, [_i, _i, _i, _i, _i, _vp, _i, _vp, _i, _vp, _i, _vp], True),
     "pd_splitk_reduce_f32": (_i, [_vp, _i, _i, _i, _vp, _i, _f, _vp, _i, _vp], True),

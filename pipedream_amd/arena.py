@@ -86,7 +86,12 @@ def _is_dense(t):
 class WeightArena(object):
     """``num_versions`` flat slots + the integer ring that orders them."""
 
-    def __init__(self, modules, master_parameters, num_versions, bf16_image=False):
+    def __init__(self, modules, master_parameters, num_versions, bf16_image=False, model_parameters=None):
+        """``model_parameters`` (16-bit tensors, the modules' own parameters, one per master in the same order):
+        the mixed-precision arrangement of runtime/optimizer.py:137-155.  The ring then stashes the 16-bit
+        model parameters (they are what forward and backward passes read), ``master_parameters`` stay
+        separate fp32 tensors outside the ring, and the fused step updates a master in place while it
+        writes its 16-bit image into the ring's write slot."""
         self._lib = _cabi.lib()
         self.modules = list(modules)
         self.num_versions = int(num_versions)
@@ -98,12 +103,32 @@ class WeightArena(object):
             raise ValueError("optimizer got an empty parameter list")
         device = masters[0].device
         _cabi.require_device(masters[0], "master parameter")
+        self.fp32_masters = None
+        self.half_dtype = None
+        if model_parameters is not None:
+            model_parameters = list(model_parameters)
+            if bf16_image:
+                raise ValueError("bf16_image keeps a 16-bit copy of fp32 module parameters; with model_parameters "
+                                 "the module parameters are the 16-bit copy")
+            if len(model_parameters) != len(masters):
+                raise ValueError("model_parameters and master_parameters differ in length")
+            self.half_dtype = model_parameters[0].dtype
+            if self.half_dtype not in (torch.bfloat16, torch.float16):
+                raise TypeError("model parameters must be bfloat16 or float16, got %s" % self.half_dtype)
+            for q, p in zip(model_parameters, masters):
+                if q.dtype != self.half_dtype or p.dtype != torch.float32 or q.shape != p.shape or q.device != device:
+                    raise TypeError("every model parameter must be a %s tensor with an fp32 master of its shape on %s"
+                                    % (self.half_dtype, device))
+                if not p.is_contiguous() or p.data_ptr() % 16:
+                    raise ValueError("fp32 masters must be contiguous, 16-byte aligned tensors")
+            self.fp32_masters = masters
+            masters = model_parameters          # what the ring stashes
 
         by_id = collections.OrderedDict()
         # 1. master parameters first, in optimizer order: they form one fp32 section that
         #    the fused step kernel walks.
         for i, p in enumerate(masters):
-            if p.dtype != torch.float32:
+            if p.dtype != (self.half_dtype or torch.float32):
                 raise TypeError("master parameters must be fp32, got %s" % p.dtype)
             if p.device != device:
                 raise ValueError("all parameters of a stage must live on one device")

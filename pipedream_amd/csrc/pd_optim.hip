@@ -29,6 +29,8 @@ struct OptArgs {
     uint32_t block_start[OPT_MAX_TENSORS + 1];  // prefix sum of per-tensor block counts
     uint32_t vec_ok;                            // bit i: all pointers of tensor i are 16-B aligned
     int n_tensors;
+    int grad_fmt;                               // PD_F32 / PD_BF16 / PD_F16: what desc.grad points at
+    int out_fmt;                                // PD_BF16 / PD_F16: format of the 16-bit copy (desc.bf16_out)
 };
 
 struct SgdHyper {
@@ -85,6 +87,18 @@ __device__ __forceinline__ void adam_elem(float g, float p, float& m, float& v, 
     p_new = __fadd_rn(p, __fdiv_rn(__fmul_rn(-h.step_size, m), denom));
 }
 
+// 16-bit formats of the mixed-precision step: gradients arrive in the model's format and are widened, the
+// new parameters are also written in it (both conversions round to nearest even)
+__device__ __forceinline__ float half_to_f32(uint16_t h, int fmt) {
+    return fmt == PD_F16 ? (float)__builtin_bit_cast(_Float16, h) : __uint_as_float((uint32_t)h << 16);
+}
+
+__device__ __forceinline__ uint16_t f32_to_bf16_rne(float f);
+
+__device__ __forceinline__ uint16_t f32_to_half(float f, int fmt) {
+    return fmt == PD_F16 ? __builtin_bit_cast(uint16_t, (_Float16)f) : f32_to_bf16_rne(f);
+}
+
 __device__ __forceinline__ uint16_t f32_to_bf16_rne(float f) {
     uint32_t u = __float_as_uint(f);
     if ((u & 0x7fffffffu) > 0x7f800000u) return (uint16_t)((u >> 16) | 0x0040u);  // quiet NaN
@@ -103,7 +117,9 @@ __device__ __forceinline__ int find_tensor(const OptArgs& a, uint32_t b) {
     return ti;
 }
 
-template <bool ADAM>
+// MIXED: gradients (and the 16-bit parameter copy) are in a 16-bit format chosen per launch; the fp32 path
+// is its own instantiation and carries none of that.
+template <bool ADAM, bool MIXED>
 __global__ __launch_bounds__(OPT_THREADS) void pd_optim_kernel(const OptArgs a, const SgdHyper sh, const AdamHyper ah) {
     const int ti = find_tensor(a, blockIdx.x);
     const pd_tensor_desc& t = a.t[ti];
@@ -120,7 +136,14 @@ __global__ __launch_bounds__(OPT_THREADS) void pd_optim_kernel(const OptArgs a, 
 #pragma unroll
         for (int u = 0; u < OPT_UNROLL; ++u) {
             const uint64_t i = v0 + (uint64_t)u * OPT_THREADS;
-            g[u] = __builtin_nontemporal_load((const float4_t*)t.grad + i);
+            if (MIXED) {
+                typedef uint16_t u16x4 __attribute__((ext_vector_type(4)));
+                const u16x4 h = __builtin_nontemporal_load((const u16x4*)t.grad + i);
+#pragma unroll
+                for (int k = 0; k < 4; ++k) g[u][k] = half_to_f32(h[k], a.grad_fmt);
+            } else {
+                g[u] = __builtin_nontemporal_load((const float4_t*)t.grad + i);
+            }
             p[u] = __builtin_nontemporal_load((const float4_t*)t.p_in + i);
             if (has_s0) s0[u] = __builtin_nontemporal_load((const float4_t*)t.state0 + i);
             if (ADAM) s1[u] = __builtin_nontemporal_load((const float4_t*)t.state1 + i);
@@ -149,7 +172,10 @@ __global__ __launch_bounds__(OPT_THREADS) void pd_optim_kernel(const OptArgs a, 
             if (ADAM) __builtin_nontemporal_store(s1[u], (float4_t*)t.state1 + i);
             if (t.bf16_out) {
                 typedef uint16_t u16x4 __attribute__((ext_vector_type(4)));
-                u16x4 h = {f32_to_bf16_rne(pn[0]), f32_to_bf16_rne(pn[1]), f32_to_bf16_rne(pn[2]), f32_to_bf16_rne(pn[3])};
+                u16x4 h;
+                if (MIXED) h = u16x4{f32_to_half(pn[0], a.out_fmt), f32_to_half(pn[1], a.out_fmt),
+                                     f32_to_half(pn[2], a.out_fmt), f32_to_half(pn[3], a.out_fmt)};
+                else h = u16x4{f32_to_bf16_rne(pn[0]), f32_to_bf16_rne(pn[1]), f32_to_bf16_rne(pn[2]), f32_to_bf16_rne(pn[3])};
                 *((u16x4*)t.bf16_out + i) = h;
             }
         }
@@ -158,7 +184,7 @@ __global__ __launch_bounds__(OPT_THREADS) void pd_optim_kernel(const OptArgs a, 
         for (int u = 0; u < OPT_UNROLL * 4; ++u) {
             const uint64_t i = chunk0 + (uint64_t)u * OPT_THREADS + threadIdx.x;
             if (i >= n) break;
-            float g = t.grad[i], p = t.p_in[i], pn;
+            float g = MIXED ? half_to_f32(((const uint16_t*)t.grad)[i], a.grad_fmt) : t.grad[i], p = t.p_in[i], pn;
             if (ADAM) {
                 float m = t.state0[i], v = t.state1[i];
                 adam_elem(g, p, m, v, pn, ah);
@@ -170,15 +196,19 @@ __global__ __launch_bounds__(OPT_THREADS) void pd_optim_kernel(const OptArgs a, 
                 if (has_s0) t.state0[i] = b;
             }
             t.p_out[i] = pn;
-            if (t.bf16_out) t.bf16_out[i] = f32_to_bf16_rne(pn);
+            if (t.bf16_out) t.bf16_out[i] = MIXED ? f32_to_half(pn, a.out_fmt) : f32_to_bf16_rne(pn);
         }
     }
 }
 
 template <bool ADAM>
 int launch_optim(const pd_tensor_desc* descs, int n_tensors, const SgdHyper& sh, const AdamHyper& ah,
-                 bool need_s0, void* stream, const char* who) {
+                 bool need_s0, void* stream, const char* who, int grad_fmt = PD_F32, int out_fmt = PD_BF16) {
     PD_REQUIRE(n_tensors >= 0, PD_EINVAL, "%s: n_tensors < 0", who);
+    PD_REQUIRE(grad_fmt == PD_F32 || grad_fmt == PD_BF16 || grad_fmt == PD_F16, PD_EINVAL, "%s: unknown gradient format %d",
+               who, grad_fmt);
+    PD_REQUIRE(out_fmt == PD_BF16 || out_fmt == PD_F16, PD_EINVAL, "%s: unknown 16-bit output format %d", who, out_fmt);
+    const bool mixed = grad_fmt != PD_F32 || out_fmt != PD_BF16;
     if (n_tensors == 0) return PD_OK;
     PD_REQUIRE(descs != nullptr, PD_EINVAL, "%s: descs is NULL", who);
     int i = 0;
@@ -194,14 +224,14 @@ int launch_optim(const pd_tensor_desc* descs, int n_tensors, const SgdHyper& sh,
             PD_REQUIRE(d.grad && d.p_in && d.p_out, PD_EINVAL, "%s: tensor %d has a NULL grad/param pointer", who, i);
             PD_REQUIRE(!need_s0 || d.state0, PD_EINVAL, "%s: tensor %d has no state0 buffer", who, i);
             PD_REQUIRE(!ADAM || d.state1, PD_EINVAL, "%s: tensor %d has no state1 buffer", who, i);
-            PD_REQUIRE(pd_aligned(d.grad, 4) && pd_aligned(d.p_in, 4) && pd_aligned(d.p_out, 4), PD_EINVAL,
-                       "%s: tensor %d is not 4-byte aligned", who, i);
+            PD_REQUIRE(pd_aligned(d.grad, grad_fmt == PD_F32 ? 4 : 2) && pd_aligned(d.p_in, 4) && pd_aligned(d.p_out, 4),
+                       PD_EINVAL, "%s: tensor %d is not aligned to its element size", who, i);
             uint64_t nb = (d.n + OPT_CHUNK - 1) / OPT_CHUNK;
             if (blocks + nb > 0x7fffffffull) {
                 PD_REQUIRE(a.n_tensors > 0, PD_ESHAPE, "%s: tensor %d too large for one launch", who, i);
                 break;  // flush what we have, continue with this tensor in the next launch
             }
-            bool ok = pd_aligned(d.grad, 16) && pd_aligned(d.p_in, 16) && pd_aligned(d.p_out, 16) &&
+            bool ok = pd_aligned(d.grad, grad_fmt == PD_F32 ? 16 : 8) && pd_aligned(d.p_in, 16) && pd_aligned(d.p_out, 16) &&
                       (!d.state0 || pd_aligned(d.state0, 16)) && (!d.state1 || pd_aligned(d.state1, 16)) &&
                       (!d.bf16_out || pd_aligned(d.bf16_out, 8));
             int k = a.n_tensors++;
@@ -213,7 +243,10 @@ int launch_optim(const pd_tensor_desc* descs, int n_tensors, const SgdHyper& sh,
         }
         if (a.n_tensors == 0) break;
         for (int k = a.n_tensors + 1; k <= OPT_MAX_TENSORS; ++k) a.block_start[k] = (uint32_t)blocks;
-        pd_optim_kernel<ADAM><<<dim3((unsigned)blocks), dim3(OPT_THREADS), 0, (hipStream_t)stream>>>(a, sh, ah);
+        a.grad_fmt = grad_fmt;
+        a.out_fmt = out_fmt;
+        if (mixed) pd_optim_kernel<ADAM, true><<<dim3((unsigned)blocks), dim3(OPT_THREADS), 0, (hipStream_t)stream>>>(a, sh, ah);
+        else pd_optim_kernel<ADAM, false><<<dim3((unsigned)blocks), dim3(OPT_THREADS), 0, (hipStream_t)stream>>>(a, sh, ah);
         PD_CHECK_LAUNCH(who);
     }
     return PD_OK;
@@ -221,9 +254,9 @@ int launch_optim(const pd_tensor_desc* descs, int n_tensors, const SgdHyper& sh,
 
 }  // namespace
 
-extern "C" int pd_sgd_step(const pd_tensor_desc* descs, int n_tensors, double lr, double momentum, double dampening,
-                           double weight_decay, int nesterov, int first_step, double loss_scale,
-                           double update_interval, void* stream) {
+static int sgd_step(const pd_tensor_desc* descs, int n_tensors, double lr, double momentum, double dampening,
+                    double weight_decay, int nesterov, int first_step, double loss_scale, double update_interval,
+                    int grad_fmt, int out_fmt, void* stream) {
     PD_REQUIRE(loss_scale != 0.0 && update_interval != 0.0, PD_EINVAL, "pd_sgd_step: zero loss_scale/update_interval");
     SgdHyper sh;
     sh.lr = (float)lr;
@@ -236,12 +269,27 @@ extern "C" int pd_sgd_step(const pd_tensor_desc* descs, int n_tensors, double lr
     sh.first_step = first_step != 0;
     sh.has_momentum = momentum != 0.0;
     AdamHyper ah = {};
-    return launch_optim<false>(descs, n_tensors, sh, ah, sh.has_momentum, stream, "pd_sgd_step");
+    return launch_optim<false>(descs, n_tensors, sh, ah, sh.has_momentum, stream, "pd_sgd_step", grad_fmt, out_fmt);
 }
 
-extern "C" int pd_adam_step(const pd_tensor_desc* descs, int n_tensors, double lr, double beta1, double beta2,
-                            double eps, double weight_decay, int64_t step, int eps_mode, double loss_scale,
-                            double update_interval, void* stream) {
+extern "C" int pd_sgd_step(const pd_tensor_desc* descs, int n_tensors, double lr, double momentum, double dampening,
+                           double weight_decay, int nesterov, int first_step, double loss_scale,
+                           double update_interval, void* stream) {
+    return sgd_step(descs, n_tensors, lr, momentum, dampening, weight_decay, nesterov, first_step, loss_scale,
+                    update_interval, PD_F32, PD_BF16, stream);
+}
+
+extern "C" int pd_sgd_step_mixed(const pd_tensor_desc* descs, int n_tensors, double lr, double momentum,
+                                 double dampening, double weight_decay, int nesterov, int first_step,
+                                 double loss_scale, double update_interval, int grad_format, int out_format,
+                                 void* stream) {
+    return sgd_step(descs, n_tensors, lr, momentum, dampening, weight_decay, nesterov, first_step, loss_scale,
+                    update_interval, grad_format, out_format, stream);
+}
+
+static int adam_step(const pd_tensor_desc* descs, int n_tensors, double lr, double beta1, double beta2, double eps,
+                     double weight_decay, int64_t step, int eps_mode, double loss_scale, double update_interval,
+                     int grad_fmt, int out_fmt, void* stream) {
     PD_REQUIRE(step >= 1, PD_EINVAL, "pd_adam_step: step must be >= 1");
     PD_REQUIRE(eps_mode == 0 || eps_mode == 1, PD_EINVAL, "pd_adam_step: eps_mode must be 0 or 1");
     PD_REQUIRE(loss_scale != 0.0 && update_interval != 0.0, PD_EINVAL, "pd_adam_step: zero loss_scale/update_interval");
@@ -265,5 +313,19 @@ extern "C" int pd_adam_step(const pd_tensor_desc* descs, int n_tensors, double l
     ah.update_interval = (float)update_interval;
     ah.eps_mode = eps_mode;
     SgdHyper sh = {};
-    return launch_optim<true>(descs, n_tensors, sh, ah, true, stream, "pd_adam_step");
+    return launch_optim<true>(descs, n_tensors, sh, ah, true, stream, "pd_adam_step", grad_fmt, out_fmt);
+}
+
+extern "C" int pd_adam_step(const pd_tensor_desc* descs, int n_tensors, double lr, double beta1, double beta2,
+                            double eps, double weight_decay, int64_t step, int eps_mode, double loss_scale,
+                            double update_interval, void* stream) {
+    return adam_step(descs, n_tensors, lr, beta1, beta2, eps, weight_decay, step, eps_mode, loss_scale, update_interval,
+                     PD_F32, PD_BF16, stream);
+}
+
+extern "C" int pd_adam_step_mixed(const pd_tensor_desc* descs, int n_tensors, double lr, double beta1, double beta2,
+                                  double eps, double weight_decay, int64_t step, int eps_mode, double loss_scale,
+                                  double update_interval, int grad_format, int out_format, void* stream) {
+    return adam_step(descs, n_tensors, lr, beta1, beta2, eps, weight_decay, step, eps_mode, loss_scale, update_interval,
+                     grad_format, out_format, stream);
 }

@@ -31,12 +31,21 @@ class _FusedOptimizer(torch.optim.Optimizer):
             arena = WeightArena([], masters, 1)
         self.arena = arena
         self._index = {}
-        for e in arena.entries[:arena.num_master]:
-            self._index[id(e.tensor)] = e
+        # mixed precision: the parameters this optimizer updates are fp32 masters outside the ring, entry i of
+        # the ring holds the 16-bit model parameter of master i
+        self.mixed = arena.fp32_masters is not None
+        self._elem = 2 if self.mixed else 4                   # bytes per element of a ring entry
+        owners = arena.fp32_masters if self.mixed else [e.tensor for e in arena.entries[:arena.num_master]]
+        for e, owner in zip(arena.entries[:arena.num_master], owners):
+            self._index[id(owner)] = e
         for p in masters:
             if id(p) not in self._index:
                 raise ValueError("parameter is not part of the weight arena")
-        n = arena.master_bytes // 4
+        self._formats = (_cabi.PD_F32, _cabi.PD_BF16)
+        if self.mixed:
+            fmt = _cabi.PD_BF16 if arena.half_dtype == torch.bfloat16 else _cabi.PD_F16
+            self._formats = (fmt, fmt)
+        n = arena.master_bytes // self._elem
         device = arena.buffer.device
         # flat state buffers share the slot layout of the master section
         # (start addresses staggered against the ring's slots, see arena.staggered_empty)
@@ -50,35 +59,57 @@ class _FusedOptimizer(torch.optim.Optimizer):
     # -- helpers -----------------------------------------------------------------------
     def _state_view(self, which, p):
         e = self._index[id(p)]
-        lo = e.offset // 4
+        lo = e.offset // self._elem
         flat = self._flat_state[which][lo:lo + e.numel]
         if e.tensor.is_contiguous():
             return flat.view(e.shape)
         return flat.as_strided(e.shape, e.stride)
 
+    def _grad_owner(self, p):
+        """The tensor whose ``.grad`` the step reads: the parameter itself, or in mixed precision the 16-bit
+        model parameter behind the master (the kernel widens it: no master gradient is ever materialised)."""
+        return self._index[id(p)].tensor if self.mixed else p
+
     def _grad_for(self, p):
-        g = p.grad
-        if g.dtype != torch.float32 or g.device != p.device or g.is_sparse:
-            raise TypeError("gradients must be dense fp32 tensors on the parameter's device")
-        if g.stride() != p.stride():
+        owner = self._grad_owner(p)
+        g = owner.grad
+        if g.dtype != owner.dtype or g.device != p.device or g.is_sparse:
+            raise TypeError("gradients must be dense %s tensors on the parameter's device" % owner.dtype)
+        if g.stride() != (p.stride() if self.mixed else owner.stride()):
             # bring the gradient into the parameter's memory order
-            g2 = torch.empty_like(p)
+            g2 = torch.empty(p.shape, dtype=g.dtype, device=g.device)
             g2.copy_(g)
             g = g2
         return g
+
+    def zero_grad(self, set_to_none=True):
+        super(_FusedOptimizer, self).zero_grad(set_to_none=set_to_none)
+        if self.mixed:
+            # the gradients the step reads live on the model parameters
+            for e in self.arena.entries[:self.arena.num_master]:
+                if set_to_none:
+                    e.tensor.grad = None
+                elif e.tensor.grad is not None:
+                    e.tensor.grad.zero_()
 
     def _fill(self, k, p, g, in_slot, out_slot, use_s0, use_s1):
         e = self._index[id(p)]
         d = self._descs[k]
         d.grad = g.data_ptr()
-        d.p_in = e.views[in_slot].data_ptr()
-        d.p_out = e.views[out_slot].data_ptr()
-        d.state0 = self._flat_state[0].data_ptr() + e.offset if use_s0 else None
-        d.state1 = self._flat_state[1].data_ptr() + e.offset if use_s1 else None
-        if self.bf16_copy is not None:
-            d.bf16_out = self.bf16_copy[out_slot].data_ptr() + e.offset // 2
+        state_offset = e.offset // self._elem * 4
+        d.state0 = self._flat_state[0].data_ptr() + state_offset if use_s0 else None
+        d.state1 = self._flat_state[1].data_ptr() + state_offset if use_s1 else None
+        if self.mixed:
+            # the master is updated in place; its 16-bit image goes into the ring's write slot
+            d.p_in = d.p_out = p.data_ptr()
+            d.bf16_out = e.views[out_slot].data_ptr()
         else:
-            d.bf16_out = None
+            d.p_in = e.views[in_slot].data_ptr()
+            d.p_out = e.views[out_slot].data_ptr()
+            if self.bf16_copy is not None:
+                d.bf16_out = self.bf16_copy[out_slot].data_ptr() + e.offset // 2
+            else:
+                d.bf16_out = None
         d.n = e.numel
 
     def load_state_dict(self, state_dict):
@@ -130,7 +161,7 @@ class SGD(_FusedOptimizer):
             for first in (False, True):
                 k = 0
                 for p in group["params"]:
-                    if p.grad is None:
+                    if self._grad_owner(p).grad is None:
                         continue
                     st = self.state[p]
                     is_first = momentum != 0 and st.get("momentum_buffer") is None
@@ -143,10 +174,10 @@ class SGD(_FusedOptimizer):
                         st["momentum_buffer"] = self._state_view(0, p)
                     k += 1
                 if k:
-                    self._lib.pd_sgd_step(self._descs, k, float(group["lr"]), float(momentum),
-                                          float(group["dampening"]), float(group["weight_decay"]),
-                                          int(bool(group["nesterov"])), int(first), float(loss_scale),
-                                          float(update_interval), stream)
+                    self._lib.pd_sgd_step_mixed(self._descs, k, float(group["lr"]), float(momentum),
+                                                float(group["dampening"]), float(group["weight_decay"]),
+                                                int(bool(group["nesterov"])), int(first), float(loss_scale),
+                                                float(update_interval), self._formats[0], self._formats[1], stream)
         self._carry_untouched(in_slot, out_slot)
         return loss
 
@@ -157,8 +188,11 @@ class SGD(_FusedOptimizer):
             return
         for group in self.param_groups:
             for p in group["params"]:
-                if p.grad is None:
+                if self._grad_owner(p).grad is None:
                     e = self._index[id(p)]
+                    if self.mixed:          # (a 16-bit entry's size need not be a multiple of 4 bytes)
+                        e.views[out_slot].copy_(e.views[in_slot])
+                        continue
                     self._lib.pd_copy(ctypes.c_void_p(e.views[out_slot].data_ptr()),
                                       ctypes.c_void_p(e.views[in_slot].data_ptr()), e.nbytes, _cabi.stream_ptr())
                     if self.bf16_copy is not None:
@@ -207,7 +241,7 @@ class Adam(_FusedOptimizer):
             beta1, beta2 = group["betas"]
             by_step = {}
             for p in group["params"]:
-                if p.grad is None:
+                if self._grad_owner(p).grad is None:
                     continue
                 st = self.state[p]
                 if "step" not in st:
@@ -223,9 +257,10 @@ class Adam(_FusedOptimizer):
                     g = self._grad_for(p)
                     keep.append(g)
                     self._fill(k, p, g, in_slot, out_slot, True, True)
-                self._lib.pd_adam_step(self._descs, len(plist), float(group["lr"]), float(beta1), float(beta2),
-                                       float(group["eps"]), float(group["weight_decay"]), t, self.eps_mode,
-                                       float(loss_scale), float(update_interval), stream)
+                self._lib.pd_adam_step_mixed(self._descs, len(plist), float(group["lr"]), float(beta1), float(beta2),
+                                             float(group["eps"]), float(group["weight_decay"]), t, self.eps_mode,
+                                             float(loss_scale), float(update_interval), self._formats[0],
+                                             self._formats[1], stream)
         SGD._carry_untouched(self, in_slot, out_slot)
         return loss
 

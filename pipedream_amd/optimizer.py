@@ -43,6 +43,15 @@ class Version(object):
         return Version(version=self.version + 1)
 
 
+def prep_param_lists(model):
+    """``(model parameters, fp32 master parameters)`` of a 16-bit module: what runtime/runtime.py:268-276
+    obtains from ``apex.fp16_utils.prep_param_lists`` (third-party, not needed here): the module's own
+    parameters and, for each, a detached fp32 clone that requires grad."""
+    model_params = [p for p in model.parameters() if p.requires_grad]
+    master_params = [p.detach().clone().float().requires_grad_() for p in model_params]
+    return model_params, master_params
+
+
 class _RingQueue(object):
     """Read-only ``deque``-like face of the ring: ``queue[i] -> (state_dicts, Version)``
     with index 0 the oldest entry, as ``deque(maxlen=num_versions)`` in the reference."""
@@ -82,6 +91,13 @@ class OptimizerWithWeightStashing(torch.optim.Optimizer):
     reference) decouples gradient accumulation from ``num_versions`` for 2BW-style
     double buffering; left at ``None`` it follows the reference rule.  ``bf16_image`` (not
     in the reference) keeps a bf16 copy of every weight version for bf16-compute stages.
+
+    ``model_parameters`` (the reference's fp16 arrangement, optimizer.py:137-155): the modules hold 16-bit
+    parameters (bfloat16 or float16), ``master_parameters`` are their fp32 masters (``prep_param_lists``).
+    The ring then stashes the 16-bit versions, and a step -- model gradients widened to fp32, divided by
+    ``loss_scale``, the base optimizer on the masters, the masters copied back into the model -- is the same
+    single launch, which reads the 16-bit gradients and writes the 16-bit image of the new weights into
+    the ring's write slot.
     """
 
     def __init__(self, optim_name, modules, master_parameters, model_parameters,
@@ -91,9 +107,8 @@ class OptimizerWithWeightStashing(torch.optim.Optimizer):
             raise NotImplementedError(
                 "optim_name %r has no fused HIP kernel (available: %s)" % (optim_name, sorted(BASE_OPTIMIZERS)))
         if model_parameters is not None:
-            raise NotImplementedError(
-                "separate fp16 model parameters (the apex path of the reference) are not supported; "
-                "keep fp32 master parameters in the modules")
+            # mixed precision (optimizer.py:137-155): 16-bit parameters in the modules, fp32 masters beside them
+            model_parameters = list(model_parameters)
         self.modules = modules
         self.master_parameters = master_parameters = list(master_parameters)
         self.model_parameters = model_parameters
@@ -110,7 +125,8 @@ class OptimizerWithWeightStashing(torch.optim.Optimizer):
                 flat_masters.extend(item["params"])
             else:
                 flat_masters.append(item)
-        self.arena = WeightArena(self.modules, flat_masters, num_versions, bf16_image=bf16_image)
+        self.arena = WeightArena(self.modules, flat_masters, num_versions, bf16_image=bf16_image,
+                                 model_parameters=model_parameters)
         self.base_optimizer = BASE_OPTIMIZERS[optim_name](master_parameters, arena=self.arena, **optimizer_args)
         self.latest_version = Version()
         self.current_version = Version()
@@ -223,8 +239,10 @@ class OptimizerWithWeightStashing(torch.optim.Optimizer):
         arena = self.arena
         in_slot = arena.live_slot
         out_slot = arena.write_slot() if self.num_versions > 1 else in_slot
+        # the reference divides by loss_scale only on the mixed-precision branch (optimizer.py:137-145)
+        loss_scale = float(self.loss_scale) if self.model_parameters is not None else 1.0
         loss = self.base_optimizer.step(closure, in_slot=in_slot, out_slot=out_slot,
-                                        loss_scale=1.0, update_interval=float(self.update_interval))
+                                        loss_scale=loss_scale, update_interval=float(self.update_interval))
         self.latest_version = self.latest_version.incr()
         if self.num_versions > 1:
             arena.store_others(out_slot)

@@ -168,8 +168,9 @@ def test_unknown_optimizer_and_fp16_lists_fail_loudly():
     model = _mlp(0).cuda()
     with pytest.raises(NotImplementedError):
         optimizer.OptimizerWithWeightStashing("RMSprop", [model], model.parameters(), None, 1.0, 2, lr=0.1)
-    with pytest.raises(NotImplementedError):
-        sgd.SGDWithWeightStashing([model], model.parameters(), list(model.parameters()), 1.0, 2, lr=0.1)
+    # model parameters are the modules' 16-bit parameters; fp32 ones are not a mixed-precision set-up
+    with pytest.raises(TypeError, match="bfloat16 or float16"):
+        sgd.SGDWithWeightStashing([model], list(model.parameters()), list(model.parameters()), 1.0, 2, lr=0.1)
 
 
 def test_bf16_image_follows_writes_that_bypass_the_fused_step():
@@ -195,3 +196,63 @@ def test_bf16_image_follows_writes_that_bypass_the_fused_step():
     assert slot != opt.arena.live_slot
     got = opt.arena.bf16_image[slot][:m.weight.numel()].view_as(m.weight).float()
     assert torch.equal(got, foreign["weight"].bfloat16().float())
+
+
+@pytest.mark.parametrize("kind,dtype,loss_scale,macrobatch", [("SGD", torch.bfloat16, 1.0, False),
+                                                              ("SGD", torch.float16, 128.0, False),
+                                                              ("Adam", torch.bfloat16, 1.0, False),
+                                                              ("Adam", torch.float16, 1024.0, True)])
+def test_mixed_precision_step_with_stashing_matches_oracle(kind, dtype, loss_scale, macrobatch):
+    """16-bit model parameters with fp32 masters (runtime/optimizer.py:137-155) under weight stashing: the
+    fused step reads the model's 16-bit gradients, divides by the loss scale, updates the masters and writes
+    the 16-bit image of the new weights into the ring.  Against the oracle's restatement of that branch:
+    versions bit-exact; masters and optimizer state rel 1e-5; the model parameters are exactly the rounded
+    masters and within one 16-bit ulp of the oracle's; every stashed version that ``load_old_params`` brings
+    back likewise."""
+    import copy
+    torch.manual_seed(0)
+    ref = torch.nn.Sequential(torch.nn.Linear(24, 17), torch.nn.Linear(17, 9)).to(dtype)
+    mine = copy.deepcopy(ref).cuda()
+    ref_model, ref_master = optimizer.prep_param_lists(ref)
+    model_params, master_params = optimizer.prep_param_lists(mine)
+    assert all(m.dtype == torch.float32 and m.requires_grad for m in master_params)
+    kw = dict(lr=0.05, momentum=0.9, weight_decay=1e-3) if kind == "SGD" else dict(lr=0.01, weight_decay=1e-3)
+    W, nv, n = 2, 3, 9
+    opt = optimizer.OptimizerWithWeightStashing(kind, [mine], master_params, model_params, loss_scale, nv,
+                                                macrobatch=macrobatch, **kw)
+    ora = so.StashingOptimizerOracle(kind, [ref], ref_master, nv, macrobatch=macrobatch, model_parameters=ref_model,
+                                     loss_scale=loss_scale, **kw)
+    assert opt.num_versions == ora.num_versions and opt.update_interval == ora.update_interval
+    ulp = 2.0 ** -7 if dtype == torch.bfloat16 else 2.0 ** -10
+    g = torch.Generator().manual_seed(1)
+
+    def same_model(stage):
+        for q, r in zip(mine.parameters(), ref.parameters()):
+            torch.testing.assert_close(q.detach().float().cpu(), r.detach().float(), rtol=ulp, atol=1e-6,
+                                       msg=lambda m: "%s: %s" % (stage, m))
+
+    for kind_ev, k in so.one_f_one_b(n, W):
+        if kind_ev == "F":
+            continue
+        for o, module in ((ora, ref), (opt, mine)):
+            o.zero_grad()
+            if o.batch_counter % o.update_interval == 0:
+                module.zero_grad()                  # the caller zeroes the model's gradients (main_with_runtime.py:406-409)
+            o.load_old_params()
+        assert opt.current_version.version == ora.current_version
+        same_model("stashed version loaded for the backward pass of minibatch %d" % k)
+        for q, r in zip(mine.parameters(), ref.parameters()):
+            grad = (torch.randn(r.shape, generator=g) * loss_scale).to(dtype)
+            r.grad = grad.clone() if r.grad is None else r.grad + grad
+            q.grad = grad.cuda() if q.grad is None else q.grad + grad.cuda()
+        for o in (ora, opt):
+            o.load_new_params()
+            o.step()
+        assert opt.queue.versions() == ora.versions() and opt.latest_version.version == ora.latest_version
+        same_model("after update %d" % k)
+        for m, rm, q in zip(master_params, ref_master, mine.parameters()):
+            torch.testing.assert_close(m.detach().cpu(), rm.detach(), rtol=1e-5, atol=1e-6)
+            assert torch.equal(q.detach(), m.detach().to(dtype))          # the model is the rounded master
+    name = "momentum_buffer" if kind == "SGD" else "exp_avg"
+    for m, alias in zip(master_params, ora._aliases):
+        torch.testing.assert_close(opt.state[m][name].cpu(), ora.base_optimizer.state[alias][name], rtol=1e-5, atol=1e-6)

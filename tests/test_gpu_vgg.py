@@ -514,7 +514,7 @@ def test_front_stage_full_size_every_layer_against_fp64():
         for n in (0, N - 1):
             for win in _windows(H, W):
                 h0, h1, w0, w1 = win
-                z = F.conv2d(_crop_with_halo(inp, n, win, 1)[None], w64, b64)[0]
+                z = F.conv2d(_crop_with_halo(inp.detach(), n, win, 1)[None], w64, b64)[0]
                 ref = torch.relu(z)
                 if idx is None:
                     close(name + " output", out[n, :, h0:h1, w0:w1], ref)
@@ -528,7 +528,7 @@ def test_front_stage_full_size_every_layer_against_fp64():
                 win4 = z.reshape(z.shape[0], (h1 - h0) // 2, 2, (w1 - w0) // 2, 2).permute(0, 1, 3, 2, 4).reshape(
                     z.shape[0], (h1 - h0) // 2, (w1 - w0) // 2, 4)
                 top = torch.topk(win4, 2, dim=-1).values
-                margin = 1e-4 * float(z.std())
+                margin = 1e-4 * float(z.detach().std())
                 positive = top[..., 0] > 0
                 assert torch.equal((got >> 2)[top[..., 0].abs() > margin] == 1, positive[top[..., 0].abs() > margin])
                 decided = positive & (top[..., 0] - top[..., 1] > margin) & (top[..., 0] > margin)

@@ -180,3 +180,49 @@ def test_oracle_macrobatch_equals_accumulate_then_step():
         opt.step()
     for pa, pb in zip(a.parameters(), b.parameters()):
         torch.testing.assert_close(pa, pb, rtol=1e-5, atol=1e-6)
+
+
+def test_mixed_precision_branch_of_the_oracle_against_hand_values():
+    """The branch of ``step`` taken with model parameters (runtime/optimizer.py:137-155), pinned by what the
+    arithmetic fixes: with plain SGD the master after n steps is ``m0 - lr * sum(float(g16)) / loss_scale``
+    computed step by step in fp32; the model is the rounded master at every step; a power-of-two loss scale
+    applied to the gradients changes nothing; and the masters keep updates too small for the 16-bit model
+    (a model updated in its own precision would not move)."""
+    import copy
+    dtype = torch.bfloat16
+    torch.manual_seed(0)
+    model = torch.nn.Linear(6, 5, bias=False).to(dtype)
+    twin = copy.deepcopy(model)
+    masters = [p.detach().clone().float().requires_grad_() for p in model.parameters()]
+    masters2 = [p.detach().clone().float().requires_grad_() for p in twin.parameters()]
+    lr = 2.0 ** -12
+    a = so.StashingOptimizerOracle("SGD", [model], masters, 2, model_parameters=list(model.parameters()),
+                                   loss_scale=1.0, lr=lr)
+    b = so.StashingOptimizerOracle("SGD", [twin], masters2, 2, model_parameters=list(twin.parameters()),
+                                   loss_scale=256.0, lr=lr)
+    m0 = masters[0].detach().clone()
+    w0 = model.weight.detach().clone()
+    g = torch.Generator().manual_seed(1)
+    want = m0.clone()
+    for step in range(20):
+        grad = torch.randn(5, 6, generator=g).to(dtype)
+        model.weight.grad = grad.clone()
+        twin.weight.grad = (grad.float() * 256.0).to(dtype)          # exact: a power of two
+        for o in (a, b):
+            o.load_old_params()
+            o.load_new_params()
+            o.step()
+        want = want - lr * grad.float()
+        assert torch.equal(masters[0].detach(), want)                 # fp32, step by step
+        assert torch.equal(masters2[0].detach(), want)                # the loss scale divides out exactly
+        assert torch.equal(model.weight.detach(), want.to(dtype))     # the model is the rounded master
+        assert a.versions() == [step, step + 1]
+    # the updates (about 2^-12 each) are below half an ulp of most bf16 weights: stepping the model in its
+    # own precision leaves those weights where they were, the masters moved
+    stalled = w0.clone()
+    g = torch.Generator().manual_seed(1)
+    for step in range(20):
+        stalled = (stalled.float() - lr * torch.randn(5, 6, generator=g).to(dtype).float()).to(dtype)
+    big = w0.float().abs() > 0.25
+    assert big.any() and torch.equal(stalled[big], w0[big])
+    assert not torch.equal(masters[0].detach()[big], m0[big])
