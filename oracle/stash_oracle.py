@@ -30,6 +30,11 @@ What is restated, and from where (paths relative to the reference checkout):
 * ``warmup_depth`` -- runtime/runtime.py:162-175.
 * ``adjust_learning_rate`` -- runtime/image_classification/main_with_runtime.py:532-563.
 
+  Its mixed-precision branch (:137-155, ``model_parameters``) includes the two routines of
+  apex.fp16_utils it calls, restated from their published behaviour (apex is a third-party dependency that
+  is not in the reference tree: model gradients copied into fp32 master gradients, masters copied back
+  into the 16-bit model); pinned by hand values in tests/test_oracle_optim.py.
+
 How each piece is pinned (tests/test_oracle_*.py): the truth table of
 runtime/tests/backprop/sgd_with_stashing.py:68-70 is reproduced on
 ``StashingOptimizerOracle``; the numpy optimizers are checked against the installed
