@@ -81,40 +81,71 @@ struct WinoArgs {
 // with wn = 0 / 1 load (lane = 32 * ((c % 8) / 4) + k % 32 holds four consecutive c).  Rows
 // k >= K of the last block of 64 are zero.  With rot180 the filter is taken as
 // f[k][r][s][c] = w[c][2-r][2-s][k] (w is then [C][3][3][K]): the input-gradient filter.
+//
+// One thread transforms the filters of one out channel and four consecutive in channels, so a wave is
+// one of those 1 KB halves and each of its 16 stores is one contiguous kilobyte.  The four waves of a
+// block take four neighbouring chunks where C allows, so that the block reads whole 128-byte lines of w.
+// vec: w is 16-byte aligned (128-bit loads along c).
+__device__ __forceinline__ float4 wf_half_sum(float4 a, float4 b, float4 c) {
+    return make_float4(0.5f * (a.x + b.x + c.x), 0.5f * (a.y + b.y + c.y), 0.5f * (a.z + b.z + c.z),
+                       0.5f * (a.w + b.w + c.w));
+}
+__device__ __forceinline__ float4 wf_half_alt(float4 a, float4 b, float4 c) {
+    return make_float4(0.5f * (a.x - b.x + c.x), 0.5f * (a.y - b.y + c.y), 0.5f * (a.z - b.z + c.z),
+                       0.5f * (a.w - b.w + c.w));
+}
+
 __global__ __launch_bounds__(256) void winograd_filter_kernel(const float* __restrict__ w, float* __restrict__ u,
-                                                              int K, int C, int k_pad, int rot180) {
-    const long id = (long)blockIdx.x * 256 + threadIdx.x;
-    if (id >= (long)k_pad * C) return;
-    int k, c;
-    if (rot180) { k = (int)(id % k_pad); c = (int)(id / k_pad); }
-    else { c = (int)(id % C); k = (int)(id / C); }
-    float g[3][3];
+                                                              int K, int C, int k_pad, int rot180, int vec) {
+    const int n_chunks = C / WG_CC;
+    const long unit = (long)blockIdx.x * 4 + threadIdx.x / 64;   // (block of 64 k, chunk, half of the block)
+    if (unit >= (long)(k_pad / 32) * n_chunks) return;
+    int half, chunk;
+    if (n_chunks % 4 == 0) {
+        chunk = (int)(unit % 4) + 4 * (int)((unit / 8) % (n_chunks / 4));
+        half = (int)((unit / 4) % 2);
+    } else {
+        half = (int)(unit % 2);
+        chunk = (int)((unit / 2) % n_chunks);
+    }
+    const int kb = (int)(unit / (2 * n_chunks));
+    const int lane = threadIdx.x % 64;
+    const int k = kb * WG_BN + half * 32 + lane % 32;
+    const int c0 = chunk * WG_CC + (lane / 32) * 4;
+    float4 g[3][3];
 #pragma unroll
     for (int r = 0; r < 3; ++r)
 #pragma unroll
         for (int s = 0; s < 3; ++s) {
-            float v = 0.f;
-            if (k < K) v = rot180 ? w[((size_t)c * 9 + (2 - r) * 3 + (2 - s)) * K + k]
-                                  : w[((size_t)k * 9 + r * 3 + s) * C + c];
+            float4 v = make_float4(0.f, 0.f, 0.f, 0.f);
+            if (k < K) {
+                if (rot180) {
+                    const float* src = w + ((size_t)c0 * 9 + (2 - r) * 3 + (2 - s)) * K + k;
+                    v = make_float4(src[0], src[(size_t)9 * K], src[(size_t)18 * K], src[(size_t)27 * K]);
+                } else {
+                    const float* src = w + ((size_t)k * 9 + r * 3 + s) * C + c0;
+                    if (vec) v = *reinterpret_cast<const float4*>(src);
+                    else v = make_float4(src[0], src[1], src[2], src[3]);
+                }
+            }
             g[r][s] = v;
         }
-    float t[4][3];
+    float4 t[4][3];
 #pragma unroll
     for (int s = 0; s < 3; ++s) {
         t[0][s] = g[0][s];
-        t[1][s] = 0.5f * (g[0][s] + g[1][s] + g[2][s]);
-        t[2][s] = 0.5f * (g[0][s] - g[1][s] + g[2][s]);
+        t[1][s] = wf_half_sum(g[0][s], g[1][s], g[2][s]);
+        t[2][s] = wf_half_alt(g[0][s], g[1][s], g[2][s]);
         t[3][s] = g[2][s];
     }
-    const int n_chunks = C / WG_CC;
-    const size_t base = ((size_t)((k / WG_BN) * n_chunks + c / WG_CC) * WG_G) * (2 * WG_FRAG) +
-                        ((k % WG_BN) / 32) * WG_FRAG + ((c % WG_CC) / 4) * 128 + (k % 32) * 4 + (c % 4);
+    float* dst = u + ((size_t)(kb * n_chunks + chunk) * WG_G) * (2 * WG_FRAG) + half * WG_FRAG + lane * 4;
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
-        const float o[4] = {t[i][0], 0.5f * (t[i][0] + t[i][1] + t[i][2]), 0.5f * (t[i][0] - t[i][1] + t[i][2]),
-                            t[i][2]};
+        const float4 o[4] = {t[i][0], wf_half_sum(t[i][0], t[i][1], t[i][2]),
+                             wf_half_alt(t[i][0], t[i][1], t[i][2]), t[i][2]};
 #pragma unroll
-        for (int m = 0; m < 4; ++m) u[base + (size_t)(i * 4 + m) * (2 * WG_FRAG)] = o[m];
+        for (int m = 0; m < 4; ++m)
+            *reinterpret_cast<float4*>(dst + (size_t)(i * 4 + m) * (2 * WG_FRAG)) = o[m];
     }
 }
 
@@ -581,9 +612,11 @@ extern "C" int pd_conv3x3_winograd_filter_f32(const float* w, float* u, int C, i
     PD_REQUIRE(w && u && w != u, PD_EINVAL, "pd_conv3x3_winograd_filter_f32: NULL or aliased pointer");
     PD_REQUIRE(C > 0 && K > 0 && wino_shape_ok(C, K), PD_ESHAPE,
                "pd_conv3x3_winograd_filter_f32: needs C %% 8 == 0 and K %% 4 == 0 (C=%d K=%d)", C, K);
+    PD_REQUIRE(pd_aligned(u, 16), PD_EINVAL, "pd_conv3x3_winograd_filter_f32: u must be 16-byte aligned");
     const int k_pad = (K + WG_BN - 1) / WG_BN * WG_BN;
-    const long total = (long)k_pad * C;
-    winograd_filter_kernel<<<(unsigned)((total + 255) / 256), 256, 0, (hipStream_t)stream>>>(w, u, K, C, k_pad, rot180);
+    const long units = (long)(k_pad / 32) * (C / WG_CC);   // one wave each
+    winograd_filter_kernel<<<(unsigned)((units + 3) / 4), 256, 0, (hipStream_t)stream>>>(
+        w, u, K, C, k_pad, rot180, pd_aligned(w, 16) ? 1 : 0);
     PD_CHECK_LAUNCH("pd_conv3x3_winograd_filter_f32");
     return PD_OK;
 }

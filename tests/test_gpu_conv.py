@@ -375,3 +375,40 @@ def test_conv_rejects_bad_operands():
         ops.conv3x3_forward(_nhwc(torch.randn(1, 5, 6, 6)), w)
     with pytest.raises(NotImplementedError):
         layers.Conv2d(4, 8, kernel_size=5, padding=2)
+
+
+@pytest.mark.parametrize("C,K", [(8, 4), (24, 36), (32, 64), (64, 100), (128, 128)])
+@pytest.mark.parametrize("rot180", [0, 1])
+@pytest.mark.parametrize("offset", [0, 1])
+def test_transformed_filter_layout_and_values(C, K, rot180, offset, conv_algorithm):
+    # U = G g G^T in fp64, placed by the documented order [k/64][c/8][g][(k%64)/32][(c%8)/4][k%32][c%4];
+    # rows k >= K of the last block of 64 must be zero.  offset 1: a filter that is only 4-byte aligned.
+    if conv_algorithm != "winograd":
+        pytest.skip("one algorithm is enough: the transform does not depend on it")
+    import ctypes
+
+    from pipedream_amd import _cabi
+    lib = _cabi.lib()
+    rng = np.random.RandomState(C * 1000 + K * 2 + rot180)
+    # memory order of the operand: [K][3][3][C], or with rot180 [C][3][3][K]
+    mem = rng.randn(*((C, 3, 3, K) if rot180 else (K, 3, 3, C)))
+    flat = torch.zeros(mem.size + 4, dtype=torch.float32).cuda()
+    wdev = flat[offset:offset + mem.size]
+    wdev.copy_(torch.tensor(mem.reshape(-1), dtype=torch.float32))
+    nbytes = ctypes.c_uint64()
+    lib.pd_conv3x3_winograd_filter_bytes(C, K, ctypes.byref(nbytes))
+    u = torch.full((nbytes.value // 4,), float("nan"), dtype=torch.float32).cuda()
+    lib.pd_conv3x3_winograd_filter_f32(wdev.data_ptr(), u.data_ptr(), C, K, rot180, _cabi.stream_ptr())
+    torch.cuda.synchronize()
+    mem32 = wdev.cpu().numpy().astype(np.float64).reshape(mem.shape)
+    # f[k][r][s][c]
+    f = mem32[:, ::-1, ::-1, :].transpose(3, 1, 2, 0) if rot180 else mem32
+    G = np.array([[1, 0, 0], [.5, .5, .5], [.5, -.5, .5], [0, 0, 1]])
+    U = np.einsum("ir,krsc,js->kcij", G, f, G).reshape(K, C, 16)
+    k_pad = (K + 63) // 64 * 64
+    want = np.zeros((k_pad // 64, C // 8, 16, 2, 2, 32, 4))
+    for k in range(K):
+        for c in range(C):
+            want[k // 64, c // 8, :, (k % 64) // 32, (c % 8) // 4, k % 32, c % 4] = U[k, c]
+    assert u.numel() == want.size
+    np.testing.assert_allclose(u.cpu().numpy().reshape(want.shape), want, rtol=1e-6, atol=1e-6)
