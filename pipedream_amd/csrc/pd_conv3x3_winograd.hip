@@ -70,6 +70,7 @@ struct WinoArgs {
     float* pool_y;          // pooling variant: [N,H/2,W/2,K], written instead of y
     uint8_t* pool_idx;      // pooling variant: [N,H/2,W/2,K] window position (bits 0-1) and sign (bit 2)
     int N, H, W, C, K;
+    int img_h;              // stacked variant: rows of one image (N is then 1 and H the rows of the whole batch)
     int relu;
     int tiles_x, tiles_y, k_blocks, n_chunks;
     int n_items, items_per_xcd;   // work items (pixel tile x channel block) in all / per die
@@ -181,7 +182,15 @@ __device__ __forceinline__ WinoItem wino_decode(const WinoArgs& a, int item) {
 //             last use.
 // One barrier per step.  After the last chunk of an item: output transform, cross-wave sum in LDS, bias,
 // ReLU, output mask and 128-bit NHWC stores.
-template <bool MASK, bool POOL>
+//
+// STACKED: the batch is taken as one image of N * img_h rows (NHWC images follow each other in memory
+// row after row), so that work items straddle images instead of padding every image to a multiple of
+// 16 rows.  img_h is even, hence no 2 x 2 tile straddles two images; a tile in the first (last) tile row
+// of an image must see zeros in the first (last) row of its 4 x 4 patch, where the stacked layout holds
+// the neighbouring image's row.  Only the threads that form row 0 (d0 - d2) resp. row 3 (d1 - d3) of
+// B^T d read those rows: for such a tile their row pointer goes to a patch of zeros in LDS (units 9 and
+// 10 of a halo row, which no piece is ever written to) -- set once per work item, nothing per step.
+template <bool MASK, bool POOL, bool STACKED>
 __global__ __launch_bounds__(WG_THREADS, 1) void winograd_fwd_kernel(const WinoArgs a) {
     __shared__ __attribute__((aligned(16))) float lds[WG_LDS_FLOATS];
 
@@ -265,13 +274,19 @@ __global__ __launch_bounds__(WG_THREADS, 1) void winograd_fwd_kernel(const WinoA
     const float sgn = ti == 1 ? 1.f : -1.f;
     const int unit0 = (cg * 2 * WG_HALO + 2 * (tt >> 3)) * WG_RAW_PITCH + (tt & 7);
     const int src_a = (unit0 + row_a * WG_RAW_PITCH) * 4, src_b = (unit0 + row_b * WG_RAW_PITCH) * 4;
+    // row offsets of the thread's tile in the i-th item of this block: src_a / src_b, or the zeros
+    auto patch_rows = [&](int i, int& oa, int& ob) {
+        oa = src_a;
+        ob = src_b;
+        if (STACKED && i < n_my) {
+            const int r0 = wino_decode(a, item0 + i * gx8).y0 + 2 * (tt >> 3);   // the tile's first output row
+            const int zeros = (cg * 2 * WG_HALO * WG_RAW_PITCH + 9) * 4;
+            if (ti == 0 && r0 % a.img_h == 0) oa = zeros;
+            if (ti == 3 && (r0 + 2) % a.img_h == 0) ob = zeros;
+        }
+    };
     float4_t t[4];
     float4_t dc[2][2];                         // column s of the patch waits in dc[s & 1] until its section
-    auto read_col = [&](const float* rs, int s) {
-        const int o = (((s & 1) * WG_HALO) * WG_RAW_PITCH + (s >> 1)) * 4;
-        dc[s & 1][0] = *(const float4_t*)(rs + src_a + o);
-        dc[s & 1][1] = *(const float4_t*)(rs + src_b + o);
-    };
     auto read_col_at = [&](const float* ra, const float* rb, int s) {   // the same through per-lane pointers
         const int o = (((s & 1) * WG_HALO) * WG_RAW_PITCH + (s >> 1)) * 4;
         dc[s & 1][0] = *(const float4_t*)(ra + o);
@@ -337,16 +352,41 @@ __global__ __launch_bounds__(WG_THREADS, 1) void winograd_fwd_kernel(const WinoA
     store_raw(1, 1);
     load_raw(l_cc);
     advance_l();
+    if (STACKED && tid < 64) {                 // the zeros: units 9 and 10 of row 0 of the 4 planes, both stages
+        const int stage = tid >> 5, plane = (tid >> 3) & 3, e = tid & 7;
+        lds[WG_RAW_OFF + stage * WG_RAW_STAGE + (plane * WG_HALO * WG_RAW_PITCH + 9) * 4 + e] = 0.f;
+    }
+    // patch rows of the step that stage 2 reads next: item p_i of this block, chunk p_cc
+    int p_i = 0, p_cc = 0;
+    const float* pra;
+    const float* prb;
+    auto set_patch_rows = [&](int stage) {
+        int oa, ob;
+        patch_rows(p_i, oa, ob);
+        pra = lds + WG_RAW_OFF + stage * WG_RAW_STAGE + oa;
+        prb = lds + WG_RAW_OFF + stage * WG_RAW_STAGE + ob;
+    };
+    auto advance_p = [&](int stage) {          // (pra, prb have just moved to that stage)
+        if (++p_cc == a.n_chunks) {
+            p_cc = 0;
+            ++p_i;
+            set_patch_rows(stage);
+        }
+    };
+    set_patch_rows(0);
     __syncthreads();
 #pragma unroll
-    for (int s = 0; s < 4; ++s) { read_col(lds + WG_RAW_OFF, s); transform_col(s); }
+    for (int s = 0; s < 4; ++s) { read_col_at(pra, prb, s); transform_col(s); }
 #pragma unroll
     for (int m = 0; m < 4; ++m) { transform_out(m); store_out(lds, m); }
     __syncthreads();
     float4_t af[2][2];                         // A fragments of GEMM pair p wait in af[p & 1] for one section
     af[0][0] = *(const float4_t*)(lds + a_lane);
     af[0][1] = *(const float4_t*)(lds + a_lane + (2 * WG_FRAG));
-    read_col(lds + WG_RAW_OFF + WG_RAW_STAGE, 0);
+    pra += WG_RAW_STAGE;                       // step 1 sits in the second stage
+    prb += WG_RAW_STAGE;
+    if (STACKED) advance_p(1);
+    read_col_at(pra, prb, 0);
 
     // Per step: four sections of 8 MFMAs (GEMM pair gp) each, every MFMA followed by a small piece of
     // the other stages' work; the scheduler may not move anything across the sub-step boundaries.  LDS
@@ -361,8 +401,7 @@ __global__ __launch_bounds__(WG_THREADS, 1) void winograd_fwd_kernel(const WinoA
     int dv = WG_V_STAGE, dr = WG_RAW_STAGE;    // signed distances to the other stage, flipped every step
     const float* pa = lds + a_lane;                                            // A fragments: stage q & 1
     float* pv = lds + WG_V_STAGE + ti * 4 * (2 * WG_FRAG) + twm * WG_FRAG + lane * 4;   // stage 2 output: (q+1) & 1
-    const float* pra = lds + WG_RAW_OFF + WG_RAW_STAGE + src_a;                // patch rows: (q+1) & 1
-    const float* prb = lds + WG_RAW_OFF + WG_RAW_STAGE + src_b;
+    // (pra, prb, the patch rows, point into stage (q+1) & 1)
     float* pw0 = lds + WG_RAW_OFF + raw_dst[0];                                // stage 1 output: q & 1
     float* pw1 = lds + WG_RAW_OFF + raw_dst[1];
     for (int m_i = 0; m_i < n_my; ++m_i) {
@@ -407,7 +446,11 @@ __global__ __launch_bounds__(WG_THREADS, 1) void winograd_fwd_kernel(const WinoA
                 if (gp == 1 && k == 4) store_raw_at(pw1, 1);
                 if (gp == 1 && k == 5) load_raw(l_cc);
                 // the pointers move to the other stage after their last use of the step
-                if (gp == 1 && k == 7) { pra -= dr; prb -= dr; }
+                if (gp == 1 && k == 7) {
+                    pra -= dr;
+                    prb -= dr;
+                    if (STACKED) advance_p(dr > 0 ? 0 : 1);
+                }
                 if (gp == 2 && k == 2) pw0 += dr;
                 if (gp == 2 && k == 4) pw1 += dr;
                 if (gp == 2 && k == 6) pa += dv;
@@ -637,12 +680,18 @@ int wino_fwd_launch(const char* who, const float* x, const float* u, const float
     a.x = x; a.u = u; a.bias = bias; a.mask = in_mask; a.out_mask = out_mask; a.y = y;
     a.pool_y = pool_y; a.pool_idx = pool_idx;
     a.N = N; a.H = H; a.W = W; a.C = C; a.K = K;
+    a.img_h = 0;
+    // images whose height is even but no multiple of the 16-row tile are stacked into one tall image
+    // (see the kernel): N * ceil(H / 16) tile rows become ceil(N * H / 16)
+    // (not with an input mask: that variant has no registers to spare for it)
+    const bool stacked = !in_mask && N > 1 && H % 2 == 0 && H % WG_PIX != 0 && (long)N * H * W * (C > K ? C : K) < (1L << 29);
+    if (stacked) { a.img_h = H; a.H = N * H; a.N = 1; }
     a.relu = relu != 0;
     a.tiles_x = (W + WG_PIX - 1) / WG_PIX;
-    a.tiles_y = (H + WG_PIX - 1) / WG_PIX;
+    a.tiles_y = (a.H + WG_PIX - 1) / WG_PIX;
     a.k_blocks = (K + WG_BN - 1) / WG_BN;
     a.n_chunks = C / WG_CC;
-    const long items = (long)N * a.tiles_x * a.tiles_y * a.k_blocks;
+    const long items = (long)a.N * a.tiles_x * a.tiles_y * a.k_blocks;
     PD_REQUIRE(items <= 0x7ffffff0L, PD_ESHAPE, "%s: too many tiles", who);
     a.n_items = (int)items;
     a.items_per_xcd = (int)((items + WG_XCD - 1) / WG_XCD);
@@ -655,9 +704,14 @@ int wino_fwd_launch(const char* who, const float* x, const float* u, const float
     if (blocks > (long)a.items_per_xcd * WG_XCD) blocks = (long)a.items_per_xcd * WG_XCD;
     dim3 grid((unsigned)blocks);
     hipStream_t s = (hipStream_t)stream;
-    if (a.pool_y) winograd_fwd_kernel<false, true><<<grid, WG_THREADS, 0, s>>>(a);
-    else if (in_mask) winograd_fwd_kernel<true, false><<<grid, WG_THREADS, 0, s>>>(a);
-    else winograd_fwd_kernel<false, false><<<grid, WG_THREADS, 0, s>>>(a);
+    if (stacked) {
+        if (a.pool_y) winograd_fwd_kernel<false, true, true><<<grid, WG_THREADS, 0, s>>>(a);
+        else winograd_fwd_kernel<false, false, true><<<grid, WG_THREADS, 0, s>>>(a);
+    } else {
+        if (a.pool_y) winograd_fwd_kernel<false, true, false><<<grid, WG_THREADS, 0, s>>>(a);
+        else if (in_mask) winograd_fwd_kernel<true, false, false><<<grid, WG_THREADS, 0, s>>>(a);
+        else winograd_fwd_kernel<false, false, false><<<grid, WG_THREADS, 0, s>>>(a);
+    }
     PD_CHECK_LAUNCH(who);
     return PD_OK;
 }

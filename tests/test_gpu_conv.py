@@ -412,3 +412,44 @@ def test_transformed_filter_layout_and_values(C, K, rot180, offset, conv_algorit
             want[k // 64, c // 8, :, (k % 64) // 32, (c % 8) // 4, k % 32, c % 4] = U[k, c]
     assert u.numel() == want.size
     np.testing.assert_allclose(u.cpu().numpy().reshape(want.shape), want, rtol=1e-6, atol=1e-6)
+
+
+@pytest.mark.parametrize("N,C,K,H,W", [(4, 8, 64, 6, 10),      # one reduction chunk: a new work item every step
+                                        (3, 16, 32, 14, 14),    # the last VGG16 block's images
+                                        (5, 24, 40, 22, 18),    # ragged in both directions, K % 64 != 0
+                                        (3, 32, 64, 28, 28),
+                                        (7, 8, 8, 2, 34),       # images of one tile row
+                                        (2, 16, 16, 56, 24)])
+def test_batch_of_images_whose_height_is_no_multiple_of_the_tile(N, C, K, H, W, conv_algorithm):
+    """Images of even height that is no multiple of 16 rows are processed as one tall image (work items
+    straddle images).  Nothing may leak across an image boundary: every image of the batch must come out
+    bit for bit as when it is convolved alone (a batch of one never takes that path), in the forward
+    pass, the pooled forward pass and the input gradient (plain and with the rectified-input mask).  The
+    batch is also checked against torch in fp64."""
+    if conv_algorithm != "winograd":
+        pytest.skip("a property of the Winograd kernels' work items")
+    torch.manual_seed(N * 100 + H)
+    x = _nhwc(torch.randn(N, C, H, W))
+    w = _nhwc(torch.randn(K, C, 3, 3) / math.sqrt(9 * C))
+    b = torch.randn(K).cuda()
+    dy = _nhwc(torch.randn(N, K, H, W))
+
+    def one(t, n):
+        return t[n:n + 1].contiguous(memory_format=torch.channels_last)
+
+    y = ops.conv3x3_forward(x, w, b, relu=True)
+    yp, idx = ops.conv3x3_forward_pool(x, w, b, relu=True)
+    dx = ops.conv3x3_input_grad(dy, w)
+    dxm = ops.conv3x3_input_grad(dy, w, x_rectified=x)
+    for n in range(N):
+        assert torch.equal(y[n], ops.conv3x3_forward(one(x, n), w, b, relu=True)[0]), n
+        yp1, idx1 = ops.conv3x3_forward_pool(one(x, n), w, b, relu=True)
+        assert torch.equal(yp[n], yp1[0]) and torch.equal(idx[n], idx1[0]), n
+        assert torch.equal(dx[n], ops.conv3x3_input_grad(one(dy, n), w)[0]), n
+        assert torch.equal(dxm[n], ops.conv3x3_input_grad(one(dy, n), w, x_rectified=one(x, n))[0]), n
+    xd = x.cpu().double().requires_grad_(True)
+    ref = F.conv2d(xd, w.cpu().double(), b.cpu().double(), padding=1)
+    torch.testing.assert_close(y.cpu().double(), F.relu(ref).detach(), rtol=1e-5, atol=2e-5)
+    torch.testing.assert_close(yp.cpu().double(), F.max_pool2d(F.relu(ref), 2, 2).detach(), rtol=1e-5, atol=2e-5)
+    ref.backward(dy.cpu().double())
+    torch.testing.assert_close(dx.cpu().double(), xd.grad, rtol=1e-5, atol=2e-5)
