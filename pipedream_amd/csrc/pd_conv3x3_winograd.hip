@@ -28,6 +28,8 @@
 //     waves that share a (tiles, channels) block each apply the output transform A^T M A to their
 //     rows of M (it is linear) and the partial results are added in the LDS staging tile; bias, ReLU
 //     and the optional output mask follow as the tile is stored as whole NHWC pixel rows.
+#include <type_traits>
+
 #include "pd_internal.h"
 
 namespace {
@@ -481,9 +483,11 @@ __global__ __launch_bounds__(WG_THREADS, 1) void winograd_fwd_kernel(const WinoA
             auto stg_index = [&](int e, int i) {
                 return ((2 * (e / 4) + (i >> 1)) * WG_PIX + 2 * (e % 4) + (i & 1)) * WG_OP;
             };
-            auto out_rows = [&](bool add) {
+            auto out_rows = [&](auto first_row, auto upper_rows, bool add) {
+                constexpr int E0 = decltype(first_row)::value;
+                constexpr bool UPPER = decltype(upper_rows)::value;    // this wave holds rows 2, 3 of M (gh = 1)
 #pragma unroll
-                for (int e = 0; e < 16; ++e) {
+                for (int e = E0; e < E0 + 8; ++e) {
                     // the accumulators stay in the accumulation registers until the row that needs them
                     // (read through an explicit instruction: the register allocator would otherwise
                     // move all of them to ordinary registers at once)
@@ -496,8 +500,8 @@ __global__ __launch_bounds__(WG_THREADS, 1) void winograd_fwd_kernel(const WinoA
                     for (int m = 0; m < 4; ++m) {
                         // rows (M0, M1) of M for gh = 0, rows (M2, M3) for gh = 1:
                         // A^T = [1 1 1 0; 0 1 -1 -1] applied to the rows this wave holds
-                        s0[m] = add ? mv[m] : mv[m] + mv[4 + m];
-                        s1[m] = add ? -mv[m] - mv[4 + m] : mv[4 + m];
+                        s0[m] = UPPER ? mv[m] : mv[m] + mv[4 + m];
+                        s1[m] = UPPER ? -mv[m] - mv[4 + m] : mv[4 + m];
                     }
                     const float part[4] = {s0[0] + s0[1] + s0[2], s0[1] - s0[2] - s0[3], s1[0] + s1[1] + s1[2],
                                            s1[1] - s1[2] - s1[3]};
@@ -545,10 +549,29 @@ __global__ __launch_bounds__(WG_THREADS, 1) void winograd_fwd_kernel(const WinoA
                     for (int c = 0; c < 4; ++c) mbits |= (mk[it][c] > 0.f ? 1u : 0u) << (it * 4 + c);
             };
             if (!POOL && a.out_mask && gh == 1) fetch_mask();
-            if (gh == 0) out_rows(false);
+            // bias of the thread's four channels for the store phase (k4 is the same there and in the pooling
+            // variant): requested at the start of the second summation phase, which hides the round trip;
+            // channels past K (and a null bias, as a buffer of size 0) read 0
+            float4_t b4;
+            auto load_bias = [&]() {
+                const __amdgpu_buffer_rsrc_t br = __builtin_amdgcn_make_buffer_rsrc(
+                    (void*)a.bias, 0, a.bias ? (uint32_t)a.K * 4 : 0u, 0x00020000);
+#pragma unroll
+                for (int c = 0; c < 4; ++c)
+                    b4[c] = __builtin_bit_cast(
+                        float, __builtin_amdgcn_raw_buffer_load_b32(br, (uint32_t)(k0 + k4 + c) * 4, 0, 0));
+            };
+            using std::integral_constant;
+            if (gh == 0) out_rows(integral_constant<int, 0>{}, integral_constant<bool, false>{}, false);
+            else out_rows(integral_constant<int, 8>{}, integral_constant<bool, true>{}, false);
             __syncthreads();
-            if (gh == 1) out_rows(true);
-            else if (!POOL && a.out_mask) fetch_mask();
+            load_bias();
+            if (gh == 0) {
+                if (!POOL && a.out_mask) fetch_mask();
+                out_rows(integral_constant<int, 8>{}, integral_constant<bool, false>{}, true);
+            } else {
+                out_rows(integral_constant<int, 0>{}, integral_constant<bool, true>{}, true);
+            }
             __syncthreads();
             if constexpr (POOL) {
                 // 2x2 max pooling of the tile (bias and ReLU first), written with one index byte per element
@@ -557,12 +580,7 @@ __global__ __launch_bounds__(WG_THREADS, 1) void winograd_fwd_kernel(const WinoA
                 // (tid >> 4) & 7, pooled rows (tid >> 7) + 4 it; tiles start at even pixels, so no window
                 // straddles two tiles.
                 const int Hp = a.H >> 1, Wp = a.W >> 1;
-                const int k4 = (tid & 15) * 4, pc = (tid >> 4) & 7, pr0 = tid >> 7;
-                float4_t b4 = {0.f, 0.f, 0.f, 0.f};
-                if (a.bias) {
-#pragma unroll
-                    for (int c = 0; c < 4; ++c) b4[c] = k0 + k4 + c < a.K ? a.bias[k0 + k4 + c] : 0.f;
-                }
+                const int pc = (tid >> 4) & 7, pr0 = tid >> 7;
                 const size_t pimg = (size_t)w.n * Hp * Wp * a.K;
                 const uint32_t pool_elems = (uint32_t)Hp * Wp * a.K;
                 const __amdgpu_buffer_rsrc_t pyr =
@@ -607,28 +625,43 @@ __global__ __launch_bounds__(WG_THREADS, 1) void winograd_fwd_kernel(const WinoA
                 // (tid >> 4) & 15, channels k4..k4+3, pixel rows (tid >> 8) + 2 it: one base offset, a scalar
                 // stride per row pair.  Pixels outside the image get an offset beyond the buffer's size: such a
                 // store is dropped.
-                float4_t b4 = {0.f, 0.f, 0.f, 0.f};
-                if (a.bias) {
-    #pragma unroll
-                    for (int c = 0; c < 4; ++c) b4[c] = k0 + k4 + c < a.K ? a.bias[k0 + k4 + c] : 0.f;
-                }
+                // The loop exists once per (ReLU, mask) combination: with the two tests inside it every
+                // iteration would wait for its own LDS read.
                 const __amdgpu_buffer_rsrc_t yr =
                     __builtin_amdgcn_make_buffer_rsrc((void*)(a.y + oimg), 0, out_bytes, 0x00020000);
                 const float* src = stg + (prow * WG_PIX + pcol) * WG_OP + k4;
+                auto store_rows = [&](auto with_relu, auto with_mask) {
+                    constexpr bool RELU = decltype(with_relu)::value, MASKED = decltype(with_mask)::value;
     #pragma unroll
-                for (int it = 0; it < NV; ++it) {
-                    const uint32_t voff = (col_ok && w.y0 + prow + 2 * it < a.H) ? obase : 0x80000000u;
-                    float4_t v = *(const float4_t*)(src + it * 2 * WG_PIX * WG_OP) + b4;
-                    if (a.relu) {
+                    for (int it = 0; it < NV; ++it) {
+                        // The row offset is added to the vector offset, not passed as the scalar one: after a
+                        // 128-bit buffer store with a register as scalar offset the compiler schedules vector
+                        // writes to the store's data registers with no wait state, and on this part the first
+                        // dword of the stored rows then came out overwritten (lanes 12-15 of every 16).  With an
+                        // immediate scalar offset it inserts the wait state itself.
+                        const uint32_t voff = ((col_ok && w.y0 + prow + 2 * it < a.H) ? obase : 0x80000000u) +
+                                              (uint32_t)(it * row_stride);
+                        float4_t v = *(const float4_t*)(src + it * 2 * WG_PIX * WG_OP) + b4;
+                        if (RELU) {
     #pragma unroll
-                        for (int c = 0; c < 4; ++c) v[c] = v[c] > 0.f ? v[c] : 0.f;
+                            for (int c = 0; c < 4; ++c) v[c] = v[c] > 0.f ? v[c] : 0.f;
+                        }
+                        if (MASKED) {
+    #pragma unroll
+                            for (int c = 0; c < 4; ++c) v[c] = (mbits >> (it * 4 + c)) & 1u ? v[c] : 0.f;
+                        }
+                        typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+                        __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(u32x4, v), yr, voff, 0, 2);
                     }
-                    if (a.out_mask) {
-    #pragma unroll
-                        for (int c = 0; c < 4; ++c) v[c] = (mbits >> (it * 4 + c)) & 1u ? v[c] : 0.f;
-                    }
-                    typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
-                    __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(u32x4, v), yr, voff, it * row_stride, 2);
+                };
+                using yes = integral_constant<bool, true>;
+                using no = integral_constant<bool, false>;
+                if (a.relu) {
+                    if (a.out_mask) store_rows(yes{}, yes{});
+                    else store_rows(yes{}, no{});
+                } else {
+                    if (a.out_mask) store_rows(no{}, yes{});
+                    else store_rows(no{}, no{});
                 }
             }
         }
