@@ -17,11 +17,17 @@ typedef float float4_t __attribute__((ext_vector_type(4)));
 namespace {
 
 constexpr int LSTM_THREADS = 256;
+constexpr long LSTM_SCALAR_UNITS = 1L << 19;   // up to here (batch x hidden units) the cell kernels take one unit per thread
 
 __device__ __forceinline__ float sigmoidf_(float x) { return 1.0f / (1.0f + expf(-x)); }
 
 // gates: [B][4H] pre-activations (x W_ih^T + h W_hh^T), overwritten with the ACTIVATED
-// gates i,f,g,o which the backward pass needs.  One thread = 4 consecutive hidden units.
+// gates i,f,g,o which the backward pass needs.  One thread = V consecutive hidden units: 4 (128-bit
+// accesses) for large batches; 1 at the recurrence's own size (batch 128 x 1024 units), where four units
+// per thread leave two waves per CU, each with some twenty transcendental evaluations in a row -- the
+// kernel is then bound by one wave's instruction latency, not by memory.  Every unit sees the same
+// operations in the same order either way.
+template <int V>
 __global__ __launch_bounds__(LSTM_THREADS) void lstm_cell_fwd_kernel(float* __restrict__ gates,
                                                                      const float* __restrict__ rec, int n_rec,
                                                                      const float* __restrict__ b_ih,
@@ -29,28 +35,29 @@ __global__ __launch_bounds__(LSTM_THREADS) void lstm_cell_fwd_kernel(float* __re
                                                                      const float* __restrict__ c_prev,
                                                                      float* __restrict__ c_out,
                                                                      float* __restrict__ h_out, int B, int H) {
-    const int H4 = H / 4;
+    typedef float vec_t __attribute__((ext_vector_type(V)));
+    const int HV = H / V;
     const int id = blockIdx.x * LSTM_THREADS + threadIdx.x;
-    if (id >= B * H4) return;
-    const int b = id / H4, j = (id % H4) * 4;
+    if (id >= B * HV) return;
+    const int b = id / HV, j = (id % HV) * V;
     float* g = gates + (size_t)b * 4 * H;
-    float4_t gi = *(const float4_t*)(g + j);
-    float4_t gf = *(const float4_t*)(g + H + j);
-    float4_t gg = *(const float4_t*)(g + 2 * H + j);
-    float4_t go = *(const float4_t*)(g + 3 * H + j);
+    vec_t gi = *(const vec_t*)(g + j);
+    vec_t gf = *(const vec_t*)(g + H + j);
+    vec_t gg = *(const vec_t*)(g + 2 * H + j);
+    vec_t go = *(const vec_t*)(g + 3 * H + j);
     // split-k partial sums of h_{t-1} W_hh^T, added in a fixed order, four partials (16 loads) in flight at
     // a time: one at a time the loop is a chain of round trips to memory
     for (int s0 = 0; s0 < n_rec; s0 += 4) {
-        float4_t p[4][4];
+        vec_t p[4][4];
 #pragma unroll
         for (int u = 0; u < 4; ++u) {
             const bool live = s0 + u < n_rec;
             const float* r = rec + ((size_t)(live ? s0 + u : s0) * B + b) * 4 * H;
 #pragma unroll
-            for (int q = 0; q < 4; ++q) p[u][q] = *(const float4_t*)(r + q * H + j);
+            for (int q = 0; q < 4; ++q) p[u][q] = *(const vec_t*)(r + q * H + j);
             if (!live) {
 #pragma unroll
-                for (int q = 0; q < 4; ++q) p[u][q] = float4_t{0.f, 0.f, 0.f, 0.f};
+                for (int q = 0; q < 4; ++q) p[u][q] = vec_t(0.f);
             }
         }
         gi += (p[0][0] + p[1][0]) + (p[2][0] + p[3][0]);
@@ -59,16 +66,16 @@ __global__ __launch_bounds__(LSTM_THREADS) void lstm_cell_fwd_kernel(float* __re
         go += (p[0][3] + p[1][3]) + (p[2][3] + p[3][3]);
     }
     if (b_ih) {
-        gi += *(const float4_t*)(b_ih + j) + *(const float4_t*)(b_hh + j);
-        gf += *(const float4_t*)(b_ih + H + j) + *(const float4_t*)(b_hh + H + j);
-        gg += *(const float4_t*)(b_ih + 2 * H + j) + *(const float4_t*)(b_hh + 2 * H + j);
-        go += *(const float4_t*)(b_ih + 3 * H + j) + *(const float4_t*)(b_hh + 3 * H + j);
+        gi += *(const vec_t*)(b_ih + j) + *(const vec_t*)(b_hh + j);
+        gf += *(const vec_t*)(b_ih + H + j) + *(const vec_t*)(b_hh + H + j);
+        gg += *(const vec_t*)(b_ih + 2 * H + j) + *(const vec_t*)(b_hh + 2 * H + j);
+        go += *(const vec_t*)(b_ih + 3 * H + j) + *(const vec_t*)(b_hh + 3 * H + j);
     }
-    float4_t cp = {0.f, 0.f, 0.f, 0.f};
-    if (c_prev) cp = *(const float4_t*)(c_prev + (size_t)b * H + j);
-    float4_t c, h;
+    vec_t cp = vec_t(0.f);
+    if (c_prev) cp = *(const vec_t*)(c_prev + (size_t)b * H + j);
+    vec_t c, h;
 #pragma unroll
-    for (int k = 0; k < 4; ++k) {
+    for (int k = 0; k < V; ++k) {
         gi[k] = sigmoidf_(gi[k]);
         gf[k] = sigmoidf_(gf[k]);
         gg[k] = tanhf(gg[k]);
@@ -76,16 +83,17 @@ __global__ __launch_bounds__(LSTM_THREADS) void lstm_cell_fwd_kernel(float* __re
         c[k] = gf[k] * cp[k] + gi[k] * gg[k];
         h[k] = go[k] * tanhf(c[k]);
     }
-    *(float4_t*)(g + j) = gi;
-    *(float4_t*)(g + H + j) = gf;
-    *(float4_t*)(g + 2 * H + j) = gg;
-    *(float4_t*)(g + 3 * H + j) = go;
-    *(float4_t*)(c_out + (size_t)b * H + j) = c;
-    *(float4_t*)(h_out + (size_t)b * H + j) = h;
+    *(vec_t*)(g + j) = gi;
+    *(vec_t*)(g + H + j) = gf;
+    *(vec_t*)(g + 2 * H + j) = gg;
+    *(vec_t*)(g + 3 * H + j) = go;
+    *(vec_t*)(c_out + (size_t)b * H + j) = c;
+    *(vec_t*)(h_out + (size_t)b * H + j) = h;
 }
 
 // dh = dy (+ dh_rec); dc = dc_next + dh*o*(1-tanh(c)^2); dgates are gradients with respect
 // to the pre-activations; dc_next is overwritten with the gradient for c_prev.
+template <int V>
 __global__ __launch_bounds__(LSTM_THREADS) void lstm_cell_bwd_kernel(const float* __restrict__ gates,
                                                                      const float* __restrict__ c_prev,
                                                                      const float* __restrict__ c,
@@ -94,38 +102,39 @@ __global__ __launch_bounds__(LSTM_THREADS) void lstm_cell_bwd_kernel(const float
                                                                      float* __restrict__ dc_io,
                                                                      float* __restrict__ dgates, int B, int H,
                                                                      int first_step) {
-    const int H4 = H / 4;
+    typedef float vec_t __attribute__((ext_vector_type(V)));
+    const int HV = H / V;
     const int id = blockIdx.x * LSTM_THREADS + threadIdx.x;
-    if (id >= B * H4) return;
-    const int b = id / H4, j = (id % H4) * 4;
+    if (id >= B * HV) return;
+    const int b = id / HV, j = (id % HV) * V;
     const float* g = gates + (size_t)b * 4 * H;
-    const float4_t gi = *(const float4_t*)(g + j);
-    const float4_t gf = *(const float4_t*)(g + H + j);
-    const float4_t gg = *(const float4_t*)(g + 2 * H + j);
-    const float4_t go = *(const float4_t*)(g + 3 * H + j);
+    const vec_t gi = *(const vec_t*)(g + j);
+    const vec_t gf = *(const vec_t*)(g + H + j);
+    const vec_t gg = *(const vec_t*)(g + 2 * H + j);
+    const vec_t go = *(const vec_t*)(g + 3 * H + j);
     const size_t o = (size_t)b * H + j;
-    float4_t cp = {0.f, 0.f, 0.f, 0.f};
-    if (c_prev) cp = *(const float4_t*)(c_prev + o);
-    const float4_t ct = *(const float4_t*)(c + o);
-    float4_t dh = *(const float4_t*)(dy + o);
+    vec_t cp = vec_t(0.f);
+    if (c_prev) cp = *(const vec_t*)(c_prev + o);
+    const vec_t ct = *(const vec_t*)(c + o);
+    vec_t dh = *(const vec_t*)(dy + o);
     if (dh_rec) {
         // the split-k partial sums of dgates W_hh, eight loads in flight at a time, added in a fixed order
         for (int s0 = 0; s0 < n_rec; s0 += 8) {
-            float4_t p[8];
+            vec_t p[8];
 #pragma unroll
             for (int u = 0; u < 8; ++u) {
                 const bool live = s0 + u < n_rec;
-                p[u] = *(const float4_t*)(dh_rec + (size_t)(live ? s0 + u : s0) * B * H + o);
-                if (!live) p[u] = float4_t{0.f, 0.f, 0.f, 0.f};
+                p[u] = *(const vec_t*)(dh_rec + (size_t)(live ? s0 + u : s0) * B * H + o);
+                if (!live) p[u] = vec_t(0.f);
             }
             dh += ((p[0] + p[1]) + (p[2] + p[3])) + ((p[4] + p[5]) + (p[6] + p[7]));
         }
     }
-    float4_t dc = {0.f, 0.f, 0.f, 0.f};
-    if (!first_step) dc = *(const float4_t*)(dc_io + o);
-    float4_t di, df, dg, dO, dcp;
+    vec_t dc = vec_t(0.f);
+    if (!first_step) dc = *(const vec_t*)(dc_io + o);
+    vec_t di, df, dg, dO, dcp;
 #pragma unroll
-    for (int k = 0; k < 4; ++k) {
+    for (int k = 0; k < V; ++k) {
         const float tc = tanhf(ct[k]);
         const float dck = dc[k] + dh[k] * go[k] * (1.0f - tc * tc);
         dO[k] = dh[k] * tc * go[k] * (1.0f - go[k]);
@@ -135,11 +144,11 @@ __global__ __launch_bounds__(LSTM_THREADS) void lstm_cell_bwd_kernel(const float
         dcp[k] = dck * gf[k];
     }
     float* d = dgates + (size_t)b * 4 * H;
-    *(float4_t*)(d + j) = di;
-    *(float4_t*)(d + H + j) = df;
-    *(float4_t*)(d + 2 * H + j) = dg;
-    *(float4_t*)(d + 3 * H + j) = dO;
-    *(float4_t*)(dc_io + o) = dcp;
+    *(vec_t*)(d + j) = di;
+    *(vec_t*)(d + H + j) = df;
+    *(vec_t*)(d + 2 * H + j) = dg;
+    *(vec_t*)(d + 3 * H + j) = dO;
+    *(vec_t*)(dc_io + o) = dcp;
 }
 
 // y = a + b  (the residual connections between LSTM layers)
@@ -215,9 +224,15 @@ extern "C" int pd_lstm_cell_fwd_f32(float* gates, const float* rec, int n_rec, c
     PD_REQUIRE(pd_aligned(gates, 16) && pd_aligned(c_out, 16) && pd_aligned(h_out, 16) &&
                    (!c_prev || pd_aligned(c_prev, 16)) && (!b_ih || (pd_aligned(b_ih, 16) && pd_aligned(b_hh, 16))),
                PD_EINVAL, "pd_lstm_cell_fwd_f32: pointers must be 16-byte aligned");
-    const int total = B * (H / 4);
-    lstm_cell_fwd_kernel<<<dim3((total + LSTM_THREADS - 1) / LSTM_THREADS), dim3(LSTM_THREADS), 0,
-                           (hipStream_t)stream>>>(gates, rec, n_rec, b_ih, b_hh, c_prev, c_out, h_out, B, H);
+    if ((long)B * H <= LSTM_SCALAR_UNITS) {
+        const int total = B * H;
+        lstm_cell_fwd_kernel<1><<<dim3((total + LSTM_THREADS - 1) / LSTM_THREADS), dim3(LSTM_THREADS), 0,
+                                  (hipStream_t)stream>>>(gates, rec, n_rec, b_ih, b_hh, c_prev, c_out, h_out, B, H);
+    } else {
+        const int total = B * (H / 4);
+        lstm_cell_fwd_kernel<4><<<dim3((total + LSTM_THREADS - 1) / LSTM_THREADS), dim3(LSTM_THREADS), 0,
+                                  (hipStream_t)stream>>>(gates, rec, n_rec, b_ih, b_hh, c_prev, c_out, h_out, B, H);
+    }
     PD_CHECK_LAUNCH("pd_lstm_cell_fwd_f32");
     return PD_OK;
 }
@@ -231,9 +246,17 @@ extern "C" int pd_lstm_cell_bwd_f32(const float* gates, const float* c_prev, con
     PD_REQUIRE(pd_aligned(gates, 16) && pd_aligned(c, 16) && pd_aligned(dy, 16) && pd_aligned(dc_io, 16) &&
                    pd_aligned(dgates, 16) && (!c_prev || pd_aligned(c_prev, 16)) && (!dh_rec || pd_aligned(dh_rec, 16)),
                PD_EINVAL, "pd_lstm_cell_bwd_f32: pointers must be 16-byte aligned");
-    const int total = B * (H / 4);
-    lstm_cell_bwd_kernel<<<dim3((total + LSTM_THREADS - 1) / LSTM_THREADS), dim3(LSTM_THREADS), 0,
-                           (hipStream_t)stream>>>(gates, c_prev, c, dy, dh_rec, n_rec, dc_io, dgates, B, H, first_step);
+    if ((long)B * H <= LSTM_SCALAR_UNITS) {
+        const int total = B * H;
+        lstm_cell_bwd_kernel<1><<<dim3((total + LSTM_THREADS - 1) / LSTM_THREADS), dim3(LSTM_THREADS), 0,
+                                  (hipStream_t)stream>>>(gates, c_prev, c, dy, dh_rec, n_rec, dc_io, dgates, B, H,
+                                                         first_step);
+    } else {
+        const int total = B * (H / 4);
+        lstm_cell_bwd_kernel<4><<<dim3((total + LSTM_THREADS - 1) / LSTM_THREADS), dim3(LSTM_THREADS), 0,
+                                  (hipStream_t)stream>>>(gates, c_prev, c, dy, dh_rec, n_rec, dc_io, dgates, B, H,
+                                                         first_step);
+    }
     PD_CHECK_LAUNCH("pd_lstm_cell_bwd_f32");
     return PD_OK;
 }
