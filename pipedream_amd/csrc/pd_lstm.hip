@@ -175,32 +175,44 @@ __global__ __launch_bounds__(LSTM_THREADS) void embedding_fwd_kernel(const int64
 
 // dweight[v][:] = sum over positions p with ids[p] == v of dout[p][:], positions in
 // increasing order (deterministic, no atomics); rows without a hit and the padding row
-// are written as zeros, so dweight needs no prior clearing.  One block per vocabulary row;
-// the ids are scanned 64 at a time with a ballot.
+// are zeros.  Two launches: a fill with zeros, then one block per token position: the block
+// of the first position that holds a row's id sums all of that row's positions, every other
+// block leaves as soon as it meets an earlier position with its id (one scan of the ids per
+// position, 64 at a time with a ballot, instead of one per vocabulary row).
+__global__ __launch_bounds__(LSTM_THREADS) void zero_fill_kernel(float4_t* __restrict__ dst, size_t n4) {
+    const size_t i = (size_t)blockIdx.x * LSTM_THREADS + threadIdx.x;
+    if (i < n4) dst[i] = float4_t{0.f, 0.f, 0.f, 0.f};
+}
+
 __global__ __launch_bounds__(LSTM_THREADS) void embedding_bwd_kernel(const int64_t* __restrict__ ids,
                                                                      const float* __restrict__ dout,
                                                                      float* __restrict__ dweight, int n_tokens, int D,
-                                                                     int64_t padding_idx) {
-    const int64_t v = blockIdx.x;
+                                                                     int64_t V, int64_t padding_idx) {
+    const int me = blockIdx.x;
+    const int64_t v = ids[me];
+    if (v < 0 || v >= V || v == padding_idx) return;
     const int lane = threadIdx.x % 64;
     // every thread owns D/(4*256) float4 columns; D <= 4096 supported by the accumulators below
     float4_t acc[4];
 #pragma unroll
     for (int r = 0; r < 4; ++r) acc[r] = (float4_t){0.f, 0.f, 0.f, 0.f};
-    if (v != padding_idx) {
-        for (int p0 = 0; p0 < n_tokens; p0 += 64) {
-            const int p = p0 + lane;
-            const bool hit = p < n_tokens && ids[p] == v;
-            unsigned long long m = __ballot(hit);
-            while (m) {
-                const int bit = __ffsll((long long)m) - 1;
-                m &= m - 1;
-                const float* src = dout + (size_t)(p0 + bit) * D;
+    bool owner = false;                        // the same in every thread of the block
+    for (int p0 = 0; p0 < n_tokens; p0 += 64) {
+        const int p = p0 + lane;
+        const bool hit = p < n_tokens && ids[p] == v;
+        unsigned long long m = __ballot(hit);
+        if (!owner && m) {
+            if (p0 + __ffsll((long long)m) - 1 != me) return;   // an earlier position owns this row
+            owner = true;
+        }
+        while (m) {
+            const int bit = __ffsll((long long)m) - 1;
+            m &= m - 1;
+            const float* src = dout + (size_t)(p0 + bit) * D;
 #pragma unroll
-                for (int r = 0; r < 4; ++r) {
-                    const int j = (r * LSTM_THREADS + threadIdx.x) * 4;
-                    if (j < D) acc[r] += *(const float4_t*)(src + j);
-                }
+            for (int r = 0; r < 4; ++r) {
+                const int j = (r * LSTM_THREADS + threadIdx.x) * 4;
+                if (j < D) acc[r] += *(const float4_t*)(src + j);
             }
         }
     }
@@ -290,8 +302,14 @@ extern "C" int pd_embedding_bwd_f32(const int64_t* ids, const float* dout, float
                "pd_embedding_bwd_f32: need D a multiple of 4 in (0, 4096] and 0 < V < 2^31");
     PD_REQUIRE(dweight && (n_tokens == 0 || (ids && dout)), PD_EINVAL, "pd_embedding_bwd_f32: NULL pointer");
     PD_REQUIRE(pd_aligned(dweight, 16) && pd_aligned(dout, 16), PD_EINVAL, "pd_embedding_bwd_f32: 16-byte alignment");
-    embedding_bwd_kernel<<<dim3((unsigned)V), dim3(LSTM_THREADS), 0, (hipStream_t)stream>>>(ids, dout, dweight,
-                                                                                          n_tokens, D, padding_idx);
+    const size_t n4 = (size_t)V * D / 4;
+    PD_REQUIRE(n4 / LSTM_THREADS < 0x7fffffffull, PD_ESHAPE, "pd_embedding_bwd_f32: table too large");
+    zero_fill_kernel<<<dim3((unsigned)((n4 + LSTM_THREADS - 1) / LSTM_THREADS)), dim3(LSTM_THREADS), 0,
+                       (hipStream_t)stream>>>((float4_t*)dweight, n4);
+    PD_CHECK_LAUNCH("pd_embedding_bwd_f32");
+    if (n_tokens > 0)
+        embedding_bwd_kernel<<<dim3((unsigned)n_tokens), dim3(LSTM_THREADS), 0, (hipStream_t)stream>>>(
+            ids, dout, dweight, n_tokens, D, V, padding_idx);
     PD_CHECK_LAUNCH("pd_embedding_bwd_f32");
     return PD_OK;
 }

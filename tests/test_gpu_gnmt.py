@@ -120,3 +120,25 @@ def test_full_size_gnmt_stage_forward_backward():
     grads = dict((k, p.grad) for k, p in mine.named_parameters())
     for k, p in ref.named_parameters():
         assert _rel(grads[k], p.grad) < 2e-5, (k, _rel(grads[k], p.grad))
+
+
+def test_embedding_gradient_sums_duplicates_in_position_order():
+    # 1500 positions over 40 rows of 1280 columns (more than one pass of the block over the columns), ids that
+    # are out of range or the padding row contribute nothing, every other row is the fp32 sum of its positions
+    # taken in increasing order: bit for bit, and rows without a position are zero
+    from pipedream_amd import ops
+    torch.manual_seed(5)
+    V, D, n = 40, 1280, 1500
+    ids = torch.randint(0, 30, (n,))
+    ids[::97] = 3                      # padding row
+    ids[5] = -1
+    ids[6] = V + 2
+    dout = torch.randn(n, D)
+    got = ops.embedding_backward(ids.cuda(), dout.cuda(), V, padding_idx=3).cpu()
+    want = torch.zeros(V, D)
+    for p in range(n):
+        v = int(ids[p])
+        if 0 <= v < V and v != 3:
+            want[v] += dout[p]
+    assert torch.equal(got, want)
+    assert not got[30:].any() and not got[3].any()
