@@ -589,6 +589,10 @@ __global__ __launch_bounds__(WG_THREADS, 1) void winograd_fwd_kernel(const WinoA
                     __builtin_amdgcn_make_buffer_rsrc((void*)(a.pool_idx + pimg), 0, pool_elems, 0x00020000);
                 const int py0 = w.y0 >> 1, px0 = w.x0 >> 1;
                 const bool col_ok = px0 + pc < Wp && k0 + k4 < a.K;
+                // (once per ReLU setting: no test of a run-time flag per element, and selects instead of
+                // branches for the running maximum)
+                auto pool_rows = [&](auto with_relu) {
+                constexpr bool RELU = decltype(with_relu)::value;
 #pragma unroll
                 for (int it = 0; it < 2; ++it) {
                     const int pr = pr0 + 4 * it;
@@ -606,12 +610,15 @@ __global__ __launch_bounds__(WG_THREADS, 1) void winograd_fwd_kernel(const WinoA
                     for (int c = 0; c < 4; ++c) {
                         float q[4];
 #pragma unroll
-                        for (int j = 0; j < 4; ++j) q[j] = (a.relu && !(v[j][c] > 0.f)) ? 0.f : v[j][c];   // as the plain epilogue
+                        for (int j = 0; j < 4; ++j) q[j] = (RELU && !(v[j][c] > 0.f)) ? 0.f : v[j][c];   // as the plain epilogue
                         float b = q[0];
                         uint32_t arg = 0;
 #pragma unroll
-                        for (int j = 1; j < 4; ++j)
-                            if (q[j] > b || q[j] != q[j]) { b = q[j]; arg = j; }
+                        for (int j = 1; j < 4; ++j) {
+                            const bool take = q[j] > b || q[j] != q[j];
+                            b = take ? q[j] : b;
+                            arg = take ? (uint32_t)j : arg;
+                        }
                         best[c] = b;
                         packed |= (arg | (b > 0.f ? 4u : 0u)) << (8 * c);
                     }
@@ -620,6 +627,9 @@ __global__ __launch_bounds__(WG_THREADS, 1) void winograd_fwd_kernel(const WinoA
                                                            ok ? eoff * 4 : 0x80000000u, 0, 0);
                     __builtin_amdgcn_raw_buffer_store_b32(packed, pir, ok ? eoff : 0x80000000u, 0, 0);
                 }
+                };
+                if (a.relu) pool_rows(integral_constant<bool, true>{});
+                else pool_rows(integral_constant<bool, false>{});
             } else {
                 // bias, ReLU, output mask (bits fetched above) and the NHWC stores.  Thread -> pixel column
                 // (tid >> 4) & 15, channels k4..k4+3, pixel rows (tid >> 8) + 2 it: one base offset, a scalar
