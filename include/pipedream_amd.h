@@ -249,6 +249,15 @@ int pd_conv3x3_winograd_fwd_nhwc_f32(const float* x, const float* u, const float
 int pd_conv3x3_winograd_fwd_pool_nhwc_f32(const float* x, const float* u, const float* bias, float* y_pool,
                                           uint8_t* idx, int N, int H, int W, int C, int K, int relu,
                                           void* stream);
+/* The same kernel as the input gradient of a convolution whose input came out of such a pooling (this
+ * epilogue's, or pd_maxpool2x2_fwd_idx_nhwc_f32's) behind a ReLU: x is the convolution's output gradient,
+ * u its filter transformed with rot180, idx [N,H,W,K] the pooling's index bytes.  Besides y [N,H,W,K],
+ * the gradient with respect to the pooled tensor masked where the recorded maximum was not positive, it
+ * writes y_full [N,2H,2W,K] = pd_maxpool2x2_bwd_idx_nhwc_f32(y, idx, relu_mask = 1): the backward of the
+ * MaxPool2d + ReLU pair (stage1.py:10-11) leaves the convolution kernel's epilogue instead of a kernel of
+ * its own that re-reads y.  Needs the full-resolution size to be exactly 2H x 2W. */
+int pd_conv3x3_winograd_fwd_unpool_nhwc_f32(const float* x, const float* u, const uint8_t* idx, float* y,
+                                            float* y_full, int N, int H, int W, int C, int K, void* stream);
 /* Weight (and optional bias) gradient of the same convolution in the Winograd domain: sums
  * dU = sum over 2x2 output tiles of (A dY A^T) (B^T d B) in persistent blocks, adds the blocks' partial
  * sums in fixed order and applies G^T . G.  Deterministic; agrees with pd_conv3x3_wgrad_nhwc_f32 to

@@ -86,6 +86,7 @@ SIGNATURES = {
     "pd_conv3x3_winograd_filter_f32": (_i, [_vp, _vp, _i, _i, _i, _vp], True),
     "pd_conv3x3_winograd_fwd_nhwc_f32": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _vp], True),
     "pd_conv3x3_winograd_fwd_pool_nhwc_f32": (_i, [_vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _vp], True),
+    "pd_conv3x3_winograd_fwd_unpool_nhwc_f32": (_i, [_vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _vp], True),
     "pd_maxpool2x2_fwd_idx_nhwc_f32": (_i, [_vp, _vp, _vp, _i, _i, _i, _i, _i, _vp], True),
     "pd_maxpool2x2_bwd_idx_nhwc_f32": (_i, [_vp, _vp, _vp, _i, _i, _i, _i, _i, _vp], True),
     "pd_conv3x3_winograd_wgrad_supported": (_i, [_i, _i], False),

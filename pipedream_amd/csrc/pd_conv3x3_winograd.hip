@@ -71,6 +71,9 @@ struct WinoArgs {
     float* y;               // [N,H,W,K]
     float* pool_y;          // pooling variant: [N,H/2,W/2,K], written instead of y
     uint8_t* pool_idx;      // pooling variant: [N,H/2,W/2,K] window position (bits 0-1) and sign (bit 2)
+    const uint8_t* unpool_idx;   // unpooling variant: [N,H,W,K] index bytes of the 2x2 pooling that produced this
+                                 // convolution's input (the convolution is an input gradient)
+    float* unpool_y;        // unpooling variant: [N,2H,2W,K], the gradient in front of that pooling
     int N, H, W, C, K;
     int img_h;              // stacked variant: rows of one image (N is then 1 and H the rows of the whole batch)
     int relu;
@@ -192,7 +195,14 @@ __device__ __forceinline__ WinoItem wino_decode(const WinoArgs& a, int item) {
 // the neighbouring image's row.  Only the threads that form row 0 (d0 - d2) resp. row 3 (d1 - d3) of
 // B^T d read those rows: for such a tile their row pointer goes to a patch of zeros in LDS (units 9 and
 // 10 of a halo row, which no piece is ever written to) -- set once per work item, nothing per step.
-template <bool MASK, bool POOL, bool STACKED>
+//
+// UNPOOL: the launch computes the input gradient of a convolution whose input came out of a 2 x 2 max
+// pooling with index bytes (the pooling epilogue above, or the pooling kernel).  The epilogue then also
+// applies that pooling's backward: every value goes to its window's recorded position in the
+// full-resolution gradient if the recorded maximum was positive (the ReLU in front of the pooling), the
+// window's other three positions get zeros, and y itself is stored with the same mask -- what the
+// pooling backward kernel would compute from y, without the kernel and without its re-read of y.
+template <bool MASK, bool POOL, bool STACKED, bool UNPOOL = false>
 __global__ __launch_bounds__(WG_THREADS, 1) void winograd_fwd_kernel(const WinoArgs a) {
     __shared__ __attribute__((aligned(16))) float lds[WG_LDS_FLOATS];
 
@@ -548,7 +558,20 @@ __global__ __launch_bounds__(WG_THREADS, 1) void winograd_fwd_kernel(const WinoA
 #pragma unroll
                     for (int c = 0; c < 4; ++c) mbits |= (mk[it][c] > 0.f ? 1u : 0u) << (it * 4 + c);
             };
-            if (!POOL && a.out_mask && gh == 1) fetch_mask();
+            // unpooling variant: the index bytes of the thread's eight stores (four channels each), requested
+            // where the mask would be
+            uint32_t iw[UNPOOL ? NV : 1];
+            auto fetch_idx = [&]() {
+                const __amdgpu_buffer_rsrc_t ir = __builtin_amdgcn_make_buffer_rsrc(
+                    (void*)(a.unpool_idx + oimg), 0, out_bytes / 4, 0x00020000);
+#pragma unroll
+                for (int it = 0; it < NV; ++it) {
+                    const uint32_t voff = (col_ok && w.y0 + prow + 2 * it < a.H) ? obase / 4 : 0x80000000u;
+                    iw[UNPOOL ? it : 0] = __builtin_amdgcn_raw_buffer_load_b32(ir, voff, it * (row_stride / 4), 2);
+                }
+            };
+            if (UNPOOL && gh == 1) fetch_idx();
+            if (!POOL && !UNPOOL && a.out_mask && gh == 1) fetch_mask();
             // bias of the thread's four channels for the store phase (k4 is the same there and in the pooling
             // variant): requested at the start of the second summation phase, which hides the round trip;
             // channels past K (and a null bias, as a buffer of size 0) read 0
@@ -567,7 +590,8 @@ __global__ __launch_bounds__(WG_THREADS, 1) void winograd_fwd_kernel(const WinoA
             __syncthreads();
             load_bias();
             if (gh == 0) {
-                if (!POOL && a.out_mask) fetch_mask();
+                if (UNPOOL) fetch_idx();
+                if (!POOL && !UNPOOL && a.out_mask) fetch_mask();
                 out_rows(integral_constant<int, 8>{}, integral_constant<bool, false>{}, true);
             } else {
                 out_rows(integral_constant<int, 0>{}, integral_constant<bool, true>{}, true);
@@ -666,7 +690,38 @@ __global__ __launch_bounds__(WG_THREADS, 1) void winograd_fwd_kernel(const WinoA
                 };
                 using yes = integral_constant<bool, true>;
                 using no = integral_constant<bool, false>;
-                if (a.relu) {
+                if constexpr (UNPOOL) {
+                    // y with the mask of bit 2, and the four positions of every window of the gradient in front
+                    // of the pooling: (2 row + i, 2 column + j) gets the value where the byte says 4 | 2 i + j
+                    const __amdgpu_buffer_rsrc_t fr = __builtin_amdgcn_make_buffer_rsrc(
+                        (void*)(a.unpool_y + 4 * oimg), 0, out_bytes * 4, 0x00020000);
+                    const uint32_t fbase = (uint32_t)((2 * (w.y0 + prow) * 2 * a.W + 2 * (w.x0 + pcol)) * a.K + k0 + k4) * 4;
+                    const uint32_t frow = (uint32_t)(2 * a.W * a.K) * 4;        // one full-resolution row
+                    typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+    #pragma unroll
+                    for (int it = 0; it < NV; ++it) {
+                        const bool ok = col_ok && w.y0 + prow + 2 * it < a.H;
+                        const uint32_t voff = (ok ? obase : 0x80000000u) + (uint32_t)(it * row_stride);
+                        const uint32_t foff = (ok ? fbase : 0x80000000u) + (uint32_t)it * (4 * frow);
+                        const float4_t v = *(const float4_t*)(src + it * 2 * WG_PIX * WG_OP) + b4;
+                        uint32_t code[4];
+    #pragma unroll
+                        for (int c = 0; c < 4; ++c) code[c] = (iw[UNPOOL ? it : 0] >> (8 * c)) & 7u;
+                        float4_t kept;
+    #pragma unroll
+                        for (int c = 0; c < 4; ++c) kept[c] = (code[c] & 4u) ? v[c] : 0.f;
+                        __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(u32x4, kept), yr, voff, 0, 2);
+    #pragma unroll
+                        for (int pos = 0; pos < 4; ++pos) {
+                            float4_t o;
+    #pragma unroll
+                            for (int c = 0; c < 4; ++c) o[c] = code[c] == (4u | pos) ? v[c] : 0.f;
+                            __builtin_amdgcn_raw_buffer_store_b128(
+                                __builtin_bit_cast(u32x4, o), fr,
+                                foff + (uint32_t)(pos >> 1) * frow + (uint32_t)((pos & 1) * a.K * 4), 0, 2);
+                        }
+                    }
+                } else if (a.relu) {
                     if (a.out_mask) store_rows(yes{}, yes{});
                     else store_rows(yes{}, no{});
                 } else {
@@ -711,7 +766,7 @@ namespace {
 
 int wino_fwd_launch(const char* who, const float* x, const float* u, const float* bias, const float* in_mask,
                     const float* out_mask, float* y, float* pool_y, uint8_t* pool_idx, int N, int H, int W, int C,
-                    int K, int relu, void* stream) {
+                    int K, int relu, void* stream, const uint8_t* unpool_idx = nullptr, float* unpool_y = nullptr) {
     PD_REQUIRE(N > 0 && H > 0 && W > 0 && C > 0 && K > 0, PD_ESHAPE, "%s: dimensions must be positive", who);
     PD_REQUIRE(wino_shape_ok(C, K), PD_ESHAPE, "%s: needs C %% 8 == 0 and K %% 4 == 0 (C=%d K=%d)", who, C, K);
     PD_REQUIRE((long)H * W * (C > K ? C : K) < (1L << 29), PD_ESHAPE, "%s: image too large", who);
@@ -722,12 +777,15 @@ int wino_fwd_launch(const char* who, const float* x, const float* u, const float
     WinoArgs a;
     a.x = x; a.u = u; a.bias = bias; a.mask = in_mask; a.out_mask = out_mask; a.y = y;
     a.pool_y = pool_y; a.pool_idx = pool_idx;
+    a.unpool_idx = unpool_idx; a.unpool_y = unpool_y;
     a.N = N; a.H = H; a.W = W; a.C = C; a.K = K;
     a.img_h = 0;
     // images whose height is even but no multiple of the 16-row tile are stacked into one tall image
     // (see the kernel): N * ceil(H / 16) tile rows become ceil(N * H / 16)
     // (not with an input mask: that variant has no registers to spare for it)
-    const bool stacked = !in_mask && N > 1 && H % 2 == 0 && H % WG_PIX != 0 && (long)N * H * W * (C > K ? C : K) < (1L << 29);
+    // (with the unpooling epilogue the full-resolution gradient, four times y, must fit a buffer descriptor too)
+    const bool stacked = !in_mask && N > 1 && H % 2 == 0 && H % WG_PIX != 0 &&
+                         (long)N * H * W * (C > K ? C : K) < (1L << 29) && (!unpool_y || (long)N * H * W * K < (1L << 27));
     if (stacked) { a.img_h = H; a.H = N * H; a.N = 1; }
     a.relu = relu != 0;
     a.tiles_x = (W + WG_PIX - 1) / WG_PIX;
@@ -747,7 +805,10 @@ int wino_fwd_launch(const char* who, const float* x, const float* u, const float
     if (blocks > (long)a.items_per_xcd * WG_XCD) blocks = (long)a.items_per_xcd * WG_XCD;
     dim3 grid((unsigned)blocks);
     hipStream_t s = (hipStream_t)stream;
-    if (stacked) {
+    if (unpool_y) {
+        if (stacked) winograd_fwd_kernel<false, false, true, true><<<grid, WG_THREADS, 0, s>>>(a);
+        else winograd_fwd_kernel<false, false, false, true><<<grid, WG_THREADS, 0, s>>>(a);
+    } else if (stacked) {
         if (a.pool_y) winograd_fwd_kernel<false, true, true><<<grid, WG_THREADS, 0, s>>>(a);
         else winograd_fwd_kernel<false, false, true><<<grid, WG_THREADS, 0, s>>>(a);
     } else {
@@ -767,6 +828,19 @@ extern "C" int pd_conv3x3_winograd_fwd_nhwc_f32(const float* x, const float* u, 
     const char* who = "pd_conv3x3_winograd_fwd_nhwc_f32";
     PD_REQUIRE(y, PD_EINVAL, "%s: NULL pointer", who);
     return wino_fwd_launch(who, x, u, bias, in_mask, out_mask, y, nullptr, nullptr, N, H, W, C, K, relu, stream);
+}
+
+extern "C" int pd_conv3x3_winograd_fwd_unpool_nhwc_f32(const float* x, const float* u, const uint8_t* idx, float* y,
+                                                       float* y_full, int N, int H, int W, int C, int K,
+                                                       void* stream) {
+    const char* who = "pd_conv3x3_winograd_fwd_unpool_nhwc_f32";
+    PD_REQUIRE(y && y_full && idx, PD_EINVAL, "%s: NULL pointer", who);
+    PD_REQUIRE(pd_aligned(y_full, 16) && pd_aligned(idx, 4), PD_EINVAL,
+               "%s: the full-resolution output must be 16-byte aligned, the index bytes 4-byte aligned", who);
+    PD_REQUIRE(H > 0 && W > 0 && K > 0 && (long)H * W * K < (1L << 27), PD_ESHAPE,
+               "%s: image too large for the full-resolution output", who);
+    return wino_fwd_launch(who, x, u, nullptr, nullptr, nullptr, y, nullptr, nullptr, N, H, W, C, K, 0, stream, idx,
+                           y_full);
 }
 
 extern "C" int pd_conv3x3_winograd_fwd_pool_nhwc_f32(const float* x, const float* u, const float* bias,

@@ -79,20 +79,65 @@ class Linear(torch.nn.Module):
 # --------------------------------------------------------------------------------------
 # Conv2d 3x3
 # --------------------------------------------------------------------------------------
+class PoolGradLink(object):
+    """Couples a ReLU + 2x2 max pooling (``MaxPool2d(relu=True)``, or ``Conv2d(relu=True, pool=True)``) with
+    the convolution that takes its output, so that the pooling's backward can leave that convolution's
+    input-gradient kernel: give the same link to both layers.
+
+    Forward: the pooling layer leaves its index bytes with the link (``offer``); the convolution, called
+    next with that very tensor, takes them (``take``) and keeps them for its backward.  Backward: the
+    convolution computes its input gradient and, in the same kernel, the gradient in front of the pooling,
+    returns the former to autograd as usual and leaves the latter with the link (``deposit``); the pooling
+    layer's backward asks for it (``claim``) with the gradient autograd hands it, and gets it only if that
+    gradient is the tensor the convolution returned -- otherwise (another consumer added its gradient, the
+    shapes have no fused kernel, ...) it runs its own backward kernel on what it received.  Results are the
+    same either way; nothing depends on the link being honoured."""
+
+    def __init__(self):
+        self._offer = None      # (pooled output, index bytes) of the forward in progress
+        self._deposit = None    # (pooled gradient, full-resolution gradient) of the backward in progress
+
+    def offer(self, pooled, idx):
+        self._offer = (pooled, idx)
+
+    def take(self, x):
+        offer, self._offer = self._offer, None
+        if offer is not None and offer[0].data_ptr() == x.data_ptr() and offer[0].shape == x.shape:
+            return offer[1]
+        return None
+
+    def deposit(self, pooled_grad, full_grad):
+        self._deposit = (pooled_grad, full_grad)
+
+    def claim(self, dy, h, w):
+        deposit, self._deposit = self._deposit, None
+        if (deposit is not None and deposit[0].data_ptr() == dy.data_ptr() and deposit[0].shape == dy.shape
+                and tuple(deposit[1].shape[2:]) == (h, w)):
+            return deposit[1]
+        return None
+
+
 class _Conv3x3Fn(torch.autograd.Function):
     @staticmethod
-    def forward(ctx, x, weight, bias, relu, grad_premasked=False, input_rectified=False, pool=False):
+    def forward(ctx, x, weight, bias, relu, grad_premasked=False, input_rectified=False, pool=False,
+                input_link=None, output_link=None):
         x = ops.to_nhwc(x)
         ctx.input_rectified = input_rectified
         ctx.relu = relu
         ctx.has_bias = bias is not None
         ctx.pool = pool
+        # the index bytes of the pooling that produced x, if that layer shares a link with this one
+        ctx.input_link = input_link
+        ctx.unpool_idx = input_link.take(x) if input_link is not None else None
+        ctx.output_link = output_link if (pool and relu) else None
         if pool:
             # convolution (+ReLU) and the 2x2 pooling behind it in one kernel: the backward rebuilds the
             # convolution's output gradient from the pooled gradient and the index bytes, already masked
             # by the ReLU, so the full-resolution output is neither written nor kept
             y, idx = ops.conv3x3_forward_pool(x, weight, bias, relu)
             ctx.save_for_backward(x, weight, idx)
+            if ctx.output_link is not None:
+                ctx.output_link.offer(y, idx)
             return y
         y = ops.conv3x3_forward(x, weight, bias, relu)
         # with grad_premasked the consumer's backward (a pooling layer with relu=True) has already
@@ -105,16 +150,25 @@ class _Conv3x3Fn(torch.autograd.Function):
         x, weight, y = ctx.saved_tensors
         dy = ops.to_nhwc(dy)
         if ctx.pool:
-            dy = ops.maxpool2x2_idx_backward(dy, y, x.shape[2], x.shape[3], relu_mask=ctx.relu)
+            full = ctx.output_link.claim(dy, x.shape[2], x.shape[3]) if ctx.output_link is not None else None
+            dy = full if full is not None else ops.maxpool2x2_idx_backward(dy, y, x.shape[2], x.shape[3],
+                                                                           relu_mask=ctx.relu)
             y = None
         # the ReLU backward (dy where y > 0) is applied by the gradient kernels while they
         # load dy, so no masked copy of dy is ever written
         dx = dw = db = None
         if ctx.needs_input_grad[0]:
-            dx = ops.conv3x3_input_grad(dy, weight, relu_out=y, x_rectified=x if ctx.input_rectified else None)
+            idx = ctx.unpool_idx
+            if idx is not None and y is None and ops.conv3x3_input_grad_unpool_supported(dy, weight):
+                # x is the output of a ReLU + pooling: the mask of its index bytes is the mask of
+                # input_rectified, and the pooling's backward comes out of the same kernel
+                dx, full = ops.conv3x3_input_grad_unpool(dy, weight, idx)
+                ctx.input_link.deposit(dx, full)
+            else:
+                dx = ops.conv3x3_input_grad(dy, weight, relu_out=y, x_rectified=x if ctx.input_rectified else None)
         if ctx.needs_input_grad[1] or (ctx.has_bias and ctx.needs_input_grad[2]):
             dw, db = ops.conv3x3_weight_grad(x, dy, with_bias=ctx.has_bias, relu_out=y)
-        return dx, dw, db, None, None, None, None
+        return dx, dw, db, None, None, None, None, None, None
 
 
 class Conv2d(torch.nn.Module):
@@ -134,10 +188,14 @@ class Conv2d(torch.nn.Module):
     ``pool=True`` appends ``MaxPool2d(2, 2)`` to the layer (after the ReLU, if any): the layer returns the
     pooled tensor, computed in the convolution kernel's epilogue where that kernel supports it, and the
     pooling module that follows in the reference's layer list is declared with
-    ``MaxPool2d(..., applied_by_producer=True)``."""
+    ``MaxPool2d(..., applied_by_producer=True)``.
+
+    ``input_link`` / ``output_link``: a ``PoolGradLink`` shared with the pooling layer that produces this
+    layer's input, resp. (with ``relu=True, pool=True``) with the convolution that takes this layer's pooled
+    output; the pooling's backward then comes out of the consuming convolution's input-gradient kernel."""
 
     def __init__(self, in_channels, out_channels, kernel_size=3, stride=1, padding=1, bias=True, relu=False,
-                 grad_premasked=False, input_rectified=False, pool=False):
+                 grad_premasked=False, input_rectified=False, pool=False, input_link=None, output_link=None):
         super(Conv2d, self).__init__()
         norm = lambda v: tuple(v) if isinstance(v, (tuple, list)) else (v, v)
         if norm(kernel_size) != (3, 3) or norm(stride) != (1, 1) or norm(padding) != (1, 1):
@@ -150,6 +208,8 @@ class Conv2d(torch.nn.Module):
         self.grad_premasked = grad_premasked
         self.input_rectified = input_rectified
         self.pool = pool
+        self.input_link = input_link
+        self.output_link = output_link
         w = torch.empty(out_channels, in_channels, 3, 3)
         torch.nn.init.kaiming_uniform_(w, a=math.sqrt(5))
         self.weight = torch.nn.Parameter(w.contiguous(memory_format=torch.channels_last))
@@ -161,7 +221,7 @@ class Conv2d(torch.nn.Module):
 
     def forward(self, x):
         return _Conv3x3Fn.apply(x, self.weight, self.bias, self.relu, self.grad_premasked, self.input_rectified,
-                                self.pool)
+                                self.pool, self.input_link, self.output_link)
 
     def extra_repr(self):
         return "{}, {}, kernel_size=(3, 3), stride=(1, 1), padding=(1, 1), relu={}".format(
@@ -198,31 +258,40 @@ class ReLU(torch.nn.Module):
 
 class _MaxPool2x2Fn(torch.autograd.Function):
     @staticmethod
-    def forward(ctx, x, relu):
+    def forward(ctx, x, relu, link=None):
         x = ops.to_nhwc(x)
         y, idx = ops.maxpool2x2_idx(x, relu=relu)
         ctx.relu = relu
         ctx.hw = (x.shape[2], x.shape[3])
+        ctx.link = link if relu else None
         ctx.save_for_backward(idx)      # one byte per output element; the input is not needed again
+        if ctx.link is not None:
+            ctx.link.offer(y, idx)
         return y
 
     @staticmethod
     def backward(ctx, dy):
         (idx,) = ctx.saved_tensors
-        return ops.maxpool2x2_idx_backward(dy, idx, ctx.hw[0], ctx.hw[1], relu_mask=ctx.relu), None
+        dy = ops.to_nhwc(dy)
+        full = ctx.link.claim(dy, ctx.hw[0], ctx.hw[1]) if ctx.link is not None else None
+        if full is None:
+            full = ops.maxpool2x2_idx_backward(dy, idx, ctx.hw[0], ctx.hw[1], relu_mask=ctx.relu)
+        return full, None, None
 
 
 class MaxPool2d(torch.nn.Module):
     """``torch.nn.MaxPool2d(kernel_size=2, stride=2)`` on NHWC activations.  ``relu=True``: a ReLU in front
     of the pooling (stage1.py:10-11), fused.  ``applied_by_producer=True``: the convolution in front of
     this module was built with ``pool=True`` and has already pooled (and rectified) its output; the module
-    keeps its place in the layer list and passes the tensor through."""
+    keeps its place in the layer list and passes the tensor through.  ``link`` (with ``relu=True``): a
+    ``PoolGradLink`` shared with the convolution that takes this layer's output."""
 
     def __init__(self, kernel_size=2, stride=2, padding=0, dilation=1, ceil_mode=False, relu=False,
-                 applied_by_producer=False):
+                 applied_by_producer=False, link=None):
         super(MaxPool2d, self).__init__()
         self.relu = relu
         self.applied_by_producer = applied_by_producer
+        self.link = link
         ks = kernel_size if isinstance(kernel_size, int) else kernel_size[0]
         st = ks if stride is None else (stride if isinstance(stride, int) else stride[0])
         if ks != 2 or st != 2 or padding not in (0, (0, 0)) or dilation not in (1, (1, 1)) or ceil_mode:
@@ -231,7 +300,7 @@ class MaxPool2d(torch.nn.Module):
     def forward(self, x):
         if self.applied_by_producer:
             return x
-        return _MaxPool2x2Fn.apply(x, self.relu)
+        return _MaxPool2x2Fn.apply(x, self.relu, self.link)
 
 
 class _DropoutFn(torch.autograd.Function):

@@ -533,6 +533,44 @@ def conv3x3_input_grad(dy, w, relu_out=None, x_rectified=None):
     return dx
 
 
+def conv3x3_input_grad_unpool_supported(dy, w):
+    """Whether conv3x3_input_grad_unpool has a kernel for this gradient (the Winograd kernel applies and the
+    full-resolution gradient fits its addressing)."""
+    n, h, wd, k = _nhwc_dims(dy)
+    kw, c = _filter_dims(w)
+    return kw == k and _use_winograd(k, c, h, wd) and h * wd * c < 1 << 27
+
+
+def conv3x3_input_grad_unpool(dy, w, idx):
+    """``conv3x3_input_grad`` for a layer whose input came out of a ReLU + 2x2 max pooling with index
+    bytes ``idx`` (``maxpool2x2_idx`` or ``conv3x3_forward_pool``): returns (dx, dx_full) with dx masked
+    where the pooled maximum was not positive and ``dx_full = maxpool2x2_idx_backward(dx, idx,
+    relu_mask=True)`` for a pooling input of exactly twice the size, both written by the convolution
+    kernel's epilogue."""
+    _check(dy, "dy")
+    _check(idx, "idx", torch.uint8)
+    n, h, wd, k = _nhwc_dims(dy)
+    kw, c = _filter_dims(w)
+    if kw != k:
+        raise ValueError("conv3x3_input_grad_unpool: dy has %d channels, filter has %d outputs" % (k, kw))
+    if tuple(idx.shape) != (n, c, h, wd) or not idx.is_contiguous(memory_format=torch.channels_last):
+        raise ValueError("conv3x3_input_grad_unpool: idx must be the channels_last index bytes of the layer's input")
+    if not conv3x3_input_grad_unpool_supported(dy, w):
+        raise ValueError("conv3x3_input_grad_unpool: no kernel for this shape (see conv3x3_input_grad_unpool_supported)")
+    lib = _cabi.lib()
+    nbytes = ctypes.c_uint64()
+    lib.pd_conv3x3_winograd_filter_bytes(k, c, ctypes.byref(nbytes))
+    u = torch.empty(nbytes.value // 4, dtype=torch.float32, device=dy.device)
+    lib.pd_conv3x3_winograd_filter_f32(_ptr(w), _ptr(u), k, c, 1, _cabi.stream_ptr())
+    dx = torch.empty((n, c, h, wd), dtype=torch.float32, device=dy.device, memory_format=torch.channels_last)
+    full = torch.empty((n, c, 2 * h, 2 * wd), dtype=torch.float32, device=dy.device,
+                       memory_format=torch.channels_last)
+    with _timed("conv3x3_winograd_kernel", 18.0 * c * k * n * h * wd):
+        lib.pd_conv3x3_winograd_fwd_unpool_nhwc_f32(_ptr(dy), _ptr(u), _ptr(idx), _ptr(dx), _ptr(full), n, h, wd, k, c,
+                                                    _cabi.stream_ptr())
+    return dx, full
+
+
 def conv3x3_weight_grad(x, dy, with_bias=True, relu_out=None):
     """(dw [K,C,3,3] channels_last, dbias [K] or None).  ``relu_out`` masks dy as in
     conv3x3_input_grad."""

@@ -47,9 +47,12 @@ class FrontStage(torch.nn.Module):
         # kernels read no mask (grad_premasked)
         # (with pool=True the convolution kernel pools in its epilogue; the pooling module keeps its place
         # in the layer list and passes the tensor through)
-        self.layer4 = layers.Conv2d(64, 64, relu=True, input_rectified=True, pool=True)
+        # (a PoolGradLink between a pooling and the convolution behind it: the pooling's backward comes out
+        # of that convolution's input-gradient kernel)
+        pool1 = layers.PoolGradLink()
+        self.layer4 = layers.Conv2d(64, 64, relu=True, input_rectified=True, pool=True, output_link=pool1)
         self.layer6 = layers.MaxPool2d(2, 2, relu=True, applied_by_producer=True)
-        self.layer7 = layers.Conv2d(64, 128, relu=True, grad_premasked=True)
+        self.layer7 = layers.Conv2d(64, 128, relu=True, grad_premasked=True, input_link=pool1)
         self.layer9 = layers.Conv2d(128, 128, relu=True, input_rectified=True, pool=True)
         self.layer11 = layers.MaxPool2d(2, 2, relu=True, applied_by_producer=True)
         _initialize_weights(self)
@@ -80,12 +83,14 @@ class Stage1(torch.nn.Module):
 
     def __init__(self):
         super(Stage1, self).__init__()
-        self.layer2 = layers.MaxPool2d(2, 2, relu=True)    # layer1 ReLU + layer2 MaxPool
-        self.layer3 = layers.Conv2d(64, 128, relu=True, grad_premasked=True)    # + layer4; masked by layer5
-        self.layer5 = layers.Conv2d(128, 128, relu=True, input_rectified=True, pool=True)   # + layer6 + layer7
+        pool1, pool2 = layers.PoolGradLink(), layers.PoolGradLink()
+        self.layer2 = layers.MaxPool2d(2, 2, relu=True, link=pool1)    # layer1 ReLU + layer2 MaxPool
+        self.layer3 = layers.Conv2d(64, 128, relu=True, grad_premasked=True, input_link=pool1)    # + layer4; masked by layer5
+        self.layer5 = layers.Conv2d(128, 128, relu=True, input_rectified=True, pool=True,
+                                    output_link=pool2)                  # + layer6 + layer7
         self.layer7 = layers.MaxPool2d(2, 2, relu=True, applied_by_producer=True)
         # layer8's ReLU is undone for the gradient by the next stage's first convolution (input_rectified)
-        self.layer8 = layers.Conv2d(128, 256, relu=True, grad_premasked=True)   # + layer9
+        self.layer8 = layers.Conv2d(128, 256, relu=True, grad_premasked=True, input_link=pool2)   # + layer9
         _initialize_weights(self)
 
     def forward(self, input0):
@@ -104,9 +109,11 @@ class Stage2(torch.nn.Module):
     def __init__(self):
         super(Stage2, self).__init__()
         self.layer1 = layers.Conv2d(256, 256, relu=True, grad_premasked=True, input_rectified=True)   # + layer2; masked by layer3
-        self.layer3 = layers.Conv2d(256, 256, relu=True, input_rectified=True, pool=True)   # + layer4 + layer5
+        pool3 = layers.PoolGradLink()
+        self.layer3 = layers.Conv2d(256, 256, relu=True, input_rectified=True, pool=True,
+                                    output_link=pool3)                  # + layer4 + layer5
         self.layer5 = layers.MaxPool2d(2, 2, relu=True, applied_by_producer=True)
-        self.layer6 = layers.Conv2d(256, 512, relu=True, grad_premasked=True)   # + layer7; masked by layer8
+        self.layer6 = layers.Conv2d(256, 512, relu=True, grad_premasked=True, input_link=pool3)   # + layer7; masked by layer8
         self.layer8 = layers.Conv2d(512, 512, relu=True, grad_premasked=True, input_rectified=True)   # + layer9
         # layer10's ReLU is undone for the gradient by the next stage's pooling layer (relu=True)
         self.layer10 = layers.Conv2d(512, 512, relu=True, grad_premasked=True, input_rectified=True)  # + layer11
@@ -125,8 +132,9 @@ class Stage3(torch.nn.Module):
 
     def __init__(self, dropout=0.5, num_classes=1000):
         super(Stage3, self).__init__()
-        self.layer1 = layers.MaxPool2d(2, 2, relu=True)
-        self.layer2 = layers.Conv2d(512, 512, relu=True, grad_premasked=True)   # + layer3; masked by layer4
+        pool4 = layers.PoolGradLink()
+        self.layer1 = layers.MaxPool2d(2, 2, relu=True, link=pool4)
+        self.layer2 = layers.Conv2d(512, 512, relu=True, grad_premasked=True, input_link=pool4)   # + layer3; masked by layer4
         self.layer4 = layers.Conv2d(512, 512, relu=True, grad_premasked=True, input_rectified=True)   # + layer5
         self.layer6 = layers.Conv2d(512, 512, relu=True, input_rectified=True, pool=True)   # + layer7 + layer8
         self.layer8 = layers.MaxPool2d(2, 2, relu=True, applied_by_producer=True)

@@ -132,6 +132,11 @@ def test_argument_validation_of_the_sequence_and_pooling_entry_points():
         lib.pd_conv3x3_winograd_fwd_pool_nhwc_f32(p, p, None, p, p, 1, 8, 8, 12, 32, 1, None)
     with pytest.raises(E, match="too large"):
         lib.pd_conv3x3_winograd_fwd_nhwc_f32(p, p, None, None, None, p, 1, 4096, 4096, 64, 64, 0, None)
+    # ... and with the pooling backward in its epilogue
+    with pytest.raises(E, match="NULL"):
+        lib.pd_conv3x3_winograd_fwd_unpool_nhwc_f32(p, p, None, p, p, 1, 8, 8, 16, 32, None)
+    with pytest.raises(E, match="too large"):
+        lib.pd_conv3x3_winograd_fwd_unpool_nhwc_f32(p, p, p, p, p, 1, 2048, 2048, 64, 64, None)
     # Winograd weight gradient: channel counts, a batch whose pixels overflow its 32-bit row counter, workspace
     with pytest.raises(E, match="unsupported channel counts"):
         lib.pd_conv3x3_winograd_wgrad_nhwc_f32(p, p, p, p, p, 1 << 30, 1, 8, 8, 48, 64, None)

@@ -453,3 +453,59 @@ def test_batch_of_images_whose_height_is_no_multiple_of_the_tile(N, C, K, H, W, 
     torch.testing.assert_close(yp.cpu().double(), F.max_pool2d(F.relu(ref), 2, 2).detach(), rtol=1e-5, atol=2e-5)
     ref.backward(dy.cpu().double())
     torch.testing.assert_close(dx.cpu().double(), xd.grad, rtol=1e-5, atol=2e-5)
+
+
+@pytest.mark.parametrize("N,C,K,H,W", [(2, 16, 32, 16, 16),     # pooled 8 x 8: one tile
+                                        (3, 64, 64, 28, 28),     # pooled 14 x 14: stacked batch
+                                        (1, 32, 64, 40, 72),     # several tiles, ragged
+                                        (2, 8, 24, 12, 20)])
+@pytest.mark.parametrize("producer", ["conv_pool", "maxpool"])
+def test_pooling_backward_in_the_consuming_convolution_kernel(N, C, K, H, W, producer, conv_algorithm):
+    """ReLU + MaxPool2d followed by a convolution, with and without a PoolGradLink between them: the linked pair
+    lets the convolution's input-gradient kernel write the gradient in front of the pooling; every output
+    and every gradient must equal the unlinked pair's bit for bit (the same values reach the same kernels),
+    and the pooling backward kernel must not run in the linked pair."""
+    if conv_algorithm != "winograd":
+        pytest.skip("the fused epilogue belongs to the Winograd kernel")
+    torch.manual_seed(N + C + H)
+
+    def build(linked):
+        link = layers.PoolGradLink() if linked else None
+        if producer == "conv_pool":
+            first = [layers.Conv2d(C, C, relu=True, pool=True, output_link=link),
+                     layers.MaxPool2d(2, 2, relu=True, applied_by_producer=True)]
+        else:
+            first = [layers.Conv2d(C, C, relu=True, grad_premasked=True), layers.MaxPool2d(2, 2, relu=True, link=link)]
+        # (the consumer reads no mask of its own: in the stages it is followed by a layer that masks its gradient)
+        return torch.nn.Sequential(*first, layers.Conv2d(C, K, input_link=link)).cuda()
+
+    plain, linked = build(False), build(True)
+    linked.load_state_dict(plain.state_dict())
+    x = torch.randn(N, C, H, W).cuda()
+    xa, xb = x.clone().requires_grad_(True), x.clone().requires_grad_(True)
+    ya, yb = plain(xa), linked(xb)
+    assert torch.equal(ya, yb)
+    dy = torch.randn_like(ya)
+    ya.backward(dy)
+    ops.kernel_timer = {}                      # records the name of every timed launch
+    try:
+        yb.backward(dy)
+        torch.cuda.synchronize()
+        ran = set(ops.kernel_timer)
+    finally:
+        ops.kernel_timer = None
+    assert "maxpool2x2_bwd_idx" not in ran and "conv3x3_winograd_kernel" in ran, ran
+    assert torch.equal(xa.grad, xb.grad)
+    for pa, pb in zip(plain.parameters(), linked.parameters()):
+        assert torch.equal(pa.grad, pb.grad)
+    # and the values: torch in fp64
+    ref = torch.nn.Sequential(torch.nn.Conv2d(C, C, 3, padding=1), torch.nn.ReLU(), torch.nn.MaxPool2d(2, 2),
+                              torch.nn.Conv2d(C, K, 3, padding=1)).double()
+    ref[0].weight.data.copy_(plain[0].weight.detach().cpu())
+    ref[0].bias.data.copy_(plain[0].bias.detach().cpu())
+    ref[3].weight.data.copy_(plain[2].weight.detach().cpu())
+    ref[3].bias.data.copy_(plain[2].bias.detach().cpu())
+    xr = x.cpu().double().requires_grad_(True)
+    ref(xr).backward(dy.cpu().double())
+    scale = float(xr.grad.abs().max())
+    torch.testing.assert_close(xb.grad.cpu().double(), xr.grad, rtol=1e-5, atol=2e-5 * max(scale, 1.0))

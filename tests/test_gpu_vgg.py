@@ -576,8 +576,10 @@ def test_front_stage_full_size_every_layer_against_fp64():
                 close(name + " input gradient", got[n, :, h0:h1, w0:w1], ref)
 
     input_grad("conv2_2", stage.layer9, dz9, a3.grad, a3.detach())
-    # conv2_1 hands its input gradient to pool1, i.e. a2.grad, unmasked (the pooling backward masks it)
-    input_grad("conv2_1", stage.layer7, dz7, a2.grad, None)
+    # conv2_1 hands its input gradient to pool1, i.e. a2.grad: its kernel also writes the gradient in front of
+    # the pooling (the link between layer4 and layer7), and stores the pooled gradient with the same mask, the
+    # pooling's "maximum > 0" bit, i.e. a2 > 0
+    input_grad("conv2_1", stage.layer7, dz7, a2.grad, a2.detach())
     input_grad("conv1_2", stage.layer4, dz4, a1.grad, a1.detach())
 
     for name, layer, inp, dz in (("conv2_2", stage.layer9, a3.detach(), dz9), ("conv2_1", stage.layer7, a2.detach(), dz7),
