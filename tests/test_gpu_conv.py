@@ -509,3 +509,32 @@ def test_pooling_backward_in_the_consuming_convolution_kernel(N, C, K, H, W, pro
     ref(xr).backward(dy.cpu().double())
     scale = float(xr.grad.abs().max())
     torch.testing.assert_close(xb.grad.cpu().double(), xr.grad, rtol=1e-5, atol=2e-5 * max(scale, 1.0))
+
+
+def _even_shapes(count, seed):
+    rng = np.random.RandomState(seed)
+    out = []
+    for _ in range(count):
+        # (the gradient kernel reduces over K: a multiple of 8; it writes C channels: a multiple of 4)
+        out.append((int(rng.randint(1, 6)), int(rng.choice([8, 12, 24, 40, 64])), int(rng.choice([8, 16, 32, 64, 72])),
+                    2 * int(rng.randint(1, 24)), 2 * int(rng.randint(1, 24))))
+    return out
+
+
+@pytest.mark.parametrize("N,C,K,H,W", _even_shapes(16, seed=31))
+def test_fused_input_gradient_and_unpooling_on_random_shapes(N, C, K, H, W, conv_algorithm):
+    """``conv3x3_input_grad_unpool`` (input gradient of a C -> K convolution on H x W images + backward of the
+    ReLU / 2x2 pooling that produced its input) against the two kernels it replaces, bit for bit, on random even
+    sizes: batches stacked into one tall image or not, ragged tiles, channel counts off the block sizes."""
+    if conv_algorithm != "winograd":
+        pytest.skip("the fused epilogue belongs to the Winograd kernel")
+    torch.manual_seed(N * 1000 + H * 10 + W)
+    full = _nhwc(torch.randn(N, C, 2 * H, 2 * W))
+    pooled, idx = ops.maxpool2x2_idx(full, relu=True)
+    w = _nhwc(torch.randn(K, C, 3, 3) / math.sqrt(9 * C))
+    dy = _nhwc(torch.randn(N, K, H, W))
+    assert ops.conv3x3_input_grad_unpool_supported(dy, w)
+    dx, dfull = ops.conv3x3_input_grad_unpool(dy, w, idx)
+    want_dx = ops.conv3x3_input_grad(dy, w, x_rectified=pooled)
+    assert torch.equal(dx, want_dx)
+    assert torch.equal(dfull, ops.maxpool2x2_idx_backward(want_dx, idx, 2 * H, 2 * W, relu_mask=True))
