@@ -1171,7 +1171,10 @@ __global__ __launch_bounds__(WW_THREADS, 1) void winograd_wgrad_kernel(const Win
     }
 
     // ---- the block's sums: partial dU in [g][k][c] order, partial dbias per (tile half, k)
-    float* part = a.part + (size_t)(pair * a.ranks + rank) * WW_PART_STRIDE;
+    // element e = (g * 64 + k) * 64 + c of a pair's dU lies at [e / 256][rank][e % 256]: the ranks' values of
+    // one kilobyte of elements are adjacent, so the kernel that sums over the ranks reads contiguous memory
+    float* part = a.part + (size_t)pair * a.ranks * WW_PART_STRIDE + (size_t)rank * 256;
+    const size_t chunk_pitch = (size_t)a.ranks * 256;
 #pragma unroll
     for (int g = 0; g < WG_GW; ++g)
 #pragma unroll
@@ -1179,7 +1182,8 @@ __global__ __launch_bounds__(WW_THREADS, 1) void winograd_wgrad_kernel(const Win
             float v;
             asm volatile("v_accvgpr_read_b32 %0, %1" : "=v"(v) : "a"(acc[g][e]));
             const int k = wm * 32 + 8 * (e / 4) + 4 * h + (e % 4);
-            part[((gh * WG_GW + g) * 64 + k) * 64 + wn * 32 + cl] = v;
+            const int el = ((gh * WG_GW + g) * 64 + k) * 64 + wn * 32 + cl;
+            part[(size_t)(el >> 8) * chunk_pitch + (el & 255)] = v;
         }
     if (gh == 0 && wn == 0) a.part_db[((size_t)(pair * a.ranks + rank) * 2 + h) * 64 + wm * 32 + cl] = db_acc;
 }
@@ -1198,14 +1202,15 @@ __global__ __launch_bounds__(256) void winograd_wgrad_sum_kernel(const float* __
     const long id = (long)blockIdx.x * 256 + threadIdx.x;
     if (id < (long)n_pairs * per_pair) {
         const int pair = (int)(id / per_pair), i = (int)(id % per_pair);
-        const float* src = part + (size_t)pair * ranks * WW_PART_STRIDE + (size_t)i * 4;
+        // (layout [element / 256][rank][element % 256], see the kernel that writes it)
+        const float* src = part + (size_t)pair * ranks * WW_PART_STRIDE + (size_t)(i >> 6) * ranks * 256 + (i & 63) * 4;
         float4_t acc[8];
 #pragma unroll
         for (int u = 0; u < 8; ++u) acc[u] = float4_t{0.f, 0.f, 0.f, 0.f};
         for (int r = r0; r < r1; r += 8) {
 #pragma unroll
             for (int u = 0; u < 8; ++u)
-                if (r + u < r1) acc[u] += *(const float4_t*)(src + (size_t)(r + u) * WW_PART_STRIDE);
+                if (r + u < r1) acc[u] += *(const float4_t*)(src + (size_t)(r + u) * 256);
         }
         ((float4_t*)du4)[(size_t)grp * n_pairs * per_pair + id] =
             ((acc[0] + acc[1]) + (acc[2] + acc[3])) + ((acc[4] + acc[5]) + (acc[6] + acc[7]));
