@@ -373,6 +373,16 @@ int pd_add_bf16(const uint16_t* a, const uint16_t* b, uint16_t* y, uint64_t n, v
 int pd_cast_f32_to_bf16(const float* x, uint16_t* y, uint64_t n, void* stream);
 int pd_cast_bf16_to_f32(const uint16_t* x, float* y, uint64_t n, void* stream);
 int pd_colsum_bf16(const uint16_t* x, float* out, uint64_t M, int N, uint64_t ld, int splits, void* stream);
+/* Up to 8 column sums in two launches (all bias and LayerNorm parameter gradients of one layer's backward
+ * instead of a dozen launches of a few microseconds): job j sums the rows of x[j], a bf16 matrix
+ * (is_bf16[j] != 0: `splits` row ranges first, into the workspace, then their sum) or an fp32 matrix (e.g.
+ * the partials pd_layernorm_bwd_bf16 leaves), [M[j]][N[j]] with leading dimension ld[j], into out[j][N[j]]
+ * (+ beta[j] * out[j]).  The argument arrays are host arrays; workspace: device memory of
+ * pd_colsum_batch_workspace_floats() floats.  (torch.nn.Linear / LayerNorm backward, as pd_colsum_bf16.) */
+int pd_colsum_batch_workspace_floats(int n_jobs, const int* is_bf16, const int* N, int splits, uint64_t* floats);
+int pd_colsum_batch(int n_jobs, const void* const* x, const int* is_bf16, float* const* out, const uint64_t* M,
+                    const int* N, const uint64_t* ld, const float* beta, float* workspace,
+                    uint64_t workspace_floats, int splits, void* stream);
 
 /* The label-smoothing criterion of the translation stages, LabelSmoothing.forward
  * (runtime/translation/seq2seq/train/smoothing.py:23-34): logits [R][V] (R = seq*batch rows of leading

@@ -115,6 +115,8 @@ SIGNATURES = {
     "pd_cast_f32_to_bf16": (_i, [_vp, _vp, _u64, _vp], True),
     "pd_cast_bf16_to_f32": (_i, [_vp, _vp, _u64, _vp], True),
     "pd_colsum_bf16": (_i, [_vp, _vp, _u64, _i, _u64, _i, _vp], True),
+    "pd_colsum_batch_workspace_floats": (_i, [_i, _vp, _vp, _i, ctypes.POINTER(_u64)], True),
+    "pd_colsum_batch": (_i, [_i, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _u64, _i, _vp], True),
     "pd_label_smoothing_fwd_f32": (_i, [_vp, _vp, _vp, _vp, _vp, _i, _i, _i64, _i64, _f, _f, _vp], True),
     "pd_label_smoothing_bwd_f32": (_i, [_vp, _vp, _vp, _vp, _vp, _i, _i, _i64, _i64, _i64, _f, _f, _vp], True),
     "pd_revert_varlen": (_i, [_vp, _vp, _vp, _i64, _i64, _i64, _i64, _i64, _vp], True),

@@ -459,6 +459,151 @@ extern "C" int pd_cast_bf16_to_f32(const uint16_t* x, float* y, uint64_t n, void
     return PD_OK;
 }
 
+namespace {
+
+// Several column sums in two launches (the bias and LayerNorm parameter gradients of one transformer
+// layer's backward: twelve launches of a few microseconds each otherwise).  A job is a bf16 matrix [M][N]
+// (first launch: fp32 partials of `splits` row ranges, as colsum_bf16_kernel; second launch: their sum)
+// or an fp32 matrix of partials that only needs the second launch.  out = sum (+ beta * out).
+constexpr int CB_MAX_JOBS = 8;
+struct ColsumJob {
+    const void* x;       // bf16 [M][ld] or fp32 [M][ld]
+    float* part;         // bf16 jobs: [splits][N]
+    float* out;          // [N]
+    uint64_t M, ld;
+    int N;
+    int is_bf16;
+    float beta;
+    int tile1, tile2;    // first block of the job in the first (512 columns a block) / second (64) launch
+};
+struct ColsumBatch {
+    ColsumJob job[CB_MAX_JOBS];
+    int n;
+};
+
+__global__ __launch_bounds__(TR_THREADS) void colsum_batch_partial_kernel(const ColsumBatch b) {
+    __shared__ float part[4][512];
+    int j = 0;
+#pragma unroll
+    for (int q = 1; q < CB_MAX_JOBS; ++q) j += (q < b.n && (int)blockIdx.x >= b.job[q].tile1) ? 1 : 0;
+    const ColsumJob& job = b.job[j];          // (jobs without a first launch have an empty tile range)
+    const uint16_t* x = (const uint16_t*)job.x;
+    const int N = job.N;
+    const uint64_t M = job.M, ld = job.ld;
+    const int lane = threadIdx.x % 64, w = threadIdx.x / 64;
+    const int col0 = ((int)blockIdx.x - job.tile1) * 512;
+    const int col = col0 + lane * 8;
+    const uint64_t rows_per = (M + gridDim.y - 1) / gridDim.y;
+    const uint64_t r0 = blockIdx.y * rows_per;
+    const uint64_t r1 = (r0 + rows_per < M) ? r0 + rows_per : M;
+    const bool vec = ((uintptr_t)x & 15) == 0 && ld % 8 == 0;
+    float s[8];
+#pragma unroll
+    for (int k = 0; k < 8; ++k) s[k] = 0.f;
+    if (vec && col + 8 <= N) {
+        for (uint64_t r = r0 + w; r < r1; r += 4) {
+            const u16x8 v = *(const u16x8*)(x + r * ld + col);
+#pragma unroll
+            for (int k = 0; k < 8; ++k) s[k] += bf2f(v[k]);
+        }
+    } else {
+        for (uint64_t r = r0 + w; r < r1; r += 4)
+#pragma unroll
+            for (int k = 0; k < 8; ++k)
+                if (col + k < N) s[k] += bf2f(x[r * ld + col + k]);
+    }
+#pragma unroll
+    for (int k = 0; k < 8; ++k) part[w][lane * 8 + k] = s[k];
+    __syncthreads();
+    for (int c = threadIdx.x; c < 512; c += TR_THREADS) {
+        const int gc = col0 + c;
+        if (gc < N) job.part[(uint64_t)blockIdx.y * N + gc] = (part[0][c] + part[1][c]) + (part[2][c] + part[3][c]);
+    }
+}
+
+__global__ __launch_bounds__(TR_THREADS) void colsum_batch_final_kernel(const ColsumBatch b, int splits) {
+    __shared__ float part[4][64];
+    int j = 0;
+#pragma unroll
+    for (int q = 1; q < CB_MAX_JOBS; ++q) j += (q < b.n && (int)blockIdx.x >= b.job[q].tile2) ? 1 : 0;
+    const ColsumJob& job = b.job[j];
+    const float* x = job.is_bf16 ? job.part : (const float*)job.x;
+    const uint64_t M = job.is_bf16 ? (uint64_t)splits : job.M, ld = job.is_bf16 ? (uint64_t)job.N : job.ld;
+    const int N = job.N;
+    const int col = ((int)blockIdx.x - job.tile2) * 64 + threadIdx.x % 64;
+    const int w = threadIdx.x / 64;
+    float s = 0.f;
+    if (col < N) {
+        float t[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+        uint64_t r = w;
+        for (; r + 28 < M; r += 32)
+#pragma unroll
+            for (int u = 0; u < 8; ++u) t[u] += x[(r + 4 * u) * ld + col];
+        for (; r < M; r += 4) t[0] += x[r * ld + col];
+        s = ((t[0] + t[1]) + (t[2] + t[3])) + ((t[4] + t[5]) + (t[6] + t[7]));
+    }
+    part[w][threadIdx.x % 64] = s;
+    __syncthreads();
+    if (w == 0 && col < N) {
+        const float t = (part[0][threadIdx.x] + part[1][threadIdx.x]) + (part[2][threadIdx.x] + part[3][threadIdx.x]);
+        float* o = job.out + col;
+        *o = job.beta != 0.f ? t + job.beta * *o : t;
+    }
+}
+
+}  // namespace
+
+extern "C" int pd_colsum_batch_workspace_floats(int n_jobs, const int* is_bf16, const int* N, int splits,
+                                                uint64_t* floats) {
+    PD_REQUIRE(floats && (n_jobs == 0 || (is_bf16 && N)), PD_EINVAL, "pd_colsum_batch_workspace_floats: NULL pointer");
+    PD_REQUIRE(n_jobs >= 0 && n_jobs <= CB_MAX_JOBS && splits >= 1 && splits <= 65535, PD_ESHAPE,
+               "pd_colsum_batch_workspace_floats: at most %d jobs, 1..65535 splits", CB_MAX_JOBS);
+    uint64_t total = 0;
+    for (int j = 0; j < n_jobs; ++j)
+        if (is_bf16[j]) total += (uint64_t)splits * (uint64_t)(N[j] > 0 ? N[j] : 0);
+    *floats = total;
+    return PD_OK;
+}
+
+extern "C" int pd_colsum_batch(int n_jobs, const void* const* x, const int* is_bf16, float* const* out,
+                               const uint64_t* M, const int* N, const uint64_t* ld, const float* beta,
+                               float* workspace, uint64_t workspace_floats, int splits, void* stream) {
+    const char* who = "pd_colsum_batch";
+    if (n_jobs == 0) return PD_OK;
+    PD_REQUIRE(n_jobs > 0 && n_jobs <= CB_MAX_JOBS && splits >= 1 && splits <= 65535, PD_ESHAPE,
+               "%s: at most %d jobs, 1..65535 splits", who, CB_MAX_JOBS);
+    PD_REQUIRE(x && is_bf16 && out && M && N && ld && beta, PD_EINVAL, "%s: NULL argument array", who);
+    ColsumBatch b;
+    b.n = n_jobs;
+    uint64_t used = 0;
+    int tiles1 = 0, tiles2 = 0;
+    for (int j = 0; j < n_jobs; ++j) {
+        PD_REQUIRE(x[j] && out[j], PD_EINVAL, "%s: NULL operand in job %d", who, j);
+        PD_REQUIRE(N[j] > 0 && M[j] > 0 && ld[j] >= (uint64_t)N[j], PD_ESHAPE, "%s: bad shape in job %d", who, j);
+        ColsumJob& job = b.job[j];
+        job.x = x[j]; job.out = out[j]; job.M = M[j]; job.ld = ld[j]; job.N = N[j];
+        job.is_bf16 = is_bf16[j] != 0; job.beta = beta[j];
+        job.part = nullptr;
+        job.tile1 = tiles1; job.tile2 = tiles2;
+        if (job.is_bf16) {
+            job.part = workspace + used;
+            used += (uint64_t)splits * N[j];
+            tiles1 += (N[j] + 511) / 512;
+        }
+        tiles2 += (N[j] + 63) / 64;
+    }
+    PD_REQUIRE(used == 0 || (workspace && workspace_floats >= used), PD_EINVAL,
+               "%s: workspace too small (%llu < %llu floats)", who, (unsigned long long)workspace_floats,
+               (unsigned long long)used);
+    if (tiles1 > 0) {
+        colsum_batch_partial_kernel<<<dim3(tiles1, splits), dim3(TR_THREADS), 0, (hipStream_t)stream>>>(b);
+        PD_CHECK_LAUNCH(who);
+    }
+    colsum_batch_final_kernel<<<dim3(tiles2), dim3(TR_THREADS), 0, (hipStream_t)stream>>>(b, splits);
+    PD_CHECK_LAUNCH(who);
+    return PD_OK;
+}
+
 extern "C" int pd_colsum_bf16(const uint16_t* x, float* out, uint64_t M, int N, uint64_t ld, int splits, void* stream) {
     PD_REQUIRE(N >= 0 && splits >= 1 && splits <= 65535, PD_ESHAPE, "pd_colsum_bf16: bad N or splits");
     if (N == 0) return PD_OK;

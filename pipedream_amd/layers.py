@@ -583,21 +583,28 @@ class _TransformerLayerFn(torch.autograd.Function):
         ln1_w, ln1_b, qkv_w, qkv_b, o_w, o_b, ln2_w, ln2_b, fc1_w, fc1_b, fc2_w, fc2_b = ctx.params
         bw = ops.bf16_weight
         dy2 = dy.contiguous().view(B * S, H)
+        sums = ops.ColsumBatch()
 
         def linear_backward(d_out, inp, w, b):
             # parameters are read (and their bf16 image taken) at backward time: the version
             # load_old_params made current
             _accumulate(w, lambda: ops.gemm_bf16(d_out, inp, trans_a=True, out_f32=True),
                         lambda acc: ops.gemm_bf16(d_out, inp, trans_a=True, out=acc, beta=1.0))
-            _accumulate(b, lambda: ops.colsum_bf16(d_out), lambda acc: ops.colsum_bf16(d_out, acc))
+            # (the bias gradient, a column sum of d_out, waits for the end of the layer: all column sums of
+            # the layer's backward then take two launches)
+            if b.grad is None:
+                b.grad = torch.empty(b.shape, dtype=torch.float32, device=d_out.device)
+                sums.add(d_out, b.grad, 0.0)
+            else:
+                sums.add(d_out, b.grad, 1.0)
             return ops.gemm_bf16(d_out, bw(w))
 
         def layernorm_backward(d_out, inp, w, b, mean, rstd):
             if w.grad is None:
-                dx, dg, db = ops.layernorm_backward(d_out, inp, w, mean, rstd)
+                dx, dg, db = ops.layernorm_backward(d_out, inp, w, mean, rstd, batch=sums)
                 w.grad, b.grad = dg, db
             else:
-                dx, _, _ = ops.layernorm_backward(d_out, inp, w, mean, rstd, w.grad, b.grad)
+                dx, _, _ = ops.layernorm_backward(d_out, inp, w, mean, rstd, w.grad, b.grad, batch=sums)
             return dx
 
         # y = fc2(gelu(fc1(LN2(x2)))) + x2
@@ -610,6 +617,7 @@ class _TransformerLayerFn(torch.autograd.Function):
         dqkv = ops.attention_backward(datt, qkv, att_aux, B, S, heads, ctx=att)
         dh1 = linear_backward(dqkv, h1, qkv_w, qkv_b)
         dx = ops.add_bf16(layernorm_backward(dh1, x2d, ln1_w, ln1_b, mean1, rstd1), dx2)
+        sums.run()
         return (dx.view(B, S, H), None, None) + (None,) * 12
 
 

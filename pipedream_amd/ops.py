@@ -863,8 +863,9 @@ def layernorm_forward(x, gamma, beta, eps=1e-5):
     return y, mean, rstd
 
 
-def layernorm_backward(dy, x, gamma, mean, rstd, dgamma_acc=None, dbeta_acc=None):
-    """Returns dx; dgamma/dbeta are added to the given fp32 accumulators or returned fresh."""
+def layernorm_backward(dy, x, gamma, mean, rstd, dgamma_acc=None, dbeta_acc=None, batch=None):
+    """Returns dx; dgamma/dbeta are added to the given fp32 accumulators or returned fresh.  With a
+    ``ColsumBatch`` the sums over the kernel's partial results are left to the batch's ``run``."""
     M, H = x.shape
     lib = _cabi.lib()
     nb = lib.pd_layernorm_bwd_partials(M)
@@ -875,11 +876,13 @@ def layernorm_backward(dy, x, gamma, mean, rstd, dgamma_acc=None, dbeta_acc=None
                               M, H, _cabi.stream_ptr())
     outs = []
     for part, acc in ((pg, dgamma_acc), (pb, dbeta_acc)):
+        beta = 0.0 if acc is None else 1.0
         if acc is None:
             acc = torch.empty(H, dtype=torch.float32, device=x.device)
-            lib.pd_colsum_f32(_ptr(part), _ptr(acc), nb, H, H, 1, 0.0, _cabi.stream_ptr())
+        if batch is not None:
+            batch.add(part, acc, beta)
         else:
-            lib.pd_colsum_f32(_ptr(part), _ptr(acc), nb, H, H, 1, 1.0, _cabi.stream_ptr())
+            lib.pd_colsum_f32(_ptr(part), _ptr(acc), nb, H, H, 1, beta, _cabi.stream_ptr())
         outs.append(acc)
     return dx, outs[0], outs[1]
 
@@ -900,6 +903,48 @@ def add_bf16(a, b):
     y = torch.empty_like(a)
     _cabi.lib().pd_add_bf16(_ptr(a), _ptr(b), _ptr(y), a.numel(), _cabi.stream_ptr())
     return y
+
+
+class ColsumBatch(object):
+    """Column sums collected during a backward pass and computed together in two launches: ``add`` a bf16
+    matrix (a Linear layer's output gradient) or an fp32 matrix of partial sums with the fp32 vector that
+    receives (``beta=0``) or accumulates (``beta=1``) its column sums, then ``run`` once.  The matrices must
+    stay alive until ``run``."""
+    MAX_JOBS = 8
+    SPLITS = 64
+
+    def __init__(self):
+        self.jobs = []
+
+    def add(self, x, out, beta):
+        if x.dim() != 2 or x.stride(1) != 1 or x.dtype not in (BF16, torch.float32):
+            raise ValueError("ColsumBatch.add: x must be a row-major bf16 or fp32 matrix")
+        if out.dtype != torch.float32 or out.numel() != x.shape[1] or not out.is_contiguous():
+            raise ValueError("ColsumBatch.add: out must be a contiguous fp32 vector of x's column count")
+        _cabi.require_device(x, "x")
+        _cabi.require_device(out, "out")
+        self.jobs.append((x, out, float(beta)))
+        if len(self.jobs) == self.MAX_JOBS:
+            self.run()
+
+    def run(self):
+        jobs, self.jobs = self.jobs, []
+        n = len(jobs)
+        if n == 0:
+            return
+        lib = _cabi.lib()
+        xs = (ctypes.c_void_p * n)(*[j[0].data_ptr() for j in jobs])
+        outs = (ctypes.c_void_p * n)(*[j[1].data_ptr() for j in jobs])
+        kinds = (ctypes.c_int * n)(*[1 if j[0].dtype == BF16 else 0 for j in jobs])
+        ms = (ctypes.c_uint64 * n)(*[j[0].shape[0] for j in jobs])
+        ns = (ctypes.c_int * n)(*[j[0].shape[1] for j in jobs])
+        lds = (ctypes.c_uint64 * n)(*[j[0].stride(0) if j[0].shape[0] > 1 else j[0].shape[1] for j in jobs])
+        betas = (ctypes.c_float * n)(*[j[2] for j in jobs])
+        need = ctypes.c_uint64()
+        lib.pd_colsum_batch_workspace_floats(n, kinds, ns, self.SPLITS, ctypes.byref(need))
+        ws = torch.empty(max(need.value, 1), dtype=torch.float32, device=jobs[0][0].device)
+        lib.pd_colsum_batch(n, xs, kinds, outs, ms, ns, lds, betas, _ptr(ws), need.value, self.SPLITS,
+                            _cabi.stream_ptr())
 
 
 def colsum_bf16(x, acc=None):

@@ -303,3 +303,31 @@ def test_full_size_layer_properties():
     grads = dict((k, p.grad) for k, p in mine.named_parameters())
     for k, p in ref.named_parameters():
         assert _rel(grads[k], p.grad) < 2e-2, (k, _rel(grads[k], p.grad))
+
+
+def test_batched_column_sums_match_the_single_ones():
+    """``ops.ColsumBatch``: bf16 matrices (odd and unaligned shapes among them) and fp32 partial-sum matrices in
+    one batch, fresh outputs and accumulation, against fp64 sums; nine jobs, so the batch runs twice."""
+    from pipedream_amd import ops
+    torch.manual_seed(3)
+    shapes = [(4096, 1024, True), (4096, 3072, True), (37, 1000, True), (513, 72, True), (16, 1024, False),
+              (40, 1024, False), (4096, 4096, True), (5, 3, True), (7, 130, False)]
+    batch = ops.ColsumBatch()
+    checks = []
+    for i, (M, N, is_bf16) in enumerate(shapes):
+        x = torch.randn(M, N, device="cuda")
+        x = x.to(torch.bfloat16) if is_bf16 else x
+        if i % 2:
+            out = torch.randn(N, device="cuda")
+            want = out.double().cpu() + x.double().sum(0).cpu()
+            batch.add(x, out, 1.0)
+        else:
+            out = torch.full((N,), float("nan"), device="cuda")
+            want = x.double().sum(0).cpu()
+            batch.add(x, out, 0.0)
+        checks.append((out, want, M))
+    batch.run()
+    for out, want, M in checks:
+        torch.testing.assert_close(out.double().cpu(), want, rtol=1e-5, atol=2e-6 * M)
+    with pytest.raises(ValueError):
+        batch.add(torch.zeros(4, 4, device="cuda"), torch.zeros(3, device="cuda"), 0.0)
