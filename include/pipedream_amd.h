@@ -336,14 +336,15 @@ int pd_gemm_bf16(int trans_a, int trans_b, int M, int N, int K,
                  int batch_outer, int batch_inner, const int64_t* strides, void* stream);
 
 /* LayerNorm over the last dimension H (multiple of 8, <= 2048): bf16 in/out, fp32 affine
- * parameters and statistics.  Backward writes dx and per-block partial sums of
- * dgamma / dbeta, [pd_layernorm_bwd_partials(M)][H] each, to be summed with pd_colsum_f32. */
+ * parameters and statistics.  Backward writes dx (+ residual, bf16 [M][H] or NULL: the gradient that
+ * bypasses the normalisation in a pre-LN layer, dx = LN'(dy) + residual) and per-block partial sums of
+ * dgamma / dbeta, [pd_layernorm_bwd_partials(M)][H] each, to be summed with pd_colsum_f32 or pd_colsum_batch. */
 int pd_layernorm_fwd_bf16(const uint16_t* x, const float* gamma, const float* beta, uint16_t* y,
                           float* mean, float* rstd, int M, int H, float eps, void* stream);
 int pd_layernorm_bwd_partials(int M);
 int pd_layernorm_bwd_bf16(const uint16_t* dy, const uint16_t* x, const float* gamma, const float* mean,
-                          const float* rstd, uint16_t* dx, float* part_dgamma, float* part_dbeta,
-                          int M, int H, void* stream);
+                          const float* rstd, uint16_t* dx, const uint16_t* residual, float* part_dgamma,
+                          float* part_dbeta, int M, int H, void* stream);
 
 /* Fused attention of one transformer layer.  qkv is [batch*seq][3H] (Q | K | V, the heads contiguous
  * inside each, H = heads*head_dim).  Forward: ctx [batch*seq][H] = softmax(Q K^T / sqrt(head_dim)) V; the

@@ -103,7 +103,7 @@ SIGNATURES = {
                           ctypes.POINTER(ctypes.c_int64), _vp], True),
     "pd_layernorm_fwd_bf16": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _f, _vp], True),
     "pd_layernorm_bwd_partials": (_i, [_i], False),
-    "pd_layernorm_bwd_bf16": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _vp], True),
+    "pd_layernorm_bwd_bf16": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _vp], True),
     "pd_attention_fwd_supported": (_i, [_i, _i], False),
     "pd_attention_fwd_bf16": (_i, [_vp, _vp, _vp, _vp, _i, _i, _i, _i, _vp], True),
     "pd_attention_bwd_bf16": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _vp], True),

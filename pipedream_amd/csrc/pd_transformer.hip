@@ -117,6 +117,7 @@ __global__ __launch_bounds__(TR_THREADS) void layernorm_bwd_kernel(const uint16_
                                                                    const float* __restrict__ mean,
                                                                    const float* __restrict__ rstd,
                                                                    uint16_t* __restrict__ dx,
+                                                                   const uint16_t* __restrict__ residual,
                                                                    float* __restrict__ part_dgamma,
                                                                    float* __restrict__ part_dbeta, int M, int H) {
     extern __shared__ float red[];   // [2][4][H]
@@ -161,6 +162,11 @@ __global__ __launch_bounds__(TR_THREADS) void layernorm_bwd_kernel(const uint16_
                 for (int k = 0; k < 8; ++k) {
                     const float xh = (rx.x[v][k] - mu) * rs;
                     o[k] = rs * (gamma[e + k] * rd.x[v][k] - s1 - xh * s2);
+                }
+                if (residual) {       // the gradient that reaches the layer's input past the normalisation
+                    const u16x8 r = *(const u16x8*)(residual + (size_t)row * H + e);
+#pragma unroll
+                    for (int k = 0; k < 8; ++k) o[k] += bf2f(r[k]);
                 }
                 store_row(dx + (size_t)row * H, H, lane, v, o);
             }
@@ -370,13 +376,13 @@ extern "C" int pd_layernorm_fwd_bf16(const uint16_t* x, const float* gamma, cons
 extern "C" int pd_layernorm_bwd_partials(int M) { return (M + LN_ROWS_PER_BLOCK - 1) / LN_ROWS_PER_BLOCK; }
 
 extern "C" int pd_layernorm_bwd_bf16(const uint16_t* dy, const uint16_t* x, const float* gamma, const float* mean,
-                                     const float* rstd, uint16_t* dx, float* part_dgamma, float* part_dbeta, int M,
-                                     int H, void* stream) {
+                                     const float* rstd, uint16_t* dx, const uint16_t* residual, float* part_dgamma,
+                                     float* part_dbeta, int M, int H, void* stream) {
     int rc = row_args_ok("pd_layernorm_bwd_bf16", M, H);
     if (rc != PD_OK) return rc;
     PD_REQUIRE(dy && x && gamma && mean && rstd && dx && part_dgamma && part_dbeta, PD_EINVAL,
                "pd_layernorm_bwd_bf16: NULL pointer");
-    PD_REQUIRE(pd_aligned(x, 16) && pd_aligned(dy, 16) && pd_aligned(dx, 16), PD_EINVAL,
+    PD_REQUIRE(pd_aligned(x, 16) && pd_aligned(dy, 16) && pd_aligned(dx, 16) && pd_aligned(residual, 16), PD_EINVAL,
                "pd_layernorm_bwd_bf16: 16-byte alignment");
     const size_t lds = (size_t)8 * H * sizeof(float);
     PD_REQUIRE(lds <= 160 * 1024, PD_ESHAPE, "pd_layernorm_bwd_bf16: H too large for the LDS reduction");
@@ -384,7 +390,7 @@ extern "C" int pd_layernorm_bwd_bf16(const uint16_t* dy, const uint16_t* x, cons
         PD_HIP(hipFuncSetAttribute((const void*)layernorm_bwd_kernel, hipFuncAttributeMaxDynamicSharedMemorySize,
                                    (int)lds));
     layernorm_bwd_kernel<<<dim3(pd_layernorm_bwd_partials(M)), dim3(TR_THREADS), lds, (hipStream_t)stream>>>(
-        dy, x, gamma, mean, rstd, dx, part_dgamma, part_dbeta, M, H);
+        dy, x, gamma, mean, rstd, dx, residual, part_dgamma, part_dbeta, M, H);
     PD_CHECK_LAUNCH("pd_layernorm_bwd_bf16");
     return PD_OK;
 }

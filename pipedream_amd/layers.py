@@ -599,24 +599,26 @@ class _TransformerLayerFn(torch.autograd.Function):
                 sums.add(d_out, b.grad, 1.0)
             return ops.gemm_bf16(d_out, bw(w))
 
-        def layernorm_backward(d_out, inp, w, b, mean, rstd):
+        def layernorm_backward(d_out, inp, w, b, mean, rstd, residual):
+            # (+ residual: the branch of the gradient that bypasses the normalisation, added as dx is stored)
             if w.grad is None:
-                dx, dg, db = ops.layernorm_backward(d_out, inp, w, mean, rstd, batch=sums)
+                dx, dg, db = ops.layernorm_backward(d_out, inp, w, mean, rstd, batch=sums, residual=residual)
                 w.grad, b.grad = dg, db
             else:
-                dx, _, _ = ops.layernorm_backward(d_out, inp, w, mean, rstd, w.grad, b.grad, batch=sums)
+                dx, _, _ = ops.layernorm_backward(d_out, inp, w, mean, rstd, w.grad, b.grad, batch=sums,
+                                                  residual=residual)
             return dx
 
         # y = fc2(gelu(fc1(LN2(x2)))) + x2
         dg = linear_backward(dy2, g, fc2_w, fc2_b)
         df = ops.gelu_backward(f, dg)
         dh2 = linear_backward(df, h2, fc1_w, fc1_b)
-        dx2 = ops.add_bf16(layernorm_backward(dh2, x2, ln2_w, ln2_b, mean2, rstd2), dy2)
+        dx2 = layernorm_backward(dh2, x2, ln2_w, ln2_b, mean2, rstd2, dy2)
         # x2 = o(attn(qkv(LN1(x)))) + x
         datt = linear_backward(dx2, att, o_w, o_b)
         dqkv = ops.attention_backward(datt, qkv, att_aux, B, S, heads, ctx=att)
         dh1 = linear_backward(dqkv, h1, qkv_w, qkv_b)
-        dx = ops.add_bf16(layernorm_backward(dh1, x2d, ln1_w, ln1_b, mean1, rstd1), dx2)
+        dx = layernorm_backward(dh1, x2d, ln1_w, ln1_b, mean1, rstd1, dx2)
         sums.run()
         return (dx.view(B, S, H), None, None) + (None,) * 12
 

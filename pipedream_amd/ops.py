@@ -863,17 +863,22 @@ def layernorm_forward(x, gamma, beta, eps=1e-5):
     return y, mean, rstd
 
 
-def layernorm_backward(dy, x, gamma, mean, rstd, dgamma_acc=None, dbeta_acc=None, batch=None):
-    """Returns dx; dgamma/dbeta are added to the given fp32 accumulators or returned fresh.  With a
-    ``ColsumBatch`` the sums over the kernel's partial results are left to the batch's ``run``."""
+def layernorm_backward(dy, x, gamma, mean, rstd, dgamma_acc=None, dbeta_acc=None, batch=None, residual=None):
+    """Returns dx (+ ``residual``, a bf16 matrix of x's shape); dgamma/dbeta are added to the given fp32
+    accumulators or returned fresh.  With a ``ColsumBatch`` the sums over the kernel's partial results are
+    left to the batch's ``run``."""
+    if residual is not None:
+        _mat_bf16(residual, "residual")
+        if residual.shape != x.shape or not residual.is_contiguous():
+            raise ValueError("layernorm_backward: residual must be a contiguous matrix of x's shape")
     M, H = x.shape
     lib = _cabi.lib()
     nb = lib.pd_layernorm_bwd_partials(M)
     dx = torch.empty_like(x)
     pg = torch.empty((nb, H), dtype=torch.float32, device=x.device)
     pb = torch.empty((nb, H), dtype=torch.float32, device=x.device)
-    lib.pd_layernorm_bwd_bf16(_ptr(dy), _ptr(x), _ptr(gamma), _ptr(mean), _ptr(rstd), _ptr(dx), _ptr(pg), _ptr(pb),
-                              M, H, _cabi.stream_ptr())
+    lib.pd_layernorm_bwd_bf16(_ptr(dy), _ptr(x), _ptr(gamma), _ptr(mean), _ptr(rstd), _ptr(dx), _ptr(residual),
+                              _ptr(pg), _ptr(pb), M, H, _cabi.stream_ptr())
     outs = []
     for part, acc in ((pg, dgamma_acc), (pb, dbeta_acc)):
         beta = 0.0 if acc is None else 1.0

@@ -171,6 +171,13 @@ def test_layernorm_softmax_gelu_vs_torch():
     acc_g, acc_b = torch.ones(256).cuda(), torch.ones(256).cuda()
     ops.layernorm_backward(dy.cuda(), x.cuda(), gamma.cuda(), mean, rstd, acc_g, acc_b)
     assert _rel(acc_g, gf.grad + 1) < 1e-5 and _rel(acc_b, bf.grad + 1) < 1e-5
+    # with the residual branch of a pre-LN layer added as dx is stored, and the parameter sums left to a batch
+    res = torch.randn(70, 256, generator=g).to(BF)
+    batch = ops.ColsumBatch()
+    dxr, dg2, db2 = ops.layernorm_backward(dy.cuda(), x.cuda(), gamma.cuda(), mean, rstd, batch=batch,
+                                           residual=res.cuda())
+    batch.run()
+    assert _rel(dxr, xf.grad + res.float()) < 4e-3 and _rel(dg2, gf.grad) < 1e-5 and _rel(db2, bf.grad) < 1e-5
 
     from pipedream_amd import _cabi
     import ctypes
