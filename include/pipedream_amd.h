@@ -334,6 +334,15 @@ int pd_gemm_bf16(int trans_a, int trans_b, int M, int N, int K,
                  void* C, int ldc, int out_f32, float alpha, float beta,
                  const float* bias, const uint16_t* residual, int ldr,
                  int batch_outer, int batch_inner, const int64_t* strides, void* stream);
+/* The same GEMM (unbatched, bf16 output) with the exact GELU of a feed-forward block in its epilogue.
+ * backward = 0:  C = op(A) op(B) + bias  (the pre-activation, kept for the backward) and aux = gelu(C),
+ *                with C taken as rounded to bf16, both written by the kernel;
+ * backward = 1:  C = (op(A) op(B)) * gelu'(aux), aux = the stored pre-activation: the gradient with respect
+ *                to it, straight from the GEMM that produces the gradient of the activation.
+ * aux is [M][ld_aux] bf16.  erf is evaluated by Abramowitz & Stegun 7.1.26 (absolute error < 1.5e-7). */
+int pd_gemm_bf16_gelu(int backward, int trans_a, int trans_b, int M, int N, int K, const uint16_t* A, int lda,
+                      const uint16_t* B, int ldb, uint16_t* C, int ldc, const float* bias, uint16_t* aux,
+                      int ld_aux, void* stream);
 
 /* LayerNorm over the last dimension H (multiple of 8, <= 2048): bf16 in/out, fp32 affine
  * parameters and statistics.  Backward writes dx (+ residual, bf16 [M][H] or NULL: the gradient that

@@ -61,8 +61,31 @@ struct GemmBf16Args {
     float beta;                 // fp32 output: C = alpha*acc + beta*C
     int out_f32;
     int tiles_m, tiles_n, total_tiles, tiles_per_xcd;
-    int vec_store;              // C (and residual) can be written with 16-byte vectors
+    int vec_store;              // C (and residual, aux) can be written with 16-byte vectors
+    // GELU in the epilogue (bf16 output): act 1 = forward, also stores aux_out = gelu(C) (C as rounded to
+    // bf16, which is what the backward reads); act 2 = backward, C = value * gelu'(aux_in)
+    int act;
+    uint16_t* aux_out;          // [M][ld_aux]
+    const uint16_t* aux_in;     // [M][ld_aux]
+    int ld_aux;
 };
+
+// erf by Abramowitz & Stegun 7.1.26 (absolute error below 1.5e-7, far inside a bf16 result's rounding): a
+// few multiply-adds, one reciprocal and one exponential, instead of the library erff, whose register demand
+// inside the 256 x 256 kernels' epilogue (all 256 registers hold accumulators there) spilled a kilobyte per lane.
+__device__ __forceinline__ float erf_as(float x) {
+    const float ax = fabsf(x);
+    const float t = __builtin_amdgcn_rcpf(1.0f + 0.3275911f * ax);
+    const float poly = t * (0.254829592f + t * (-0.284496736f + t * (1.421413741f + t * (-1.453152027f + t * 1.061405429f))));
+    const float r = 1.0f - poly * __expf(-ax * ax);
+    return x < 0.f ? -r : r;
+}
+__device__ __forceinline__ float gelu_f(float x) { return 0.5f * x * (1.0f + erf_as(x * 0.70710678118654752f)); }
+__device__ __forceinline__ float gelu_grad_f(float x) {
+    const float cdf = 0.5f * (1.0f + erf_as(x * 0.70710678118654752f));
+    const float pdf = 0.39894228040143268f * __expf(-0.5f * x * x);
+    return cdf + x * pdf;
+}
 
 __device__ __forceinline__ uint16_t f2bf(float f) { return pd_f2bf(f); }
 __device__ __forceinline__ float bf2f(uint16_t h) { return __uint_as_float((uint32_t)h << 16); }
@@ -102,7 +125,10 @@ __device__ __forceinline__ void store_tile(const GemmBf16Args& a, float16_t (&ac
                         *p = v;
                     } else {
                         if (a.residual) v += bf2f(a.residual[c_off + (long long)row * a.ldr + col]);
-                        ((uint16_t*)a.C)[off] = f2bf(v);
+                        if (a.act == 2) v *= gelu_grad_f(bf2f(a.aux_in[(long long)row * a.ld_aux + col]));
+                        const uint16_t o = f2bf(v);
+                        ((uint16_t*)a.C)[off] = o;
+                        if (a.act == 1) a.aux_out[(long long)row * a.ld_aux + col] = f2bf(gelu_f(bf2f(o)));
                     }
                 }
             }
@@ -152,10 +178,21 @@ __device__ __forceinline__ void store_tile(const GemmBf16Args& a, float16_t (&ac
 #pragma unroll
                         for (int q = 0; q < 8; ++q) v[q] += bf2f(rr[q]);
                     }
+                    if (a.act == 2) {
+                        const u16x8 xx = *(const u16x8*)(a.aux_in + (long long)row * a.ld_aux + col);
+#pragma unroll
+                        for (int q = 0; q < 8; ++q) v[q] *= gelu_grad_f(bf2f(xx[q]));
+                    }
                     u16x8 o;
 #pragma unroll
                     for (int q = 0; q < 8; ++q) o[q] = f2bf(v[q]);
                     *(u16x8*)((uint16_t*)a.C + c_off + (long long)row * a.ldc + col) = o;
+                    if (a.act == 1) {
+                        u16x8 gg;
+#pragma unroll
+                        for (int q = 0; q < 8; ++q) gg[q] = f2bf(gelu_f(bf2f(o[q])));
+                        *(u16x8*)(a.aux_out + (long long)row * a.ld_aux + col) = gg;
+                    }
                 }
             }
         }
@@ -651,10 +688,11 @@ int launch_gemm_bf16(int ta, int tb, GemmBf16Args g, int batch, hipStream_t s) {
 
 }  // namespace
 
-extern "C" int pd_gemm_bf16(int trans_a, int trans_b, int M, int N, int K, const uint16_t* A, int lda,
-                            const uint16_t* B, int ldb, void* C, int ldc, int out_f32, float alpha, float beta,
-                            const float* bias, const uint16_t* residual, int ldr, int batch_outer, int batch_inner,
-                            const int64_t* strides /* sa_o, sa_i, sb_o, sb_i, sc_o, sc_i or NULL */, void* stream) {
+static int gemm_bf16_run(int trans_a, int trans_b, int M, int N, int K, const uint16_t* A, int lda,
+                         const uint16_t* B, int ldb, void* C, int ldc, int out_f32, float alpha, float beta,
+                         const float* bias, const uint16_t* residual, int ldr, int batch_outer, int batch_inner,
+                         const int64_t* strides, void* stream, int act, uint16_t* aux_out, const uint16_t* aux_in,
+                         int ld_aux) {
     PD_REQUIRE(M >= 0 && N >= 0 && K >= 0 && batch_outer >= 1 && batch_inner >= 1, PD_ESHAPE,
                "pd_gemm_bf16: bad dimensions");
     if (M == 0 || N == 0) return PD_OK;
@@ -685,8 +723,10 @@ extern "C" int pd_gemm_bf16(int trans_a, int trans_b, int M, int N, int K, const
     g.alpha = alpha;
     g.beta = beta;
     g.out_f32 = out_f32 != 0;
+    g.act = act; g.aux_out = aux_out; g.aux_in = aux_in; g.ld_aux = ld_aux;
     g.vec_store = N % 8 == 0 && ldc % 8 == 0 && pd_aligned(C, 16) && g.sc_o % 8 == 0 && g.sc_i % 8 == 0 &&
-                  (!residual || (ldr % 8 == 0 && pd_aligned(residual, 16)));
+                  (!residual || (ldr % 8 == 0 && pd_aligned(residual, 16))) &&
+                  (!act || (ld_aux % 8 == 0 && pd_aligned(act == 1 ? (const void*)aux_out : (const void*)aux_in, 16)));
     const int batch = batch_outer * batch_inner;
     hipStream_t s = (hipStream_t)stream;
     PD_REQUIRE((long long)((M + 63) / 64) * ((N + 63) / 64) * batch < (1ll << 28), PD_ESHAPE, "pd_gemm_bf16: too many tiles");
@@ -702,4 +742,21 @@ extern "C" int pd_gemm_bf16(int trans_a, int trans_b, int M, int N, int K, const
     if (N <= 64 && M >= 256) return launch_gemm_bf16<256, 64, 4, 1>(trans_a, trans_b, g, batch, s);
     if (M >= 128 && N >= 128 && tiles128 >= 128) return launch_gemm_bf16<128, 128, 2, 2>(trans_a, trans_b, g, batch, s);
     return launch_gemm_bf16<64, 64, 2, 2>(trans_a, trans_b, g, batch, s);
+}
+
+extern "C" int pd_gemm_bf16(int trans_a, int trans_b, int M, int N, int K, const uint16_t* A, int lda,
+                            const uint16_t* B, int ldb, void* C, int ldc, int out_f32, float alpha, float beta,
+                            const float* bias, const uint16_t* residual, int ldr, int batch_outer, int batch_inner,
+                            const int64_t* strides /* sa_o, sa_i, sb_o, sb_i, sc_o, sc_i or NULL */, void* stream) {
+    return gemm_bf16_run(trans_a, trans_b, M, N, K, A, lda, B, ldb, C, ldc, out_f32, alpha, beta, bias, residual, ldr,
+                         batch_outer, batch_inner, strides, stream, 0, nullptr, nullptr, 0);
+}
+
+extern "C" int pd_gemm_bf16_gelu(int backward, int trans_a, int trans_b, int M, int N, int K, const uint16_t* A,
+                                 int lda, const uint16_t* B, int ldb, uint16_t* C, int ldc, const float* bias,
+                                 uint16_t* aux, int ld_aux, void* stream) {
+    PD_REQUIRE(aux && ld_aux >= N, PD_EINVAL, "pd_gemm_bf16_gelu: aux must be an [M][ld_aux] matrix with ld_aux >= N");
+    PD_REQUIRE(!backward || !bias, PD_EINVAL, "pd_gemm_bf16_gelu: the backward form takes no bias");
+    return gemm_bf16_run(trans_a, trans_b, M, N, K, A, lda, B, ldb, C, ldc, 0, 1.0f, 0.0f, bias, nullptr, 0, 1, 1,
+                         nullptr, stream, backward ? 2 : 1, backward ? nullptr : aux, backward ? aux : nullptr, ld_aux);
 }

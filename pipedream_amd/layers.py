@@ -568,8 +568,7 @@ class _TransformerLayerFn(torch.autograd.Function):
         att, att_aux = ops.attention_forward(qkv, B, S, heads)
         x2 = ops.gemm_bf16(att, bw(o_w), trans_b=True, bias=o_b, residual=x2d)
         h2, mean2, rstd2 = ops.layernorm_forward(x2, ln2_w, ln2_b, eps)
-        f = ops.gemm_bf16(h2, bw(fc1_w), trans_b=True, bias=fc1_b)
-        g = ops.gelu(f)
+        f, g = ops.gemm_bf16_gelu(h2, bw(fc1_w), trans_b=True, bias=fc1_b)      # g = gelu(f) in the epilogue
         y = ops.gemm_bf16(g, bw(fc2_w), trans_b=True, bias=fc2_b, residual=x2)
         ctx.dims = (B, S, H, heads)
         ctx.params = (ln1_w, ln1_b, qkv_w, qkv_b, o_w, o_b, ln2_w, ln2_b, fc1_w, fc1_b, fc2_w, fc2_b)
@@ -585,7 +584,7 @@ class _TransformerLayerFn(torch.autograd.Function):
         dy2 = dy.contiguous().view(B * S, H)
         sums = ops.ColsumBatch()
 
-        def linear_backward(d_out, inp, w, b):
+        def linear_backward(d_out, inp, w, b, through_gelu_of=None):
             # parameters are read (and their bf16 image taken) at backward time: the version
             # load_old_params made current
             _accumulate(w, lambda: ops.gemm_bf16(d_out, inp, trans_a=True, out_f32=True),
@@ -597,6 +596,8 @@ class _TransformerLayerFn(torch.autograd.Function):
                 sums.add(d_out, b.grad, 0.0)
             else:
                 sums.add(d_out, b.grad, 1.0)
+            if through_gelu_of is not None:       # the input is gelu(f): return the gradient with respect to f
+                return ops.gemm_bf16_gelu_backward(d_out, bw(w), through_gelu_of)
             return ops.gemm_bf16(d_out, bw(w))
 
         def layernorm_backward(d_out, inp, w, b, mean, rstd, residual):
@@ -610,8 +611,7 @@ class _TransformerLayerFn(torch.autograd.Function):
             return dx
 
         # y = fc2(gelu(fc1(LN2(x2)))) + x2
-        dg = linear_backward(dy2, g, fc2_w, fc2_b)
-        df = ops.gelu_backward(f, dg)
+        df = linear_backward(dy2, g, fc2_w, fc2_b, through_gelu_of=f)
         dh2 = linear_backward(df, h2, fc1_w, fc1_b)
         dx2 = layernorm_backward(dh2, x2, ln2_w, ln2_b, mean2, rstd2, dy2)
         # x2 = o(attn(qkv(LN1(x)))) + x

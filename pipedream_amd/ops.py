@@ -769,6 +769,43 @@ def gemm_bf16(a, b, trans_a=False, trans_b=False, out=None, out_f32=False, alpha
     return out
 
 
+def gemm_bf16_gelu(a, b, trans_b=False, bias=None):
+    """(f, g) with f = a op(b) + bias and g = gelu(f) (f as rounded to bf16), both from the GEMM kernel's
+    epilogue: the first linear layer of a feed-forward block and its activation."""
+    _mat_bf16(a, "a")
+    _mat_bf16(b, "b")
+    M, K = a.shape
+    Kb, N = (b.size(1), b.size(0)) if trans_b else (b.size(0), b.size(1))
+    if K != Kb:
+        raise ValueError("gemm_bf16_gelu: inner dimensions differ (%d vs %d)" % (K, Kb))
+    if bias is not None:
+        _check(bias, "bias")
+    f = torch.empty((M, N), dtype=BF16, device=a.device)
+    g = torch.empty((M, N), dtype=BF16, device=a.device)
+    with _timed("gemm_bf16", 2.0 * M * N * K):
+        _cabi.lib().pd_gemm_bf16_gelu(0, 0, int(trans_b), M, N, K, _ptr(a), a.stride(0), _ptr(b), b.stride(0), _ptr(f),
+                                      N, _ptr(bias), _ptr(g), N, _cabi.stream_ptr())
+    return f, g
+
+
+def gemm_bf16_gelu_backward(dy, w, f):
+    """df = (dy w) * gelu'(f): the input gradient of the second linear layer of a feed-forward block taken
+    through the activation in the GEMM's epilogue; ``f`` is the stored pre-activation [M, N]."""
+    _mat_bf16(dy, "dy")
+    _mat_bf16(w, "w")
+    _mat_bf16(f, "f")
+    M, K = dy.shape
+    Kb, N = w.shape
+    if K != Kb or tuple(f.shape) != (M, N) or not f.is_contiguous():
+        raise ValueError("gemm_bf16_gelu_backward: shapes %s x %s -> %s do not fit"
+                         % (tuple(dy.shape), tuple(w.shape), tuple(f.shape)))
+    df = torch.empty((M, N), dtype=BF16, device=dy.device)
+    with _timed("gemm_bf16", 2.0 * M * N * K):
+        _cabi.lib().pd_gemm_bf16_gelu(1, 0, 0, M, N, K, _ptr(dy), dy.stride(0), _ptr(w), w.stride(0), _ptr(df), N, None,
+                                      _ptr(f), N, _cabi.stream_ptr())
+    return df
+
+
 def _batched(ta, tb, M, N, K, A, a_off, lda, B, b_off, ldb, C, c_off, ldc, alpha, bo, bi, strides):
     arr = (ctypes.c_int64 * 6)(*strides)
     es = 2

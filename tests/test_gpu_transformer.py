@@ -338,3 +338,27 @@ def test_batched_column_sums_match_the_single_ones():
         torch.testing.assert_close(out.double().cpu(), want, rtol=1e-5, atol=2e-6 * M)
     with pytest.raises(ValueError):
         batch.add(torch.zeros(4, 4, device="cuda"), torch.zeros(3, device="cuda"), 0.0)
+
+
+@pytest.mark.parametrize("M,N,K", [(4096, 4096, 1024), (512, 1024, 256), (200, 72, 64), (64, 8, 8)])
+def test_gemm_with_gelu_in_its_epilogue(M, N, K):
+    """``gemm_bf16_gelu`` / ``gemm_bf16_gelu_backward`` against the GEMM followed by the element-wise kernels
+    (the same operations; only the erf approximation and one bf16 rounding differ) and against torch in fp32."""
+    from pipedream_amd import ops
+    torch.manual_seed(M + N)
+    a = (torch.randn(M, K) / math.sqrt(K)).to(BF).cuda()
+    w = torch.randn(N, K).to(BF).cuda()
+    bias = torch.randn(N).cuda()
+    f, g = ops.gemm_bf16_gelu(a, w, trans_b=True, bias=bias)
+    f0 = ops.gemm_bf16(a, w, trans_b=True, bias=bias)
+    assert torch.equal(f, f0)                                     # the pre-activation is the plain GEMM's
+    assert _rel(g, ops.gelu(f0).cpu()) < 2e-3                     # bf16 steps apart at most
+    assert _rel(g, F.gelu(f0.float().cpu())) < 4e-3
+    dy = (torch.randn(M, 256) / 16).to(BF).cuda()
+    w2 = torch.randn(256, N).to(BF).cuda()
+    df = ops.gemm_bf16_gelu_backward(dy, w2, f)
+    two_step = ops.gelu_backward(f, ops.gemm_bf16(dy, w2))
+    assert _rel(df, two_step.cpu()) < 4e-3
+    ff = f.float().cpu().requires_grad_()
+    F.gelu(ff).backward(dy.float().cpu() @ w2.float().cpu())
+    assert _rel(df, ff.grad) < 6e-3
