@@ -285,7 +285,10 @@ int pd_conv3x3_wgrad_nhwc_f32(const float* x, const float* dy, const float* relu
  * holds until the process ends.  The call allocates and frees nothing.  A shape whose
  * pd_conv3x3_wgrad_workspace_bytes() exceeds that size is refused with PD_ESHAPE (the few-channel first
  * layer fits at any batch size; 64-channel layers up to about 100k pixels per call).  All calls on one
- * GPU share the array: calls that overlap on one GPU (different streams or threads) race. */
+ * GPU share the array: calls that overlap on one GPU (different streams or threads) race.
+ * The first call on a device looks up the array's device address (hipGetSymbolAddress, under a mutex)
+ * and keeps it; make that first call outside graph capture.  The address is that of the device current
+ * at the call (hipGetDevice), so `stream` must belong to the current device. */
 #define PD_CONV3X3_WGRAD_NOALLOC_MAX_WORKSPACE (16u << 20)
 int pd_conv3x3_wgrad_noalloc_nhwc_f32(const float* x, const float* dy, const float* relu_out, float* dw,
                                       float* dbias, int N, int H, int W, int C, int K, void* stream);

@@ -117,9 +117,10 @@ __device__ __forceinline__ int find_tensor(const OptArgs& a, uint32_t b) {
     return ti;
 }
 
-// MIXED: gradients (and the 16-bit parameter copy) are in a 16-bit format chosen per launch; the fp32 path
-// is its own instantiation and carries none of that.
-template <bool ADAM, bool MIXED>
+// GRAD16: gradients arrive in the 16-bit format a.grad_fmt (else fp32).  OUT_RT: the 16-bit copy of the new
+// parameters is written in the format a.out_fmt (else bf16).  The plain fp32 step is its own instantiation and
+// carries none of that.
+template <bool ADAM, bool GRAD16, bool OUT_RT>
 __global__ __launch_bounds__(OPT_THREADS) void pd_optim_kernel(const OptArgs a, const SgdHyper sh, const AdamHyper ah) {
     const int ti = find_tensor(a, blockIdx.x);
     const pd_tensor_desc& t = a.t[ti];
@@ -136,7 +137,7 @@ __global__ __launch_bounds__(OPT_THREADS) void pd_optim_kernel(const OptArgs a, 
 #pragma unroll
         for (int u = 0; u < OPT_UNROLL; ++u) {
             const uint64_t i = v0 + (uint64_t)u * OPT_THREADS;
-            if (MIXED) {
+            if (GRAD16) {
                 typedef uint16_t u16x4 __attribute__((ext_vector_type(4)));
                 const u16x4 h = __builtin_nontemporal_load((const u16x4*)t.grad + i);
 #pragma unroll
@@ -173,7 +174,7 @@ __global__ __launch_bounds__(OPT_THREADS) void pd_optim_kernel(const OptArgs a, 
             if (t.bf16_out) {
                 typedef uint16_t u16x4 __attribute__((ext_vector_type(4)));
                 u16x4 h;
-                if (MIXED) h = u16x4{f32_to_half(pn[0], a.out_fmt), f32_to_half(pn[1], a.out_fmt),
+                if (OUT_RT) h = u16x4{f32_to_half(pn[0], a.out_fmt), f32_to_half(pn[1], a.out_fmt),
                                      f32_to_half(pn[2], a.out_fmt), f32_to_half(pn[3], a.out_fmt)};
                 else h = u16x4{f32_to_bf16_rne(pn[0]), f32_to_bf16_rne(pn[1]), f32_to_bf16_rne(pn[2]), f32_to_bf16_rne(pn[3])};
                 *((u16x4*)t.bf16_out + i) = h;
@@ -184,7 +185,7 @@ __global__ __launch_bounds__(OPT_THREADS) void pd_optim_kernel(const OptArgs a, 
         for (int u = 0; u < OPT_UNROLL * 4; ++u) {
             const uint64_t i = chunk0 + (uint64_t)u * OPT_THREADS + threadIdx.x;
             if (i >= n) break;
-            float g = MIXED ? half_to_f32(((const uint16_t*)t.grad)[i], a.grad_fmt) : t.grad[i], p = t.p_in[i], pn;
+            float g = GRAD16 ? half_to_f32(((const uint16_t*)t.grad)[i], a.grad_fmt) : t.grad[i], p = t.p_in[i], pn;
             if (ADAM) {
                 float m = t.state0[i], v = t.state1[i];
                 adam_elem(g, p, m, v, pn, ah);
@@ -196,7 +197,7 @@ __global__ __launch_bounds__(OPT_THREADS) void pd_optim_kernel(const OptArgs a, 
                 if (has_s0) t.state0[i] = b;
             }
             t.p_out[i] = pn;
-            if (t.bf16_out) t.bf16_out[i] = MIXED ? f32_to_half(pn, a.out_fmt) : f32_to_bf16_rne(pn);
+            if (t.bf16_out) t.bf16_out[i] = OUT_RT ? f32_to_half(pn, a.out_fmt) : f32_to_bf16_rne(pn);
         }
     }
 }
@@ -208,7 +209,7 @@ int launch_optim(const pd_tensor_desc* descs, int n_tensors, const SgdHyper& sh,
     PD_REQUIRE(grad_fmt == PD_F32 || grad_fmt == PD_BF16 || grad_fmt == PD_F16, PD_EINVAL, "%s: unknown gradient format %d",
                who, grad_fmt);
     PD_REQUIRE(out_fmt == PD_BF16 || out_fmt == PD_F16, PD_EINVAL, "%s: unknown 16-bit output format %d", who, out_fmt);
-    const bool mixed = grad_fmt != PD_F32 || out_fmt != PD_BF16;
+    const bool grad16 = grad_fmt != PD_F32, out_rt = out_fmt != PD_BF16;
     if (n_tensors == 0) return PD_OK;
     PD_REQUIRE(descs != nullptr, PD_EINVAL, "%s: descs is NULL", who);
     int i = 0;
@@ -245,8 +246,10 @@ int launch_optim(const pd_tensor_desc* descs, int n_tensors, const SgdHyper& sh,
         for (int k = a.n_tensors + 1; k <= OPT_MAX_TENSORS; ++k) a.block_start[k] = (uint32_t)blocks;
         a.grad_fmt = grad_fmt;
         a.out_fmt = out_fmt;
-        if (mixed) pd_optim_kernel<ADAM, true><<<dim3((unsigned)blocks), dim3(OPT_THREADS), 0, (hipStream_t)stream>>>(a, sh, ah);
-        else pd_optim_kernel<ADAM, false><<<dim3((unsigned)blocks), dim3(OPT_THREADS), 0, (hipStream_t)stream>>>(a, sh, ah);
+        const dim3 grid((unsigned)blocks), block(OPT_THREADS);
+        if (grad16) pd_optim_kernel<ADAM, true, true><<<grid, block, 0, (hipStream_t)stream>>>(a, sh, ah);
+        else if (out_rt) pd_optim_kernel<ADAM, false, true><<<grid, block, 0, (hipStream_t)stream>>>(a, sh, ah);
+        else pd_optim_kernel<ADAM, false, false><<<grid, block, 0, (hipStream_t)stream>>>(a, sh, ah);
         PD_CHECK_LAUNCH(who);
     }
     return PD_OK;

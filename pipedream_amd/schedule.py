@@ -30,6 +30,21 @@ def _on(stream):
     return torch.cuda.stream(stream) if stream is not None else contextlib.nullcontext()
 
 
+def _join(stream):
+    """Start of a loop on a stream of its own: whatever the caller queued on its current stream before
+    (the arena's initial copies and fills, ``module.cuda()``, loader tensors) is ordered before the
+    stage's first kernel.  Side streams do not wait for the stream they were created on by themselves."""
+    if stream is not None:
+        stream.wait_stream(torch.cuda.current_stream())
+
+
+def _leave(stream):
+    """End of a loop: the caller's current stream waits for the stage's last kernel, so reading
+    parameters, ``state_dict()`` or a checkpoint after the loop needs no host synchronisation."""
+    if stream is not None:
+        torch.cuda.current_stream().wait_stream(stream)
+
+
 def stage_train_loop(r, optimizer, num_minibatches, loader=None, lr_schedule=None, on_forward=None,
                      no_input_pipelining=False, stream=None):
     """Generator running one stage's 1F1B schedule.
@@ -38,8 +53,11 @@ def stage_train_loop(r, optimizer, num_minibatches, loader=None, lr_schedule=Non
     ``adjust_learning_rate`` does (main_with_runtime.py:562-563).  ``on_forward(i, r)`` is
     called after each steady-state forward (where the reference reads ``r.loss``).  ``stream``: the
     stream this stage's kernels are launched on (default: torch's current stream); it is made current
-    only around the stage's own calls, never across a ``yield``."""
+    only around the stage's own calls, never across a ``yield``.  The stream is ordered behind the
+    caller's current stream when the loop starts and the caller's current stream behind it when the
+    loop ends."""
     n = num_minibatches
+    _join(stream)
     r.train(n)
     r.set_loader(loader if (r.stage is None or r.stage == 0) else None)
     warmup = 0 if no_input_pipelining else min(r.num_warmup_minibatches, n)
@@ -79,19 +97,30 @@ def stage_train_loop(r, optimizer, num_minibatches, loader=None, lr_schedule=Non
         for blocked in backward_and_update():
             yield blocked
     r.wait()
+    _leave(stream)
 
 
 def stage_eval_loop(r, num_minibatches, loader=None, on_forward=None, no_input_pipelining=False, stream=None):
     """Generator running one stage's forward-only schedule, the body of ``validate()`` in the
-    reference's caller (runtime/image_classification/main_with_runtime.py:429-487): ``W`` warm-up
-    forwards, then ``n - W`` times [forward, ack].  The ack is the clock: a stage takes its next
+    reference's caller (runtime/image_classification/main_with_runtime.py:429-498): ``W`` warm-up
+    forwards, then ``n - W`` times [forward, ack], then the ``W`` acknowledgements still outstanding
+    (:497-498), so that every stage takes and passes on one ack per minibatch and no queue is left
+    holding anything.  The ack is the clock: a stage takes its next
     steady-state minibatch only after its consumer has acknowledged the oldest outstanding one.
     Call it under ``torch.no_grad()`` as the reference does.  ``on_forward(i, r)`` is called after each
     steady-state forward (where the reference reads ``r.output`` / ``r.loss``)."""
     n = num_minibatches
+    _join(stream)
     r.eval(n)
     r.set_loader(loader if (r.stage is None or r.stage == 0) else None)
     warmup = 0 if no_input_pipelining else min(r.num_warmup_minibatches, n)
+
+    def ack():
+        while not r.can_run_ack():
+            yield r
+        with _on(stream):
+            r.run_ack()
+
     for i in range(n):
         while not r.can_run_forward():
             yield r
@@ -102,11 +131,13 @@ def stage_eval_loop(r, num_minibatches, loader=None, on_forward=None, no_input_p
         if on_forward is not None:
             with _on(stream):
                 on_forward(i - warmup, r)
-        while not r.can_run_ack():
-            yield r
-        with _on(stream):
-            r.run_ack()
+        for blocked in ack():
+            yield blocked
+    for _ in range(warmup):
+        for blocked in ack():
+            yield blocked
     r.wait()
+    _leave(stream)
 
 
 def run_pipeline(loops):

@@ -78,11 +78,13 @@ class Stage0(torch.nn.Module):
 class Stage1(torch.nn.Module):
     """Stage 1 of the 4-way split.  Its last ReLU's backward is applied by ``Stage2`` (the first convolution
     there masks its input gradient), so the gradient this stage receives must come from ``Stage2``:
-    ``premasked_output_grads`` states it, ``StageRuntime`` checks it on every hand-off."""
-    premasked_output_grads = (True,)
+    ``premasked_output_grads`` states it, ``StageRuntime`` checks it on every hand-off.
+    ``plain_handoff=True`` builds the stage with the reference's contract instead: it takes dL/d(out) as
+    runtime/communication.py:683-702 carries it and applies its last ReLU's backward itself."""
 
-    def __init__(self):
+    def __init__(self, plain_handoff=False):
         super(Stage1, self).__init__()
+        self.premasked_output_grads = (not plain_handoff,)
         pool1, pool2 = layers.PoolGradLink(), layers.PoolGradLink()
         self.layer2 = layers.MaxPool2d(2, 2, relu=True, link=pool1)    # layer1 ReLU + layer2 MaxPool
         self.layer3 = layers.Conv2d(64, 128, relu=True, grad_premasked=True, input_link=pool1)    # + layer4; masked by layer5
@@ -90,7 +92,7 @@ class Stage1(torch.nn.Module):
                                     output_link=pool2)                  # + layer6 + layer7
         self.layer7 = layers.MaxPool2d(2, 2, relu=True, applied_by_producer=True)
         # layer8's ReLU is undone for the gradient by the next stage's first convolution (input_rectified)
-        self.layer8 = layers.Conv2d(128, 256, relu=True, grad_premasked=True, input_link=pool2)   # + layer9
+        self.layer8 = layers.Conv2d(128, 256, relu=True, grad_premasked=not plain_handoff, input_link=pool2)   # + layer9
         _initialize_weights(self)
 
     def forward(self, input0):
@@ -102,13 +104,15 @@ class Stage1(torch.nn.Module):
 class Stage2(torch.nn.Module):
     """Stage 2 of the 4-way split.  Takes ``Stage1``'s rectified output and applies that ReLU's backward to
     the gradient it hands back (``masks_input_grads``); its own last ReLU's backward is applied by the
-    pooling layer that opens ``Stage3`` (``premasked_output_grads``)."""
-    masks_input_grads = (True,)
-    premasked_output_grads = (True,)
+    pooling layer that opens ``Stage3`` (``premasked_output_grads``).  ``plain_handoff=True``: neither; the
+    stage hands back the gradient of its input as it is and masks the gradient it receives itself."""
 
-    def __init__(self):
+    def __init__(self, plain_handoff=False):
         super(Stage2, self).__init__()
-        self.layer1 = layers.Conv2d(256, 256, relu=True, grad_premasked=True, input_rectified=True)   # + layer2; masked by layer3
+        self.masks_input_grads = (not plain_handoff,)
+        self.premasked_output_grads = (not plain_handoff,)
+        self.layer1 = layers.Conv2d(256, 256, relu=True, grad_premasked=True,
+                                    input_rectified=not plain_handoff)   # + layer2; masked by layer3
         pool3 = layers.PoolGradLink()
         self.layer3 = layers.Conv2d(256, 256, relu=True, input_rectified=True, pool=True,
                                     output_link=pool3)                  # + layer4 + layer5
@@ -116,7 +120,8 @@ class Stage2(torch.nn.Module):
         self.layer6 = layers.Conv2d(256, 512, relu=True, grad_premasked=True, input_link=pool3)   # + layer7; masked by layer8
         self.layer8 = layers.Conv2d(512, 512, relu=True, grad_premasked=True, input_rectified=True)   # + layer9
         # layer10's ReLU is undone for the gradient by the next stage's pooling layer (relu=True)
-        self.layer10 = layers.Conv2d(512, 512, relu=True, grad_premasked=True, input_rectified=True)  # + layer11
+        self.layer10 = layers.Conv2d(512, 512, relu=True, grad_premasked=not plain_handoff,
+                                     input_rectified=True)  # + layer11
         _initialize_weights(self)
 
     def forward(self, input0):
@@ -127,13 +132,14 @@ class Stage2(torch.nn.Module):
 
 class Stage3(torch.nn.Module):
     """Last stage of the 4-way split; its opening ReLU + MaxPool applies the backward of ``Stage2``'s last
-    ReLU (``masks_input_grads``)."""
-    masks_input_grads = (True,)
+    ReLU (``masks_input_grads``).  ``plain_handoff=True``: a plain pooling layer (stage3.py:12), the
+    gradient handed back is that of the stage's input."""
 
-    def __init__(self, dropout=0.5, num_classes=1000):
+    def __init__(self, dropout=0.5, num_classes=1000, plain_handoff=False):
         super(Stage3, self).__init__()
+        self.masks_input_grads = (not plain_handoff,)
         pool4 = layers.PoolGradLink()
-        self.layer1 = layers.MaxPool2d(2, 2, relu=True, link=pool4)
+        self.layer1 = layers.MaxPool2d(2, 2, relu=not plain_handoff, link=pool4)
         self.layer2 = layers.Conv2d(512, 512, relu=True, grad_premasked=True, input_link=pool4)   # + layer3; masked by layer4
         self.layer4 = layers.Conv2d(512, 512, relu=True, grad_premasked=True, input_rectified=True)   # + layer5
         self.layer6 = layers.Conv2d(512, 512, relu=True, input_rectified=True, pool=True)   # + layer7 + layer8
@@ -159,12 +165,17 @@ def arch():
     return "vgg16"
 
 
-def model(criterion, dropout=0.5):
+def model(criterion, dropout=0.5, plain_handoff=False):
+    """The four stages and the criterion.  By default stages 1 -> 2 and 2 -> 3 exchange gradients that the
+    consumer has already masked with the producer's last ReLU (one pass over the hand-off tensor saved per
+    boundary; both sides declare it and ``StageRuntime`` checks it).  ``plain_handoff=True`` builds the same
+    layers with the reference's contract on every boundary -- the gradient of the tensor that was sent,
+    nothing applied to it -- for pipelines that mix these stages with stages from elsewhere."""
     return [
         (Stage0(), ["input0"], ["out0"]),
-        (Stage1(), ["out0"], ["out1"]),
-        (Stage2(), ["out1"], ["out2"]),
-        (Stage3(dropout=dropout), ["out2"], ["out3"]),
+        (Stage1(plain_handoff=plain_handoff), ["out0"], ["out1"]),
+        (Stage2(plain_handoff=plain_handoff), ["out1"], ["out2"]),
+        (Stage3(dropout=dropout, plain_handoff=plain_handoff), ["out2"], ["out3"]),
         (criterion, ["out3"], ["loss"]),
     ]
 

@@ -89,6 +89,55 @@ def test_adam_multi_tensor_vs_oracle(eps_mode, wd):
             assert torch.equal(d_h[i], d_p[i].to(torch.bfloat16))
 
 
+_TORCH16 = {"bf16": torch.bfloat16, "f16": torch.float16}
+
+
+@pytest.mark.parametrize("grad_fmt,out_fmt", [("f32", "f16"), ("f32", "bf16"), ("bf16", "bf16"), ("f16", "f16"),
+                                              ("bf16", "f16"), ("f16", "bf16")])
+@pytest.mark.parametrize("adam", [False, True])
+def test_mixed_step_every_format_pair_vs_oracle(grad_fmt, out_fmt, adam):
+    """Every (gradient format, 16-bit copy format) pair the header allows for pd_*_step_mixed, aligned and
+    ragged sizes: the fp32 results equal the oracle's step on the widened gradient, the 16-bit copy is the
+    rounded fp32 result bit for bit.  (fp32 gradients with an fp16 copy once read the gradients as 16-bit.)"""
+    lib = _cabi.lib()
+    code = {"f32": _cabi.PD_F32, "bf16": _cabi.PD_BF16, "f16": _cabi.PD_F16}
+    rng = np.random.RandomState(5)
+    sizes = [5, 4096, 4097, 100003]
+    ps = [rng.randn(n).astype(np.float32) for n in sizes]
+    ms = [np.zeros(n, np.float32) for n in sizes]
+    vs = [np.zeros(n, np.float32) for n in sizes]
+    bufs = [None] * len(sizes)
+    d_p = [_dev(p) for p in ps]
+    d_m = [torch.zeros_like(t) for t in d_p]
+    d_v = [torch.zeros_like(t) for t in d_p]
+    d_h = [torch.zeros(t.numel(), dtype=_TORCH16[out_fmt], device="cuda") for t in d_p]
+    for step in range(1, 4):
+        gs = [rng.randn(n).astype(np.float32) for n in sizes]
+        d_g = [_dev(g) for g in gs]
+        if grad_fmt != "f32":
+            d_g = [g.to(_TORCH16[grad_fmt]) for g in d_g]
+            gs = [g.float().cpu().numpy() for g in d_g]
+        entries = [dict(g=g, p_in=p, p_out=p, s0=m, s1=v if adam else None, bf16=h)
+                   for g, p, m, v, h in zip(d_g, d_p, d_m, d_v, d_h)]
+        if adam:
+            lib.pd_adam_step_mixed(_desc_array(entries), len(entries), 1e-3, 0.9, 0.999, 1e-8, 1e-2, step, 0, 1.0, 1.0,
+                                   code[grad_fmt], code[out_fmt], _cabi.stream_ptr())
+        else:
+            lib.pd_sgd_step_mixed(_desc_array(entries), len(entries), 0.05, 0.9, 0.0, 1e-4, 0, int(step == 1), 1.0,
+                                  1.0, code[grad_fmt], code[out_fmt], _cabi.stream_ptr())
+        torch.cuda.synchronize()
+        for i in range(len(sizes)):
+            if adam:
+                ps[i], ms[i], vs[i] = so.adam_step_numpy(ps[i], gs[i], ms[i], vs[i], step, 1e-3, 0.9, 0.999, 1e-8, 1e-2, 0)
+                np.testing.assert_allclose(d_v[i].cpu().numpy(), vs[i], rtol=RTOL, atol=1e-9)
+                np.testing.assert_allclose(d_m[i].cpu().numpy(), ms[i], rtol=RTOL, atol=ATOL)
+            else:
+                ps[i], bufs[i] = so.sgd_step_numpy(ps[i], gs[i], bufs[i], 0.05, 0.9, 0.0, 1e-4, False)
+                np.testing.assert_allclose(d_m[i].cpu().numpy(), bufs[i], rtol=RTOL, atol=ATOL)
+            np.testing.assert_allclose(d_p[i].cpu().numpy(), ps[i], rtol=RTOL, atol=ATOL)
+            assert torch.equal(d_h[i], d_p[i].to(_TORCH16[out_fmt]))
+
+
 def test_unaligned_views_take_the_scalar_path():
     lib = _cabi.lib()
     rng = np.random.RandomState(2)

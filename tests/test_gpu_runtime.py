@@ -203,9 +203,14 @@ def test_forward_only_run_with_ack_clock():
                                                         on_forward=on_last if s == 2 else None)
                                for s, r in enumerate(rts)])
     torch.cuda.synchronize()
-    # every stage acknowledged n - W minibatches, in order, and never ran further ahead than W + 1
-    assert acks == [list(range(n - 2)), list(range(n - 1)), list(range(n))]
+    # every stage acknowledged all n minibatches, in order (the last W of them after its last forward,
+    # main_with_runtime.py:497-498), and never ran further ahead than W + 1
+    assert acks == [list(range(n))] * 3
     assert ahead == [3, 2, 1]
+    assert [r.backward_minibatch_id for r in rts] == [n, n, n]
+    # a complete run leaves nothing behind in any queue, in either direction
+    fabric = rts[0].comm_handler.fabric
+    assert all(len(q) == 0 for q in fabric.queues.values()), {k: len(q) for k, q in fabric.queues.items() if q}
     assert all(not m.training for r in rts for m in r.modules())
     # values: the oracle's modules in eval() mode (dropout is the identity)
     for m in ref:
@@ -217,8 +222,9 @@ def test_forward_only_run_with_ack_clock():
             torch.testing.assert_close(out, want, rtol=1e-5, atol=1e-6)
             assert abs(loss - float(crit(want, y))) <= 1e-5 * abs(float(crit(want, y))) + 1e-6
     assert len(outputs) == n
-    # a training run right after it starts clean: stale acknowledgements are dropped, gradients flow again
-    fabric = rts[0].comm_handler.fabric
+    # an interrupted run (a stage that stopped before its drain) leaves acknowledgements behind; the next
+    # run of that stage starts clean
+    fabric.put(handoff.ACK, 0, True, torch.zeros(1, dtype=torch.int64, device="cuda"), seq=0)
     rts[0].train(1)
     assert len(fabric.queue(handoff.ACK, 0, True)) == 0
 

@@ -312,6 +312,34 @@ def test_full_size_layer_properties():
         assert _rel(grads[k], p.grad) < 2e-2, (k, _rel(grads[k], p.grad))
 
 
+def test_full_size_stage_six_layers_vs_oracle():
+    """The whole stage at its benchmark size -- 6 layers, hidden 1024, 16 heads, FFN 4096, micro-batch
+    8 x 512 tokens -- forward and backward against the oracle: output, input gradient and every one of the
+    72 parameter gradients within rel-L2 2e-2, i.e. the bf16 error grown over six layers stays inside the bar.
+    The worst figures are printed."""
+    ref, mine = _pair(6, 1024, 16, 4096, seed=7)
+    assert sum(p.numel() for p in mine.parameters()) == 75577344
+    g = torch.Generator().manual_seed(8)
+    x = torch.randn(8, 512, 1024, generator=g)
+    dy = (torch.randn(8, 512, 1024, generator=g) * 0.05).to(BF)
+    xg = x.cuda().requires_grad_()
+    y = mine(xg)
+    y.backward(dy.cuda())
+    xr = x.clone().requires_grad_()
+    yr = ref(xr)
+    yr.backward(dy)
+    errs = {"output": _rel(y, yr), "input gradient": _rel(xg.grad, xr.grad)}
+    grads = dict((k, p.grad) for k, p in mine.named_parameters())
+    for k, p in ref.named_parameters():
+        assert grads[k].dtype == torch.float32 and grads[k].shape == p.grad.shape
+        errs[k] = _rel(grads[k], p.grad)
+    worst = sorted(errs.items(), key=lambda kv: -kv[1])[:5]
+    print("six-layer stage at full size, worst rel-L2 errors:", [(k, "%.2e" % v) for k, v in worst])
+    print("output %.2e, input gradient %.2e" % (errs["output"], errs["input gradient"]))
+    bad = {k: v for k, v in errs.items() if not v < 2e-2}
+    assert not bad, bad
+
+
 def test_batched_column_sums_match_the_single_ones():
     """``ops.ColsumBatch``: bf16 matrices (odd and unaligned shapes among them) and fp32 partial-sum matrices in
     one batch, fresh outputs and accumulation, against fp64 sums; nine jobs, so the batch runs twice."""

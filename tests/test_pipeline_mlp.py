@@ -71,8 +71,8 @@ def _run_product(n, per_stage_streams=False):
     forward/backward ran on, the final state_dicts and the ReLU masks of every forward."""
     from pipedream_amd import schedule
     stages = _build_product()
+    # no host synchronisation around the run: the loops order their streams against the caller's themselves
     streams = schedule.stage_streams(len(stages)) if per_stage_streams else [None] * len(stages)
-    torch.cuda.synchronize()
     assert [r.num_warmup_minibatches for r, _ in stages] == [1, 0]
     assert [o.num_versions for _, o in stages] == [2, 1]
     batches = gold.make_batches()[:n]
@@ -100,7 +100,6 @@ def _run_product(n, per_stage_streams=False):
             on_forward=(lambda i, rr: losses.append(float(rr.loss.detach()))) if si == 1 else None,
             stream=streams[si]))
     schedule.run_pipeline(loops)
-    torch.cuda.synchronize()
     params = [{k: v.detach().cpu() for k, v in r.modules()[0].state_dict().items()} for r, _ in stages]
     return losses, versions, params, masks
 
