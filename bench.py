@@ -539,16 +539,24 @@ CPU_BASELINES = {"vgg16_pipeline": cpu_vgg16_pipeline, "gnmt": cpu_gnmt, "gnmt_c
                  "transformer": cpu_transformer}
 
 
-def secondary(args):
-    run, kernel, peak, bound = {"vgg16_pipeline": (vgg16_pipeline_run, "conv3x3_winograd_kernel", PEAK_FP32_MFMA_TFLOPS, "mfma"),
-                                "gnmt": (gnmt_run, "gemm_f32", PEAK_FP32_MFMA_TFLOPS, "mfma"),
-                                "gnmt_criterion": (gnmt_criterion_run, "label_smoothing_bwd", 8000.0, "hbm"),
-                                "transformer": (transformer_run, "gemm_bf16", 2500.0, "mfma")}[args.workload]
-    if args.workload == "vgg16_pipeline":
-        elapsed, stats, batch, dtype, desc = run(args.steps, args.warmup, stage_streams=not args.single_stream)
-        desc += ", one stream for all stages" if args.single_stream else ", one stream per stage"
+_SECONDARY = {"vgg16_pipeline": (vgg16_pipeline_run, "conv3x3_winograd_kernel", PEAK_FP32_MFMA_TFLOPS, "mfma"),
+              "gnmt": (gnmt_run, "gemm_f32", PEAK_FP32_MFMA_TFLOPS, "mfma"),
+              "gnmt_criterion": (gnmt_criterion_run, "label_smoothing_bwd", 8000.0, "hbm"),
+              "transformer": (transformer_run, "gemm_bf16", 2500.0, "mfma")}
+
+
+def secondary_record(workload, steps, warmup, single_stream=False, with_cpu_baseline=True, with_kernels=True):
+    """One of the other configurations, measured like the headline one: the record of its line."""
+    import gc
+    import torch
+    run, kernel, peak, bound = _SECONDARY[workload]
+    if workload == "vgg16_pipeline":
+        elapsed, stats, batch, dtype, desc = run(steps, warmup, stage_streams=not single_stream)
+        desc += ", one stream for all stages" if single_stream else ", one stream per stage"
     else:
-        elapsed, stats, batch, dtype, desc = run(args.steps, args.warmup)
+        elapsed, stats, batch, dtype, desc = run(steps, warmup)
+    gc.collect()
+    torch.cuda.empty_cache()
     k = dict(stats[kernel])
     if bound == "hbm":
         # the byte-moving kernels record algorithmic bytes as their work: the rate is in TB/s
@@ -561,20 +569,31 @@ def secondary(args):
         extra = {"direct_equivalent": k["TFLOP/s"]}
         k["TFLOP/s"] = k["TFLOP/s"] * 16.0 / 36.0
     out = {
-        "metric": "samples/sec per stage (fwd+bwd+stashed update)", "value": batch * args.steps / elapsed,
-        "unit": "samples/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
-        "ms_per_step": 1e3 * elapsed / args.steps, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "metric": "samples/sec per stage (fwd+bwd+stashed update)", "value": batch * steps / elapsed,
+        "unit": "samples/s", "n_gpus": 1, "steps": steps, "warmup": warmup,
+        "ms_per_step": 1e3 * elapsed / steps, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": dtype, "data": "synthetic", "config": {"workload": desc, "global_batch": batch,
                                                         "parallelism": "1 stage on 1 GPU"},
         "roofline": {"bound": bound, "achieved": k["TFLOP/s"], "peak": peak,
                      "unit": "GB/s" if bound == "hbm" else "TFLOP/s",
                      "frac": k["TFLOP/s"] / peak, "traffic": None, "kernel": kernel, "launches": k["launches"],
                      "avg_us": k["avg_us"], **extra},
-        "kernels": stats,
     }
-    if not args.no_cpu_baseline:
-        out["cpu_baseline"] = CPU_BASELINES[args.workload]()
-    print(json.dumps(out))
+    if with_kernels:
+        out["kernels"] = stats
+    if with_cpu_baseline:
+        out["cpu_baseline"] = CPU_BASELINES[workload]()
+    return out
+
+
+def secondary(args):
+    print(json.dumps(secondary_record(args.workload, args.steps, args.warmup, args.single_stream,
+                                      not args.no_cpu_baseline)))
+
+
+# steps / warm-up steps of the other configurations inside the default run (each a few hundred milliseconds
+# of GPU time; their CPU baselines are the bounded samples above, a few seconds each)
+DEFAULT_RUN_WORKLOADS = {"vgg16_pipeline": (10, 3), "gnmt": (20, 5), "transformer": (40, 8)}
 
 
 def main():
@@ -589,6 +608,8 @@ def main():
                          "criterion and the transformer stage")
     ap.add_argument("--single-stream", action="store_true",
                     help="vgg16_pipeline: launch all four stages on one stream instead of one stream per stage")
+    ap.add_argument("--headline-only", action="store_true",
+                    help="default workload: leave out the `workloads` object (the other configurations)")
     ap.add_argument("--pmc-probe", action="store_true",
                     help="run the counter-calibration copy and two benchmark steps, print no JSON")
     ap.add_argument("--traffic-bytes", type=float, default=None,
@@ -647,6 +668,16 @@ def main():
     }
     if not args.no_cpu_baseline:
         out["cpu_baseline"] = cpu_baseline()
+    if not args.headline_only:
+        # the other configurations in the same record: throughput, dominant kernel against its roofline and
+        # the CPU oracle's rate on a bounded sample, each measured after the headline's timed region
+        import gc
+        del stats
+        gc.collect()
+        torch.cuda.empty_cache()
+        out["workloads"] = {name: secondary_record(name, steps, warmup, with_cpu_baseline=not args.no_cpu_baseline,
+                                                   with_kernels=False)
+                            for name, (steps, warmup) in DEFAULT_RUN_WORKLOADS.items()}
     print(json.dumps(out))
 
 

@@ -22,7 +22,7 @@ from oracle import stash_oracle as so
 pytestmark = pytest.mark.gpu
 
 SGD_KW = dict(lr=0.01, momentum=0.9, weight_decay=5e-4)
-MAX_SWITCHES_PER_PASS = 8   # provisional until observed
+MAX_SWITCHES_PER_PASS = 3
 
 
 def _nhwc(t):
