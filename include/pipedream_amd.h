@@ -337,6 +337,12 @@ int pd_gemm_bf16(int trans_a, int trans_b, int M, int N, int K,
                  void* C, int ldc, int out_f32, float alpha, float beta,
                  const float* bias, const uint16_t* residual, int ldr,
                  int batch_outer, int batch_inner, const int64_t* strides, void* stream);
+/* Tuning and test hook: force the tile of the direct-to-LDS kernel behind pd_gemm_bf16 / pd_gemm_bf16_gelu
+ * for products it can take (K a multiple of 128): (128, 128) or (256, 256); (0, 0) restores the built-in
+ * choice (256 x 256 when there are at least 256 such tiles and K >= 2048, else 128 x 128).  Process-wide,
+ * not thread-safe against concurrent GEMM calls.  No counterpart in the reference (its GEMMs are library calls). */
+int pd_gemm_bf16_set_tile(int bm, int bn);
+
 /* The same GEMM (unbatched, bf16 output) with the exact GELU of a feed-forward block in its epilogue.
  * backward = 0:  C = op(A) op(B) + bias  (the pre-activation, kept for the backward) and aux = gelu(C),
  *                with C taken as rounded to bf16, both written by the kernel;

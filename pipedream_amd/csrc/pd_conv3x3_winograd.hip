@@ -1106,6 +1106,24 @@ __global__ __launch_bounds__(WW_THREADS, 1) void winograd_wgrad_kernel(const Win
                     rr[0][b][j] = __builtin_fmaf(rr_c0, dyr[1][b][j], dyr[0][b][j]);
                     rr[1][b][j] = __builtin_fmaf(rr_c1, dyr[0][b][j], dyr[1][b][j]);
                 }
+            // all sixteen are formed here, before the next strip's dY is requested: the requests then land in the
+            // registers the old values leave (left to itself the compiler forms the second row's values where
+            // they are used, keeps the old dY alive until then and copies the new one over it at the loop's end,
+            // sixteen moves per step)
+#pragma unroll
+            for (int ii = 0; ii < 2; ++ii)
+#pragma unroll
+                for (int b = 0; b < 2; ++b)
+#pragma unroll
+                    for (int j = 0; j < 4; ++j) asm volatile("" : "+v"(rr[ii][b][j]) : : "memory");
+            // (the old dY values count as used once more after that: a value that dies in the multiply-add gets the
+            // result written over it, and the result, which lives on, would again keep the request's register busy)
+#pragma unroll
+            for (int r = 0; r < 2; ++r)
+#pragma unroll
+                for (int b = 0; b < 2; ++b)
+#pragma unroll
+                    for (int j = 0; j < 4; ++j) asm volatile("" : : "v"(dyr[r][b][j]));
             load_dy(dp, d_left > 0);           // strip q+1
             next_d();
             __builtin_amdgcn_sched_barrier(0);

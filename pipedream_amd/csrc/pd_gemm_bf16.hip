@@ -688,6 +688,9 @@ int launch_gemm_bf16(int ta, int tb, GemmBf16Args g, int batch, hipStream_t s) {
 
 }  // namespace
 
+// tile choice forced by pd_gemm_bf16_set_tile (0 = the built-in choice)
+static int g_force_bm = 0, g_force_bn = 0;
+
 static int gemm_bf16_run(int trans_a, int trans_b, int M, int N, int K, const uint16_t* A, int lda,
                          const uint16_t* B, int ldb, void* C, int ldc, int out_f32, float alpha, float beta,
                          const float* bias, const uint16_t* residual, int ldr, int batch_outer, int batch_inner,
@@ -735,13 +738,28 @@ static int gemm_bf16_run(int trans_a, int trans_b, int M, int N, int K, const ui
     // direct-to-LDS kernel: whole ring rounds of k, and per-lane byte offsets that fit 32 bits
     const bool dma_ok = K % (DK * NS) == 0 && (long long)256 * (lda > ldb ? lda : ldb) * 2 < (1ll << 31);
     const bool wide = M >= 256 && N >= 256;       // a 256 x 256 tile is mostly inside the matrix
-    if (dma_ok && wide && tiles256 >= 256) return launch_gemm_bf16_dma<256, 256>(trans_a, trans_b, g, batch, s);
+    if (g_force_bm && dma_ok) {
+        if (g_force_bm == 256 && g_force_bn == 256) return launch_gemm_bf16_dma<256, 256>(trans_a, trans_b, g, batch, s);
+        if (g_force_bm == 128 && g_force_bn == 128) return launch_gemm_bf16_dma<128, 128>(trans_a, trans_b, g, batch, s);
+    }
+    // A 256 x 256 tile pays about 25 us of ring fill and epilogue that nothing overlaps (one block per CU); below
+    // a reduction depth of 2048 two co-resident 128 x 128 blocks per CU, which overlap each other's, are faster
+    // (4096 x 4096 x 1024: 43 against 50 us; x 2048: 80 against 74 us).
+    if (dma_ok && wide && tiles256 >= 256 && K >= 2048) return launch_gemm_bf16_dma<256, 256>(trans_a, trans_b, g, batch, s);
     if (dma_ok && M >= 128 && N >= 128) return launch_gemm_bf16_dma<128, 128>(trans_a, trans_b, g, batch, s);
     if (wide && tiles256 >= 192) return launch_gemm_bf16<256, 256, 2, 4>(trans_a, trans_b, g, batch, s);
     // narrow outputs (attention: N = head dimension): tall tiles, all waves stacked along M
     if (N <= 64 && M >= 256) return launch_gemm_bf16<256, 64, 4, 1>(trans_a, trans_b, g, batch, s);
     if (M >= 128 && N >= 128 && tiles128 >= 128) return launch_gemm_bf16<128, 128, 2, 2>(trans_a, trans_b, g, batch, s);
     return launch_gemm_bf16<64, 64, 2, 2>(trans_a, trans_b, g, batch, s);
+}
+
+extern "C" int pd_gemm_bf16_set_tile(int bm, int bn) {
+    const bool known = (bm == 0 && bn == 0) || (bm == 128 && bn == 128) || (bm == 256 && bn == 256);
+    PD_REQUIRE(known, PD_EINVAL, "pd_gemm_bf16_set_tile: tiles are 128 x 128 or 256 x 256 (0, 0 = built-in choice)");
+    g_force_bm = bm;
+    g_force_bn = bn;
+    return PD_OK;
 }
 
 extern "C" int pd_gemm_bf16(int trans_a, int trans_b, int M, int N, int K, const uint16_t* A, int lda,

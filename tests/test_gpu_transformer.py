@@ -58,22 +58,47 @@ def test_gemm_bf16_epilogues():
 @pytest.mark.parametrize("ta,tb", [(False, True), (False, False), (True, False), (True, True)])
 @pytest.mark.parametrize("M,N,K", [(4096, 4096, 128), (4088, 4104, 256), (4096, 3072, 128), (3992, 3600, 256),
                                    (1000, 1016, 384), (4000, 3592, 224), (3584, 3584, 96)])
-def test_gemm_bf16_large_tiles(M, N, K, ta, tb):
-    """K a multiple of 128 runs the direct-to-LDS ring kernel (one to three ring rounds): with
-    256 x 256 tiles when there are at least 256 of them, else with 128 x 128 tiles; other K
-    the register-staged large-tile kernel; M and N that are not tile multiples exercise the
-    clamped loads and the masked vector stores.
-    The fp32 reference product is computed on the device by torch from the same bf16 inputs."""
-    from pipedream_amd import ops
+@pytest.mark.parametrize("tile", [128, 256])
+def test_gemm_bf16_large_tiles(M, N, K, ta, tb, tile):
+    """K a multiple of 128 runs the direct-to-LDS ring kernel (one to three ring rounds), here with each of
+    its two tile sizes forced in turn (the built-in choice takes 256 x 256 tiles only for K >= 2048); other K
+    the register-staged kernels; M and N that are not tile multiples exercise the clamped loads and the masked
+    vector stores.  The fp32 reference product is computed on the device by torch from the same bf16 inputs."""
+    from pipedream_amd import _cabi, ops
     g = torch.Generator().manual_seed(M + N + K)
     a = torch.randn((K, M) if ta else (M, K), generator=g).to(BF).cuda()
     b = torch.randn((N, K) if tb else (K, N), generator=g).to(BF).cuda()
     want = (a.float().t() if ta else a.float()) @ (b.float().t() if tb else b.float())
-    got32 = ops.gemm_bf16(a, b, trans_a=ta, trans_b=tb, out_f32=True)
+    _cabi.lib().pd_gemm_bf16_set_tile(tile, tile)
+    try:
+        got32 = ops.gemm_bf16(a, b, trans_a=ta, trans_b=tb, out_f32=True)
+        got16 = ops.gemm_bf16(a, b, trans_a=ta, trans_b=tb)
+    finally:
+        _cabi.lib().pd_gemm_bf16_set_tile(0, 0)
     assert _rel(got32, want.cpu()) < 1e-5
     torch.testing.assert_close(got32, want, rtol=1e-4, atol=2e-6 * math.sqrt(K) * 9)
-    got16 = ops.gemm_bf16(a, b, trans_a=ta, trans_b=tb)
     assert torch.equal(got16, got32.to(BF))
+
+
+def test_gemm_bf16_built_in_tile_choice_and_hook_errors():
+    """Deep reductions take the 256 x 256 kernel by themselves, shallow ones the 128 x 128 kernel; both agree with
+    the forced runs bit for bit (the tile size does not change the order of a dot product's additions)."""
+    from pipedream_amd import _cabi, ops
+    lib = _cabi.lib()
+    with pytest.raises(_cabi.PipedreamAmdError):
+        lib.pd_gemm_bf16_set_tile(64, 64)
+    g = torch.Generator().manual_seed(11)
+    for K in (1024, 2048):
+        a = (torch.randn(4096, K, generator=g) / 8).to(BF).cuda()
+        b = (torch.randn(4096, K, generator=g) / 8).to(BF).cuda()
+        auto = ops.gemm_bf16(a, b, trans_b=True, out_f32=True)
+        for tile in (128, 256):
+            lib.pd_gemm_bf16_set_tile(tile, tile)
+            try:
+                forced = ops.gemm_bf16(a, b, trans_b=True, out_f32=True)
+            finally:
+                lib.pd_gemm_bf16_set_tile(0, 0)
+            assert torch.equal(auto, forced)
 
 
 def test_gemm_bf16_large_tile_epilogues():
@@ -368,8 +393,16 @@ def test_batched_column_sums_match_the_single_ones():
         batch.add(torch.zeros(4, 4, device="cuda"), torch.zeros(3, device="cuda"), 0.0)
 
 
+@pytest.fixture(params=[0, 256], ids=["built_in_tile", "tile_256"])
+def gemm_tile(request):
+    from pipedream_amd import _cabi
+    _cabi.lib().pd_gemm_bf16_set_tile(request.param, request.param)
+    yield request.param
+    _cabi.lib().pd_gemm_bf16_set_tile(0, 0)
+
+
 @pytest.mark.parametrize("M,N,K", [(4096, 4096, 1024), (512, 1024, 256), (200, 72, 64), (64, 8, 8)])
-def test_gemm_with_gelu_in_its_epilogue(M, N, K):
+def test_gemm_with_gelu_in_its_epilogue(M, N, K, gemm_tile):
     """``gemm_bf16_gelu`` / ``gemm_bf16_gelu_backward`` against the GEMM followed by the element-wise kernels
     (the same operations; only the erf approximation and one bf16 rounding differ) and against torch in fp32."""
     from pipedream_amd import ops
