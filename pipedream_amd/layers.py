@@ -50,8 +50,42 @@ class _LinearFn(torch.autograd.Function):
         return dx, dw, db, None
 
 
+class _Linear16Fn(torch.autograd.Function):
+    """The same layer with 16-bit (bfloat16) parameters and activations, as the modules of a stage built with
+    ``StageRuntime(fp16=True)`` hold them (runtime/runtime.py:227-229): products on the bf16 MFMA GEMM with
+    fp32 accumulation, gradients returned in the parameters' format (what the mixed-precision optimizer step
+    reads, runtime/optimizer.py:137-145)."""
+
+    @staticmethod
+    def forward(ctx, x, weight, bias):
+        x2 = ops.cast_bf16(x.reshape(-1, x.shape[-1])) if x.dtype == torch.float32 else x.reshape(-1, x.shape[-1])
+        x2 = x2.contiguous()
+        y = ops.gemm_bf16(x2, weight, trans_b=True, bias=ops.cast_f32(bias) if bias is not None else None)
+        ctx.has_bias = bias is not None
+        ctx.x_shape, ctx.x_dtype = x.shape, x.dtype
+        ctx.save_for_backward(x2, weight)
+        return y.view(*x.shape[:-1], weight.shape[0])
+
+    @staticmethod
+    def backward(ctx, dy):
+        x2, weight = ctx.saved_tensors
+        dy2 = dy.reshape(-1, dy.shape[-1]).contiguous()
+        dx = dw = db = None
+        if ctx.needs_input_grad[0]:
+            dx = ops.gemm_bf16(dy2, weight).view(ctx.x_shape)
+            if ctx.x_dtype == torch.float32:
+                dx = ops.cast_f32(dx)
+        if ctx.needs_input_grad[1]:
+            dw = ops.gemm_bf16(dy2, x2, trans_a=True)
+        if ctx.has_bias and ctx.needs_input_grad[2]:
+            db = ops.cast_bf16(ops.colsum_bf16(dy2))
+        return dx, dw, db
+
+
 class Linear(torch.nn.Module):
-    """``torch.nn.Linear`` (optionally with the following ReLU fused into the GEMM epilogue)."""
+    """``torch.nn.Linear`` (optionally with the following ReLU fused into the GEMM epilogue).  Converted to
+    bfloat16 (``module.bfloat16()``, or ``StageRuntime(fp16=True, half_dtype=torch.bfloat16)``) the layer runs on
+    the bf16 GEMM; float16 parameters have no kernel here and raise."""
 
     def __init__(self, in_features, out_features, bias=True, relu=False):
         super(Linear, self).__init__()
@@ -69,6 +103,14 @@ class Linear(torch.nn.Module):
             torch.nn.init.uniform_(self.bias, -bound, bound)
 
     def forward(self, x):
+        if self.weight.dtype != torch.float32:
+            if self.weight.dtype != torch.bfloat16:
+                raise NotImplementedError("Linear with %s parameters: the 16-bit GEMM of this build is bfloat16 "
+                                          "(StageRuntime(fp16=True, half_dtype=torch.bfloat16))" % self.weight.dtype)
+            if self.relu:
+                raise NotImplementedError("Linear(relu=True) has no 16-bit kernel; follow the layer with GELU or "
+                                          "keep the stage in fp32")
+            return _Linear16Fn.apply(x, self.weight, self.bias)
         return _LinearFn.apply(x, self.weight, self.bias, self.relu)
 
     def extra_repr(self):
@@ -660,6 +702,27 @@ class _CastFn(torch.autograd.Function):
         return (ops.cast_f32(dy) if ctx.to_bf16 else ops.cast_bf16(dy)), None
 
 
+class _GeluFn(torch.autograd.Function):
+    @staticmethod
+    def forward(ctx, x):
+        ctx.save_for_backward(x)
+        return ops.gelu(x)
+
+    @staticmethod
+    def backward(ctx, dy):
+        (x,) = ctx.saved_tensors
+        return ops.gelu_backward(x, dy.contiguous())
+
+
+class GELU(torch.nn.Module):
+    """``torch.nn.GELU()`` (erf form) on bfloat16 activations."""
+
+    def forward(self, x):
+        if x.dtype != torch.bfloat16:
+            raise NotImplementedError("GELU: only bfloat16 activations have a kernel")
+        return _GeluFn.apply(x.contiguous())
+
+
 def to_bf16(x):
     return x if x.dtype == torch.bfloat16 else _CastFn.apply(x, True)
 
@@ -738,4 +801,5 @@ class CrossEntropyLoss(torch.nn.Module):
         self.ignore_index = ignore_index
 
     def forward(self, logits, target):
-        return _CrossEntropyFn.apply(logits, target, self.ignore_index)
+        # (bfloat16 logits of a 16-bit stage are widened first: the loss is evaluated in fp32)
+        return _CrossEntropyFn.apply(to_f32(logits), target, self.ignore_index)

@@ -329,3 +329,105 @@ def test_matched_relu_contract_trains():
         for (k, p), (_, q) in zip(mod.named_parameters(), m.named_parameters()):
             err = float((p.grad.cpu() - q.grad).norm() / q.grad.norm())
             assert err < 1e-4, (k, err)
+
+
+class _Body16(torch.nn.Module):
+    def __init__(self, d_in, d_hidden, d_out):
+        super(_Body16, self).__init__()
+        from pipedream_amd import layers
+        self.fc1 = layers.Linear(d_in, d_hidden)
+        self.act = layers.GELU()
+        self.fc2 = layers.Linear(d_hidden, d_out)
+
+    def forward(self, x):
+        return self.fc2(self.act(self.fc1(x)))
+
+
+def _runtime16(body, half_dtype, loss_scale):
+    from pipedream_amd import runtime
+    from pipedream_amd.layers import CrossEntropyLoss
+    return runtime.StageRuntime(
+        model=[(body, ["input0"], ["out0"]), (CrossEntropyLoss(), ["out0"], ["loss"])], distributed_backend="gloo",
+        fp16=True, loss_scale=loss_scale, training_tensor_shapes={}, eval_tensor_shapes={}, training_tensor_dtypes={},
+        inputs_module_destinations={"input": 0}, target_tensor_names={"target"},
+        configuration_maps={"module_to_stage_map": None, "stage_to_rank_map": None, "stage_to_depth_map": None},
+        master_addr="127.0.0.1", rank=None, local_rank=0, num_ranks_in_server=1, verbose_freq=0,
+        model_type=runtime.IMAGE_CLASSIFICATION, half_dtype=half_dtype)
+
+
+def test_sixteen_bit_stage_runtime_with_masters_matches_oracle():
+    """``StageRuntime(fp16=True)`` (runtime/runtime.py:227-229, 268-276, 306-321, 397-398) with the caller's
+    fp16 sequence (``r.zero_grad()`` instead of ``optimizer.zero_grad()``, main_with_runtime.py:406-413): the
+    modules hold bfloat16 parameters, the optimizer steps fp32 masters through the fused mixed-precision kernel
+    and stashes 16-bit versions.  Against torch's bfloat16 CPU modules under the oracle's restatement of that
+    branch: versions bit-exact, losses and the masters' movement within the bf16 bar (rel 2e-2), model parameters
+    exactly the rounded masters; the checkpoint carries the masters."""
+    from pipedream_amd import sgd
+    torch.manual_seed(0)
+    ref32 = torch.nn.Sequential(torch.nn.Linear(32, 64), torch.nn.GELU(), torch.nn.Linear(64, 16))
+    body = _Body16(32, 64, 16)
+    body.fc1.load_state_dict(ref32[0].state_dict())
+    body.fc2.load_state_dict(ref32[2].state_dict())
+    loss_scale, W, nv, n = 128.0, 1, 2, 7
+    r = _runtime16(body, torch.bfloat16, loss_scale)
+    assert all(p.dtype == torch.bfloat16 for p in r.model_parameters)
+    assert all(p.dtype == torch.float32 and p.requires_grad for p in r.master_parameters)
+    assert [tuple(a.shape) for a in r.model_parameters] == [tuple(b.shape) for b in r.master_parameters]
+    kw = dict(lr=0.05, momentum=0.9, weight_decay=1e-4)
+    opt = sgd.SGDWithWeightStashing(r.modules(), r.master_parameters, r.model_parameters, loss_scale, nv, **kw)
+    ref = ref32.bfloat16()
+    ref_model = list(ref.parameters())
+    ref_master = [p.detach().clone().float().requires_grad_() for p in ref_model]
+    ora = so.StashingOptimizerOracle("SGD", [ref], ref_master, nv, model_parameters=ref_model, loss_scale=loss_scale, **kw)
+    start = [m.detach().clone() for m in ref_master]
+    batches = _batches(n, d_in=32, classes=16)
+    r.train(n)
+    r.set_loader(batches)
+    pend = []
+    for kind, k in so.one_f_one_b(n, W):
+        x, y = batches[k]
+        if kind == "F":
+            r.run_forward()
+            assert r.tensors[-1]["input0"].dtype == torch.bfloat16        # converted on the way in
+            out = ref(x.bfloat16())
+            loss = torch.nn.functional.cross_entropy(out.float(), y)
+            assert abs(float(r.loss.detach()) - float(loss.detach())) <= 2e-2 * abs(float(loss.detach()))
+            pend.append(loss)
+            continue
+        r.zero_grad()
+        ref.zero_grad()
+        for o in (ora, opt):
+            o.load_old_params()
+        assert opt.current_version.version == ora.current_version == so.backward_version(k, W)
+        r.run_backward()
+        (pend.pop(0) * loss_scale).backward()
+        for o in (ora, opt):
+            o.load_new_params()
+            o.step()
+        assert opt.queue.versions() == ora.versions()
+        for q, m in zip(r.model_parameters, r.master_parameters):
+            assert q.grad.dtype == torch.bfloat16
+            assert torch.equal(q.detach(), m.detach().bfloat16())          # the model is the rounded master
+    for m, rm, m0 in zip(r.master_parameters, ref_master, start):
+        moved = (rm.detach() - m0).norm()
+        assert float(((m.detach().cpu() - m0) - (rm.detach() - m0)).norm() / moved) < 2e-2
+    # the checkpoint holds the masters (runtime/runtime.py:310-311) and restores them (:317-321)
+    state = r.state_dict()
+    assert [tuple(t.shape) for t in state["master_parameters"]] == [tuple(m.shape) for m in r.master_parameters]
+    other = _runtime16(_Body16(32, 64, 16), torch.bfloat16, loss_scale)
+    other.load_state_dict(state)
+    for a, b in zip(other.master_parameters, r.master_parameters):
+        assert torch.equal(a.detach(), b.detach())
+    for a, b in zip(other.parameters(), r.parameters()):
+        assert torch.equal(a.detach(), b.detach())
+
+
+def test_float16_stage_is_converted_and_refused_at_its_first_layer():
+    """The reference's format: the conversion and the parameter lists are the same; the stage kernels of this
+    build are bfloat16, and the layer says so instead of computing something else."""
+    r = _runtime16(_Body16(32, 64, 16), None, 1.0)
+    assert r.half_dtype == torch.float16 and all(p.dtype == torch.float16 for p in r.model_parameters)
+    r.train(1)
+    r.set_loader(_batches(1, d_in=32, classes=16))
+    with pytest.raises(NotImplementedError, match="bfloat16"):
+        r.run_forward()
