@@ -251,10 +251,12 @@ def cpu_baseline(timed_steps=6):
 
 # ---- other configurations (not the default line): one stage each, same step definition ----------
 
-def _run_steps(step, steps, warmup):
+def _run_steps(step, steps, warmup, before_instrumented=None):
     """Throughput over `steps` un-instrumented steps, then a short instrumented pass for the per-kernel
     figures (an event pair around each of the thousands of launches of these stages would slow the
-    timed region itself)."""
+    timed region itself).  `before_instrumented` is called between the two (a stage that runs passes of
+    different minibatches side by side goes back to one stream there, so that a launch's duration is the
+    kernel's own)."""
     import torch
     from pipedream_amd import ops
     for _ in range(warmup):
@@ -265,6 +267,8 @@ def _run_steps(step, steps, warmup):
         step()
     torch.cuda.synchronize()
     elapsed = time.perf_counter() - t0
+    if before_instrumented is not None:
+        before_instrumented()
     ops.kernel_timer = {}
     for _ in range(min(steps, 4)):
         step()
@@ -278,38 +282,64 @@ def _run_steps(step, steps, warmup):
     return elapsed, stats
 
 
-def gnmt_run(steps, warmup):
+def gnmt_run(steps, warmup, overlap=True):
     """Embedding (32320 x 1024) + 4 LSTM layers (hidden 1024, residuals), T = 50, batch 128, fp32,
     AdamWithWeightStashing with stash depth 3 (2 forwards in flight)."""
+    import contextlib
     import torch
-    from pipedream_amd import adam
+    from pipedream_amd import adam, schedule
     from pipedream_amd.stages import gnmt
     torch.manual_seed(0)
     m = gnmt.Stage0(dropout=0.0).cuda()
     opt = adam.AdamWithWeightStashing([m], list(m.parameters()), None, 1.0, 3, lr=1e-3, betas=(0.9, 0.999))
     ids = torch.randint(0, 32320, (50, 128)).cuda()
     dy = (torch.randn(50, 128, 1024) * 1e-2).cuda()
-    pend = [m(ids) for _ in range(2)]
+    # minibatch j runs on stream j mod 3: the forward recurrence of minibatch k + 2 beside the backward
+    # recurrence of minibatch k (schedule.MinibatchStreams; same results as one stream, bit for bit)
+    rings = [schedule.MinibatchStreams(2) if overlap else None]
+    if rings[0] is not None:
+        rings[0].join()
+    count = {"f": 0, "b": 0}
+    pend = []
+
+    def one_stream():
+        if rings[0] is not None:
+            rings[0].leave()
+            rings[0] = None
+
+    def forward():
+        ring = rings[0]
+        with (ring.forward(count["f"]) if ring is not None else contextlib.nullcontext()):
+            pend.append(m(ids))
+        count["f"] += 1
 
     def step():
-        pend.append(m(ids))
-        opt.zero_grad()
-        opt.load_old_params()
-        pend.pop(0).backward(dy)
-        opt.load_new_params()
-        opt.step()
+        forward()
+        ring = rings[0]
+        with (ring.backward(count["b"]) if ring is not None else contextlib.nullcontext()):
+            opt.zero_grad()
+            opt.load_old_params()
+            pend.pop(0).backward(dy)
+            opt.load_new_params()
+            opt.step()
+        count["b"] += 1
 
-    elapsed, stats = _run_steps(step, steps, warmup)
+    forward()
+    forward()
+    elapsed, stats = _run_steps(step, steps, warmup, one_stream)
     return elapsed, stats, 128, "f32", ("GNMT-style stage: embedding 32320x1024 + 4 LSTM layers hidden 1024 with residuals, "
-                                         "seq 50, batch 128, fp32, Adam, stash depth 3")
+                                         "seq 50, batch 128, fp32, Adam, stash depth 3"
+                                         + (", forward of a new minibatch beside the backward of the oldest (one stream "
+                                            "per minibatch in flight)" if overlap else ", one stream"))
 
 
-def transformer_run(steps, warmup):
+def transformer_run(steps, warmup, overlap=True):
     """6 pre-LN transformer layers (hidden 1024, 16 heads, FFN 4096), micro-batch 8 x 512 tokens,
     bf16 compute, fp32 master weights + Adam every 4 micro-batches, 2 weight versions.  One step =
     one micro-batch forward + backward (+ the update on every 4th)."""
+    import contextlib
     import torch
-    from pipedream_amd import adam
+    from pipedream_amd import adam, schedule
     from pipedream_amd.stages import transformer
     torch.manual_seed(0)
     m = transformer.Stage0().cuda()
@@ -317,20 +347,43 @@ def transformer_run(steps, warmup):
                                       lr=1e-3, betas=(0.9, 0.999))
     x = torch.randn(8, 512, 1024).cuda()
     dy = (torch.randn(8, 512, 1024) * 0.05).bfloat16().cuda()
-    pend = [m(x)]
+    # micro-batch j runs on stream j mod 2: the forward pass of a new micro-batch beside the backward pass of
+    # the one in flight (schedule.MinibatchStreams; same results as one stream, bit for bit)
+    rings = [schedule.MinibatchStreams(1) if overlap else None]
+    if rings[0] is not None:
+        rings[0].join()
+    count = {"f": 0, "b": 0}
+    pend = []
+
+    def one_stream():
+        if rings[0] is not None:
+            rings[0].leave()
+            rings[0] = None
+
+    def forward():
+        ring = rings[0]
+        with (ring.forward(count["f"]) if ring is not None else contextlib.nullcontext()):
+            pend.append(m(x))
+        count["f"] += 1
 
     def step():
-        pend.append(m(x))
-        opt.zero_grad()
-        opt.load_old_params()
-        pend.pop(0).backward(dy)
-        opt.load_new_params()
-        opt.step()
+        forward()
+        ring = rings[0]
+        with (ring.backward(count["b"]) if ring is not None else contextlib.nullcontext()):
+            opt.zero_grad()
+            opt.load_old_params()
+            pend.pop(0).backward(dy)
+            opt.load_new_params()
+            opt.step()
+        count["b"] += 1
 
-    elapsed, stats = _run_steps(step, steps, warmup)
+    forward()
+    elapsed, stats = _run_steps(step, steps, warmup, one_stream)
     return elapsed, stats, 8, "bf16", ("PipeDream-2BW stage: 6 transformer layers (hidden 1024, 16 heads, FFN 4096, GELU, "
                                         "pre-LN), seq 512, micro-batch 8, 4-micro-batch accumulation, 2 weight versions, "
-                                        "bf16 compute, fp32 master Adam")
+                                        "bf16 compute, fp32 master Adam"
+                                        + (", forward of a new micro-batch beside the backward of the one in flight (one "
+                                           "stream per micro-batch in flight)" if overlap else ", one stream"))
 
 
 def gnmt_criterion_run(steps, warmup):
@@ -553,6 +606,8 @@ def secondary_record(workload, steps, warmup, single_stream=False, with_cpu_base
     if workload == "vgg16_pipeline":
         elapsed, stats, batch, dtype, desc = run(steps, warmup, stage_streams=not single_stream)
         desc += ", one stream for all stages" if single_stream else ", one stream per stage"
+    elif workload in ("gnmt", "transformer"):
+        elapsed, stats, batch, dtype, desc = run(steps, warmup, overlap=not single_stream)
     else:
         elapsed, stats, batch, dtype, desc = run(steps, warmup)
     gc.collect()
@@ -579,6 +634,10 @@ def secondary_record(workload, steps, warmup, single_stream=False, with_cpu_base
                      "frac": k["TFLOP/s"] / peak, "traffic": None, "kernel": kernel, "launches": k["launches"],
                      "avg_us": k["avg_us"], **extra},
     }
+    if workload in ("gnmt", "transformer") and not single_stream:
+        # the timed steps run the passes of different minibatches side by side; the launch durations behind
+        # the roofline come from instrumented steps on one stream, where a launch has the GPU to itself
+        out["roofline"]["measured_on"] = "one stream (instrumented steps after the timed region)"
     if with_kernels:
         out["kernels"] = stats
     if with_cpu_baseline:
@@ -607,7 +666,8 @@ def main():
                          "line for the full VGG16 as four co-resident stages, the LSTM stage, the GNMT classifier + "
                          "criterion and the transformer stage")
     ap.add_argument("--single-stream", action="store_true",
-                    help="vgg16_pipeline: launch all four stages on one stream instead of one stream per stage")
+                    help="vgg16_pipeline: launch all four stages on one stream instead of one stream per stage; "
+                         "gnmt, transformer: forward and backward passes on one stream instead of one stream per minibatch in flight")
     ap.add_argument("--headline-only", action="store_true",
                     help="default workload: leave out the `workloads` object (the other configurations)")
     ap.add_argument("--pmc-probe", action="store_true",

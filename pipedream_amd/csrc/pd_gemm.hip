@@ -281,10 +281,10 @@ typedef __attribute__((address_space(3))) void* lds_void_ptr;
 typedef __attribute__((address_space(1))) const void* global_void_ptr;
 
 constexpr int SK_COLS = 128;             // tile columns
-constexpr int SK_STAGES = 8;             // ring stages of BK = 16
+// (ring stages of BK = 16, SK_STAGES below: 8 or 4)
 
 // WM = 2: up to 128 rows, waves 2 x 2, 64 x 64 each.  WM = 1: up to 64 rows, waves 1 x 4, 64 x 32 each.
-template <int WM, bool B_KC>
+template <int WM, bool B_KC, int SK_STAGES>
 struct Skinny {
     static constexpr int BM = 64 * WM;
     static constexpr int WN = 4 / WM;
@@ -390,9 +390,9 @@ __device__ __forceinline__ void sk_wait_vmcnt() {
     __builtin_amdgcn_s_waitcnt((N & 15) | ((N >> 4) << 14) | (7 << 4) | (15 << 8));
 }
 
-template <int WM, bool B_KC>
+template <int WM, bool B_KC, int SK_STAGES>
 __global__ __launch_bounds__(GEMM_THREADS) void pd_gemm_skinny_kernel(const GemmArgs a) {
-    using S = Skinny<WM, B_KC>;
+    using S = Skinny<WM, B_KC, SK_STAGES>;
     constexpr int TN = S::TN;
     __shared__ __attribute__((aligned(1024))) char lds[S::LDS_BYTES];
     const int lane = threadIdx.x % 64;
@@ -418,25 +418,21 @@ __global__ __launch_bounds__(GEMM_THREADS) void pd_gemm_skinny_kernel(const Gemm
         sk.init(a, n0, wave, lane, (uint32_t)(size_t)(lds_void_ptr)lds);
         // k of stage number i, clamped to the last stage of the range
 #define SK_K(i) (k_begin + min((i), total - 1) * BK)
-        sk.template issue<0>(a, lds, SK_K(0), wave);
-        sk.template issue<1>(a, lds, SK_K(1), wave);
-        sk.template issue<2>(a, lds, SK_K(2), wave);
-        sk.template issue<3>(a, lds, SK_K(3), wave);
-        sk.template issue<4>(a, lds, SK_K(4), wave);
-        sk.template issue<5>(a, lds, SK_K(5), wave);
-        sk.template issue<6>(a, lds, SK_K(6), wave);
-        static_assert(SK_STAGES == 8, "the ring fill and the unrolled loop are written for 8 stages");
+#define SK_FILL(ST) if constexpr (ST < SK_STAGES - 1) sk.template issue<ST>(a, lds, SK_K(ST), wave);
+        SK_FILL(0) SK_FILL(1) SK_FILL(2) SK_FILL(3) SK_FILL(4) SK_FILL(5) SK_FILL(6)
+#undef SK_FILL
+        static_assert(SK_STAGES == 8 || SK_STAGES == 4, "the ring fill and the unrolled loop are written for 4 or 8 stages");
         // Stage i (ring slot ST): wait until it has landed everywhere; every wave is then also past
-        // its reads of stage i-1, so that slot is refilled with stage i+7; then read and multiply.
+        // its reads of stage i-1, so that slot is refilled with stage i + SK_STAGES - 1; then read and multiply.
 #define SK_STAGE(ST)                                                                                      \
-        {                                                                                                     \
+        if constexpr (ST < SK_STAGES) {                                                                       \
             const int i = i0 + ST;                                                                            \
             sk_wait_vmcnt<S::IN_FLIGHT * S::IPT>();                                                          \
             __builtin_amdgcn_s_barrier();                                                                     \
-            sk.template issue<(ST + 7) % 8>(a, lds, SK_K(i + 7), wave);                                      \
+            sk.template issue<(ST + SK_STAGES - 1) % SK_STAGES>(a, lds, SK_K(i + SK_STAGES - 1), wave);      \
             if (i < total) {                                                                                  \
                 float4_t fa[2][2], fb[TN][2];                                                                 \
-                sk.template read<ST>(fa, fb);                                                                 \
+                sk.template read<ST % SK_STAGES>(fa, fb);                                                     \
                 _Pragma("unroll") for (int g = 0; g < 2; ++g)                                                 \
                 _Pragma("unroll") for (int q = 0; q < 4; ++q)                                                 \
                 _Pragma("unroll") for (int ii = 0; ii < 2; ++ii)                                              \
@@ -556,12 +552,16 @@ extern "C" int pd_gemm_splitk_f32(int trans_a, int trans_b, int M, int N, int K,
     if (!trans_a && M <= 128 && N % 4 == 0 && g.a_vec && g.b_vec && g.k_per_split % BK == 0 && K % BK == 0 &&
         (size_t)128 * (lda > ldb ? lda : ldb) * 4 < (1ull << 31)) {
         const dim3 grid((N + SK_COLS - 1) / SK_COLS, 1, splits);
+        // up to 64 rows: 8 ring stages (96 KB; these products stream large weight matrices from HBM once).
+        // 65 to 128 rows (the LSTM recurrences): 4 stages, 64 KB, so that two blocks share a CU -- of one launch,
+        // or of the forward recurrence of one minibatch and the backward recurrence of another running on
+        // different streams; with 8 stages (128 KB) a second block only found room between launches.
         if (M <= 64) {
-            if (trans_b) pd_gemm_skinny_kernel<1, true><<<grid, GEMM_THREADS, 0, s>>>(g);
-            else pd_gemm_skinny_kernel<1, false><<<grid, GEMM_THREADS, 0, s>>>(g);
+            if (trans_b) pd_gemm_skinny_kernel<1, true, 8><<<grid, GEMM_THREADS, 0, s>>>(g);
+            else pd_gemm_skinny_kernel<1, false, 8><<<grid, GEMM_THREADS, 0, s>>>(g);
         } else {
-            if (trans_b) pd_gemm_skinny_kernel<2, true><<<grid, GEMM_THREADS, 0, s>>>(g);
-            else pd_gemm_skinny_kernel<2, false><<<grid, GEMM_THREADS, 0, s>>>(g);
+            if (trans_b) pd_gemm_skinny_kernel<2, true, 4><<<grid, GEMM_THREADS, 0, s>>>(g);
+            else pd_gemm_skinny_kernel<2, false, 4><<<grid, GEMM_THREADS, 0, s>>>(g);
         }
         PD_CHECK_LAUNCH("pd_gemm_splitk_f32");
         return PD_OK;

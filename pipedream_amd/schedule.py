@@ -45,8 +45,67 @@ def _leave(stream):
         torch.cuda.current_stream().wait_stream(stream)
 
 
+class MinibatchStreams(object):
+    """Streams that let a stage's forward pass of one minibatch run beside the backward pass of an older one.
+
+    In steady-state 1F1B a stage issues forward(k + W), backward(k), update(k), forward(k + W + 1), ...  The
+    forward pass of minibatch k + W and the backward pass of minibatch k share no data (different activations,
+    the newest weight version against a stashed one, and the update writes the ring's oldest slot, which neither
+    reads), yet on one stream they run one after the other.  Here minibatch j does everything -- forward,
+    backward, update -- on stream j mod (W + 1).  The forward pass of minibatch k + W + 1 needs the weights
+    that update(k) wrote: same stream, ordered by itself.  The only order that crosses streams is
+    update(k - 1) before backward(k) / update(k) (optimizer state and accumulated gradients), kept by one
+    event.  Results are bit-identical to the single-stream order: the same kernels on the same operands.
+
+    What it buys depends on the stage: kernels that fill the GPU by themselves (convolutions) gain nothing;
+    the LSTM stage, whose recurrences are chains of short dependent launches, runs two chains side by side.
+
+    Use: ``with ring.forward(j): ...`` around the forward pass of minibatch ``j``, ``with ring.backward(k): ...``
+    around ``zero_grad`` .. ``step`` of minibatch ``k`` (``stage_train_loop(..., minibatch_streams=ring)`` does
+    it), ``ring.join()`` before the first and ``ring.leave()`` after the last pass to order the ring against
+    the caller's current stream.  All streams have the default priority."""
+
+    def __init__(self, warmup):
+        self.streams = [torch.cuda.Stream() for _ in range(int(warmup) + 1)]
+        self._updated = None          # event behind the latest update
+        # A parameter's gradient-accumulation node lives as long as any graph that reaches the parameter, i.e. for
+        # ever under 1F1B, and stays on the stream of the first forward pass; the engine orders it against the
+        # stream a later backward pass runs on by itself.  That is intended here, so its warning is switched off.
+        quiet = getattr(torch.autograd.graph, "set_warn_on_accumulate_grad_stream_mismatch", None)
+        if quiet is not None:
+            quiet(False)
+
+    def stream_of(self, minibatch):
+        return self.streams[minibatch % len(self.streams)]
+
+    def join(self):
+        here = torch.cuda.current_stream()
+        for s in self.streams:
+            s.wait_stream(here)
+
+    def leave(self):
+        here = torch.cuda.current_stream()
+        for s in self.streams:
+            here.wait_stream(s)
+
+    @contextlib.contextmanager
+    def forward(self, minibatch):
+        with torch.cuda.stream(self.stream_of(minibatch)):
+            yield
+
+    @contextlib.contextmanager
+    def backward(self, minibatch):
+        s = self.stream_of(minibatch)
+        with torch.cuda.stream(s):
+            if self._updated is not None:
+                s.wait_event(self._updated)
+            yield
+            self._updated = torch.cuda.Event()
+            self._updated.record(s)
+
+
 def stage_train_loop(r, optimizer, num_minibatches, loader=None, lr_schedule=None, on_forward=None,
-                     no_input_pipelining=False, stream=None):
+                     no_input_pipelining=False, stream=None, minibatch_streams=None):
     """Generator running one stage's 1F1B schedule.
 
     ``lr_schedule(step) -> lr`` is written into every param group each iteration, as
@@ -55,8 +114,14 @@ def stage_train_loop(r, optimizer, num_minibatches, loader=None, lr_schedule=Non
     stream this stage's kernels are launched on (default: torch's current stream); it is made current
     only around the stage's own calls, never across a ``yield``.  The stream is ordered behind the
     caller's current stream when the loop starts and the caller's current stream behind it when the
-    loop ends."""
+    loop ends.  ``minibatch_streams``: a ``MinibatchStreams(r.num_warmup_minibatches)`` instead of ``stream``;
+    the forward pass of a new minibatch then runs beside the backward pass of the oldest one in flight."""
     n = num_minibatches
+    if minibatch_streams is not None and stream is not None:
+        raise ValueError("give either stream or minibatch_streams")
+    ring = minibatch_streams
+    if ring is not None:
+        ring.join()
     _join(stream)
     r.train(n)
     r.set_loader(loader if (r.stage is None or r.stage == 0) else None)
@@ -65,13 +130,13 @@ def stage_train_loop(r, optimizer, num_minibatches, loader=None, lr_schedule=Non
     def forward():
         while not r.can_run_forward():
             yield r
-        with _on(stream):
+        with (ring.forward(r.forward_minibatch_id) if ring is not None else _on(stream)):
             r.run_forward()
 
     def backward_and_update():
         while not r.can_run_backward():
             yield r
-        with _on(stream):
+        with (ring.backward(r.backward_minibatch_id) if ring is not None else _on(stream)):
             optimizer.zero_grad()
             optimizer.load_old_params()
             r.run_backward()
@@ -89,7 +154,7 @@ def stage_train_loop(r, optimizer, num_minibatches, loader=None, lr_schedule=Non
             for param_group in optimizer.param_groups:
                 param_group['lr'] = lr
         if on_forward is not None:
-            with _on(stream):
+            with (ring.forward(r.forward_minibatch_id - 1) if ring is not None else _on(stream)):
                 on_forward(i, r)
         for blocked in backward_and_update():
             yield blocked
@@ -98,6 +163,8 @@ def stage_train_loop(r, optimizer, num_minibatches, loader=None, lr_schedule=Non
             yield blocked
     r.wait()
     _leave(stream)
+    if ring is not None:
+        ring.leave()
 
 
 def stage_eval_loop(r, num_minibatches, loader=None, on_forward=None, no_input_pipelining=False, stream=None):

@@ -142,3 +142,47 @@ def test_embedding_gradient_sums_duplicates_in_position_order():
             want[v] += dout[p]
     assert torch.equal(got, want)
     assert not got[30:].any() and not got[3].any()
+
+
+def test_forward_beside_backward_on_a_stream_ring_gives_the_same_bits():
+    """``schedule.MinibatchStreams``: minibatch j runs forward, backward and update on stream j mod (W + 1), so
+    the forward recurrence of a new minibatch runs beside the backward recurrence of the oldest one.  At the
+    stage's real width (hidden 1024, batch 128; a short sequence), with no host synchronisation inside the run:
+    outputs, parameters and Adam state equal the single-stream run bit for bit, versions included."""
+    from pipedream_amd import adam, schedule
+    from pipedream_amd.stages import gnmt
+    V, H, T, B, W, n = 1000, 1024, 6, 128, 2, 8
+    g = torch.Generator().manual_seed(5)
+    ids = [torch.randint(0, V, (T, B), generator=g).cuda() for _ in range(n)]
+    gs = [(torch.randn(T, B, H, generator=g) * 1e-2).cuda() for _ in range(n)]
+
+    def run(ring):
+        torch.manual_seed(4)
+        m = gnmt.Stage0(V, H, dropout=0.0).cuda()
+        opt = adam.AdamWithWeightStashing([m], list(m.parameters()), None, 1.0, W + 1, lr=1e-3, betas=(0.9, 0.999))
+        outs, pend = [], []
+        if ring is not None:
+            ring.join()
+        for kind, k in so.one_f_one_b(n, W):
+            if kind == "F":
+                with (ring.forward(k) if ring is not None else torch.cuda.stream(torch.cuda.current_stream())):
+                    pend.append(m(ids[k]))
+                    outs.append(pend[-1].detach())
+            else:
+                with (ring.backward(k) if ring is not None else torch.cuda.stream(torch.cuda.current_stream())):
+                    opt.zero_grad()
+                    opt.load_old_params()
+                    pend.pop(0).backward(gs[k])
+                    opt.load_new_params()
+                    opt.step()
+        if ring is not None:
+            ring.leave()
+        state = [opt.state[p][name] for p in m.parameters() for name in ("exp_avg", "exp_avg_sq")]
+        return ([o.cpu() for o in outs], [p.detach().cpu() for p in m.parameters()], [t.cpu() for t in state],
+                opt.queue.versions())
+
+    one = run(None)
+    many = run(schedule.MinibatchStreams(W))
+    assert one[3] == many[3]
+    for a, b in zip(one[:3], many[:3]):
+        assert len(a) == len(b) and all(torch.equal(x, y) for x, y in zip(a, b))

@@ -66,7 +66,7 @@ def _build_product(num_minibatches=20):
     return stages
 
 
-def _run_product(n, per_stage_streams=False):
+def _run_product(n, per_stage_streams=False, minibatch_rings=False):
     """n minibatches through the two co-resident stages.  Returns losses, the version every
     forward/backward ran on, the final state_dicts and the ReLU masks of every forward."""
     from pipedream_amd import schedule
@@ -98,7 +98,8 @@ def _run_product(n, per_stage_streams=False):
         loops.append(schedule.stage_train_loop(
             r, opt, n, loader=batches if si == 0 else None,
             on_forward=(lambda i, rr: losses.append(float(rr.loss.detach()))) if si == 1 else None,
-            stream=streams[si]))
+            stream=streams[si],
+            minibatch_streams=schedule.MinibatchStreams(r.num_warmup_minibatches) if minibatch_rings else None))
     schedule.run_pipeline(loops)
     params = [{k: v.detach().cpu() for k, v in r.modules()[0].state_dict().items()} for r, _ in stages]
     return losses, versions, params, masks
@@ -170,6 +171,19 @@ def test_one_stream_per_stage_gives_the_same_bits():
     n = 12
     one = _run_product(n)
     many = _run_product(n, per_stage_streams=True)
+    assert one[0] == many[0] and one[1] == many[1]
+    for a, b in zip(one[2], many[2]):
+        assert a.keys() == b.keys() and all(torch.equal(a[k], b[k]) for k in a)
+    assert all(torch.equal(a, b) for a, b in zip(one[3], many[3]))
+
+
+@pytest.mark.gpu
+def test_minibatch_stream_rings_give_the_same_bits():
+    """Every stage with a ``MinibatchStreams`` ring (forward of a new minibatch beside the backward of the oldest
+    in flight), the stages ordered by the hand-off's events: identical to the single-stream run, bit for bit."""
+    n = 12
+    one = _run_product(n)
+    many = _run_product(n, minibatch_rings=True)
     assert one[0] == many[0] and one[1] == many[1]
     for a, b in zip(one[2], many[2]):
         assert a.keys() == b.keys() and all(torch.equal(a[k], b[k]) for k in a)

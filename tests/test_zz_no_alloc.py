@@ -4,6 +4,7 @@ array, so the results must agree bit for bit -- on two calls in a row, the secon
 (the array keeps the first call's partial sums), for the few-channel and the 64-channel kernels, with and
 without the ReLU mask.  A shape beyond the array is refused."""
 import ctypes
+import gc
 
 import pytest
 import torch
@@ -38,15 +39,16 @@ def _both(lib, N, H, W, C, K, masked, seed):
                 lib.pd_conv3x3_wgrad_noalloc_nhwc_f32(_ptr(x), _ptr(dy), _ptr(mask), _ptr(dw), _ptr(db),
                                                       N, H, W, C, K, stream)
                 _both.warm = True
+            gc.collect()
             torch.cuda.synchronize()
             before, free_before = torch.cuda.memory_allocated(), torch.cuda.mem_get_info()[0]
             lib.pd_conv3x3_wgrad_noalloc_nhwc_f32(_ptr(x), _ptr(dy), _ptr(mask), _ptr(dw), _ptr(db),
                                                   N, H, W, C, K, stream)
             torch.cuda.synchronize()
-            # neither torch's allocator nor the device's free memory (a hipMalloc inside the library
-            # would show there) moved
-            assert torch.cuda.memory_allocated() == before
-            assert torch.cuda.mem_get_info()[0] == free_before
+            # nothing was taken from torch's allocator, nothing from the device (a hipMalloc inside the library
+            # would show there); either figure may still fall when frees that earlier tests left pending complete
+            assert torch.cuda.memory_allocated() <= before
+            assert torch.cuda.mem_get_info()[0] >= free_before
         out.append((dw, db))
     torch.cuda.synchronize()
     return x, dy, mask, out, need.value
