@@ -101,6 +101,8 @@ def gemm(a, b, trans_a=False, trans_b=False, bias=None, relu=False, out=None, be
 
 SPLITK_TARGET_BLOCKS = 256     # one block per CU
 SPLITK_MIN_K = 128             # k per split is never smaller than this
+SPLITK_FULL_HOUSE = 768        # blocks of the 128 x 128 kernel the GPU holds at once (three per CU)
+SPLITK_DEEP_K = 1024           # ... worth filling by a split only if every part still reduces over this much
 
 
 def splitk_factor(M, N, K, trans_a=False):
@@ -108,12 +110,20 @@ def splitk_factor(M, N, K, trans_a=False):
     Mirrors the tile choice of pd_gemm_splitk_f32: its streaming kernel for M <= 128 (A not transposed,
     K a multiple of 16) owns all rows x 128 columns per block; otherwise tiles are 128 x 128 when M > 64
     and N >= 128, else 64 x 64."""
+    t_general = 0
     if not trans_a and M <= 128 and K % 16 == 0:
         tiles = -(-N // 128)
     else:
-        t = 128 if (M > 64 and N >= 128) else 64
+        t = t_general = 128 if (M > 64 and N >= 128) else 64
         tiles = -(-M // t) * -(-N // t)
     if tiles * 2 > SPLITK_TARGET_BLOCKS or K < 2 * SPLITK_MIN_K:
+        # between one block per CU and a full house (the 128 x 128 kernel runs three blocks per CU): a deep
+        # reduction is split two or three ways so that every CU holds three blocks instead of one or two
+        # (4096 x 1024 x 6400, the LSTM weight gradients: 256 tiles -> 768 blocks)
+        if t_general == 128 and tiles <= SPLITK_FULL_HOUSE // 2:
+            splits = SPLITK_FULL_HOUSE // tiles
+            if K // splits >= SPLITK_DEEP_K:
+                return splits
         return 1
     return max(1, min(SPLITK_TARGET_BLOCKS // tiles, K // SPLITK_MIN_K, 64))
 

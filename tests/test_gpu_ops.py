@@ -251,3 +251,22 @@ def test_linear_layer_matches_torch_nn():
     torch.testing.assert_close(mine.weight.grad.cpu(), ref.weight.grad, rtol=1e-5, atol=1e-5)
     torch.testing.assert_close(mine.bias.grad.cpu(), ref.bias.grad, rtol=1e-5, atol=1e-5)
     assert list(mine.state_dict().keys()) == list(ref.state_dict().keys())
+
+
+@pytest.mark.parametrize("ta,tb", [(False, True), (False, False), (True, False), (True, True)])
+def test_gemm_many_tiles_and_deep_split(ta, tb):
+    """6400 x 4096 (1600 tiles of 128 x 128) and 2048 x 2048 with a reduction of 4096 (256 tiles: split three ways
+    so that three blocks share each CU).  Against torch's product of the same operands in fp64."""
+    from pipedream_amd import ops
+    g = torch.Generator().manual_seed(7)
+    for (M, N, K) in ((6400, 4096, 64), (2048, 2048, 4096)):
+        a = torch.randn((K, M) if ta else (M, K), generator=g).cuda()
+        b = torch.randn((N, K) if tb else (K, N), generator=g).cuda()
+        bias = torch.randn(N, generator=g).cuda()
+        got = ops.gemm(a, b, trans_a=ta, trans_b=tb, bias=bias)
+        want = (a.double().t() if ta else a.double()) @ (b.double().t() if tb else b.double()) + bias.double()
+        err = float((got.double() - want).norm() / want.norm())
+        assert err < 1e-6, (M, N, K, err)
+        torch.testing.assert_close(got.double(), want, rtol=1e-5, atol=1e-5 * (K ** 0.5))
+    assert ops.splitk_factor(2048, 2048, 4096) == 3 and ops.splitk_factor(4096, 1024, 6400, True) == 3
+    assert ops.splitk_factor(6400, 4096, 1024) == 1 and ops.splitk_factor(6400, 1024, 4096) == 1
