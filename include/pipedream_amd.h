@@ -224,6 +224,14 @@ int pd_conv3x3_filter_rot180_f32(const float* w, float* out, int K, int C, void*
 int pd_conv3x3_dgrad_nhwc_f32(const float* dy, const float* w_rot, const float* relu_out,
                               const float* x_rectified, float* dx,
                               int N, int H, int W, int K, int C, void* stream);
+/* Tuning and test hook for the three pd_conv3x3_winograd_fwd* entry points.  A batch of images whose height is
+ * even but no multiple of 16 is processed as one tall image; if its width is a multiple of 8 (4) but not of 16
+ * pixels, a work item can then be two (four) pieces of 16 x 8 (16 x 4) pixels instead of one 16 x 16 square, which
+ * leaves no padding columns.  mode 0 (default): pieces when they lower the number of work items of the busiest
+ * compute unit; 1: pieces wherever the shape allows; -1: never.  Results are bit-identical either way.
+ * Process-wide, not thread-safe against concurrent convolution calls.  No counterpart in the reference. */
+int pd_conv3x3_winograd_set_pieces(int mode);
+
 /* The same convolution (and, with rot180, its input gradient) by the Winograd algorithm
  * F(2x2, 3x3) in fp32: 2.25x fewer multiplications; results agree with the direct kernels to
  * fp32 rounding (about 2e-6 relative).  Needs C % 8 == 0 and K % 4 == 0

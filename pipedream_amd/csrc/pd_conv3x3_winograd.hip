@@ -48,14 +48,22 @@ constexpr int WG_FRAG = 256;                     // floats in one wave-wide frag
 constexpr int WG_V_STAGE = WG_G * 2 * WG_FRAG;   // floats of transformed input per chunk: [g][wm][lane][4]
 constexpr int WG_OP = WG_BN + 4;                 // pitch of the output staging tile
 constexpr int WG_XCD = 8;
-constexpr int WG_HALO = WG_PIX + 2;              // input halo tile: 18 x 18 pixels
-constexpr int WG_PIECES = WG_HALO * WG_HALO * 2; // 16-byte pieces (pixel, 4-channel half) of one chunk of it
+constexpr int WG_HALO = WG_PIX + 2;              // input halo tile: 18 rows x (16 + 2 per segment) pixels
 // The halo tile in LDS: four planes (channel half, column parity) of 18 rows x 12 16-byte units; the
 // unit of (half, row, col) is ((half * 2 + (col & 1)) * 18 + row) * 12 + (col >> 1).  The eight tiles
 // of a tile row then read eight consecutive units and the next tile row lands 8 units further
 // (mod 16): a wave's 128-bit reads of one patch position are free of bank conflicts.
+// Each plane ends with two units of zeros (what a stacked batch's tiles read for the patch row that lies in the
+// neighbouring image).
+//
+// Segments.  A work item's 16 x 16 pixels need not be one square of the image: with SEG = 2 (4) they are two (four)
+// pieces of 16 rows x 8 (4) columns, consecutive in a row-major numbering of all such pieces of the stacked batch.
+// An image width of 56 (28) pixels is then covered exactly by 7 pieces per 16 rows instead of 4 (2) squares of
+// which the last is half (a quarter) empty.  Every piece has its own halo, so the halo tile is 18 rows x
+// (16 + 2 SEG) columns, the pieces' halos side by side; a tile of piece s finds its patch s units further right.
 constexpr int WG_RAW_PITCH = 12;
-constexpr int WG_RAW_STAGE = 4 * WG_HALO * WG_RAW_PITCH * 4;   // floats
+constexpr int WG_PLANE = WG_HALO * WG_RAW_PITCH + 2;           // 16-byte units of one plane
+constexpr int WG_RAW_STAGE = 4 * WG_PLANE * 4;                 // floats
 // LDS map (floats): two stages of transformed input, two stages of raw halo tile, output staging tile
 constexpr int WG_RAW_OFF = 2 * WG_V_STAGE;
 constexpr int WG_OUT_OFF = WG_RAW_OFF + 2 * WG_RAW_STAGE;
@@ -78,6 +86,7 @@ struct WinoArgs {
     int img_h;              // stacked variant: rows of one image (N is then 1 and H the rows of the whole batch)
     int relu;
     int tiles_x, tiles_y, k_blocks, n_chunks;
+    int segs_per_row, n_segs;     // segmented variant: pieces per 16 rows of the stacked batch, pieces in all
     int n_items, items_per_xcd;   // work items (pixel tile x channel block) in all / per die
 };
 
@@ -171,6 +180,25 @@ __device__ __forceinline__ WinoItem wino_decode(const WinoArgs& a, int item) {
     return w;
 }
 
+// Piece s of a work item: first output row and column, and whether it exists (the last item may have fewer).
+// SEG = 1: the item's square.
+struct SegPos { int y0, x0; bool ok; };
+template <int SEG>
+__device__ __forceinline__ SegPos seg_pos(const WinoArgs& a, int item, int s) {
+    SegPos p;
+    if (SEG == 1) {
+        const WinoItem w = wino_decode(a, item);
+        p.y0 = w.y0; p.x0 = w.x0; p.ok = true;
+    } else {
+        const int sg = (item / a.k_blocks) * SEG + s;
+        const int rb = sg / a.segs_per_row;
+        p.y0 = rb * WG_PIX;
+        p.x0 = (sg - rb * a.segs_per_row) * (WG_PIX / SEG);
+        p.ok = sg < a.n_segs;
+    }
+    return p;
+}
+
 // Persistent kernel: gridDim.x (a multiple of 8, at most one block per CU) blocks share the work items.
 // Block b lives on die b % 8 and takes the items  (b % 8) * items_per_xcd + b / 8 + i * gridDim.x / 8,
 // i = 0, 1, ...: at any time the blocks of one die work on neighbouring items (the channel blocks of one
@@ -193,8 +221,8 @@ __device__ __forceinline__ WinoItem wino_decode(const WinoArgs& a, int item) {
 // 16 rows.  img_h is even, hence no 2 x 2 tile straddles two images; a tile in the first (last) tile row
 // of an image must see zeros in the first (last) row of its 4 x 4 patch, where the stacked layout holds
 // the neighbouring image's row.  Only the threads that form row 0 (d0 - d2) resp. row 3 (d1 - d3) of
-// B^T d read those rows: for such a tile their row pointer goes to a patch of zeros in LDS (units 9 and
-// 10 of a halo row, which no piece is ever written to) -- set once per work item, nothing per step.
+// B^T d read those rows: for such a tile their row pointer goes to a patch of zeros in LDS (the two units
+// behind a plane's rows, which no piece is ever written to) -- set once per work item, nothing per step.
 //
 // UNPOOL: the launch computes the input gradient of a convolution whose input came out of a 2 x 2 max
 // pooling with index bytes (the pooling epilogue above, or the pooling kernel).  The epilogue then also
@@ -202,8 +230,13 @@ __device__ __forceinline__ WinoItem wino_decode(const WinoArgs& a, int item) {
 // full-resolution gradient if the recorded maximum was positive (the ReLU in front of the pooling), the
 // window's other three positions get zeros, and y itself is stored with the same mask -- what the
 // pooling backward kernel would compute from y, without the kernel and without its re-read of y.
-template <bool MASK, bool POOL, bool STACKED, bool UNPOOL = false>
+template <bool MASK, bool POOL, bool STACKED, bool UNPOOL = false, int SEG = 1>
 __global__ __launch_bounds__(WG_THREADS, 1) void winograd_fwd_kernel(const WinoArgs a) {
+    static_assert(SEG == 1 || (STACKED && !MASK), "segments go with the stacked batch");
+    constexpr int SEGW = WG_PIX / SEG;           // columns of a piece
+    constexpr int HALO_W = WG_PIX + 2 * SEG;     // columns of the halo tile
+    constexpr int PIECES = WG_HALO * HALO_W * 2; // 16-byte pieces (pixel, 4-channel half) of one chunk of it
+    static_assert(PIECES <= 2 * WG_THREADS && HALO_W <= 2 * WG_RAW_PITCH, "halo tile");
     __shared__ __attribute__((aligned(16))) float lds[WG_LDS_FLOATS];
 
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
@@ -216,17 +249,19 @@ __global__ __launch_bounds__(WG_THREADS, 1) void winograd_fwd_kernel(const WinoA
     if (n_my == 0) return;                                           // whole block, before any barrier
 
     // ---- stage 1 role: pieces p = tid and tid + 512 of the halo tile; piece = (halo pixel, channel half)
-    int hy[2], hx[2], raw_dst[2];
+    int hy[2], hx[2], hseg[2], raw_dst[2];       // (hx: column inside the piece's own halo; hseg: the piece)
     uint32_t pcg[2];
 #pragma unroll
     for (int j = 0; j < 2; ++j) {
         const int p = tid + WG_THREADS * j, pix = p >> 1, half = p & 1;
-        hy[j] = pix / WG_HALO;
-        hx[j] = pix - hy[j] * WG_HALO;
+        hy[j] = pix / HALO_W;
+        const int col = pix - hy[j] * HALO_W;
+        hseg[j] = SEG == 1 ? 0 : col / (SEGW + 2);
+        hx[j] = col - hseg[j] * (SEGW + 2);
         pcg[j] = half * 16;
-        raw_dst[j] = (((half * 2 + (hx[j] & 1)) * WG_HALO + hy[j]) * WG_RAW_PITCH + (hx[j] >> 1)) * 4;
+        raw_dst[j] = ((half * 2 + (col & 1)) * WG_PLANE + hy[j] * WG_RAW_PITCH + (col >> 1)) * 4;
     }
-    const bool second_piece = tid + WG_THREADS < WG_PIECES;
+    const bool second_piece = tid + WG_THREADS < PIECES;
     const float* ximg = a.x;
     const float* mimg = MASK ? a.mask : a.x;
     const uint32_t img_bytes = (uint32_t)a.H * a.W * a.C * 4;
@@ -235,14 +270,16 @@ __global__ __launch_bounds__(WG_THREADS, 1) void winograd_fwd_kernel(const WinoA
     // past the last item) gets an offset beyond the buffer's size, for which a buffer load returns 0
     auto set_load_item = [&](int i) {
         if (i < n_my) {
-            const WinoItem w = wino_decode(a, item0 + i * gx8);
-            const size_t img = (size_t)w.n * a.H * a.W * a.C;
-            ximg = a.x + img;
-            if (MASK) mimg = a.mask + img;
+            if (SEG == 1) {
+                const size_t img = (size_t)wino_decode(a, item0 + i * gx8).n * a.H * a.W * a.C;
+                ximg = a.x + img;
+                if (MASK) mimg = a.mask + img;
+            }
 #pragma unroll
             for (int j = 0; j < 2; ++j) {
-                const int gy = w.y0 - 1 + hy[j], gx = w.x0 - 1 + hx[j];
-                loff[j] = (gy >= 0 && gy < a.H && gx >= 0 && gx < a.W && (j == 0 || second_piece))
+                const SegPos sp = seg_pos<SEG>(a, item0 + i * gx8, hseg[j]);
+                const int gy = sp.y0 - 1 + hy[j], gx = sp.x0 - 1 + hx[j];
+                loff[j] = (sp.ok && gy >= 0 && gy < a.H && gx >= 0 && gx < a.W && (j == 0 || second_piece))
                               ? (uint32_t)((gy * a.W + gx) * a.C) * 4 + pcg[j] : 0x80000000u;
             }
         } else {
@@ -284,15 +321,16 @@ __global__ __launch_bounds__(WG_THREADS, 1) void winograd_fwd_kernel(const WinoA
     const int row_a = ti == 0 ? 0 : ti == 2 ? 2 : 1;
     const int row_b = ti == 2 ? 1 : ti == 3 ? 3 : 2;
     const float sgn = ti == 1 ? 1.f : -1.f;
-    const int unit0 = (cg * 2 * WG_HALO + 2 * (tt >> 3)) * WG_RAW_PITCH + (tt & 7);
+    const int tseg = SEG == 1 ? 0 : (tt & 7) / (8 / SEG);     // the piece the thread's tile belongs to
+    const int unit0 = cg * 2 * WG_PLANE + 2 * (tt >> 3) * WG_RAW_PITCH + (tt & 7) + tseg;
     const int src_a = (unit0 + row_a * WG_RAW_PITCH) * 4, src_b = (unit0 + row_b * WG_RAW_PITCH) * 4;
     // row offsets of the thread's tile in the i-th item of this block: src_a / src_b, or the zeros
     auto patch_rows = [&](int i, int& oa, int& ob) {
         oa = src_a;
         ob = src_b;
         if (STACKED && i < n_my) {
-            const int r0 = wino_decode(a, item0 + i * gx8).y0 + 2 * (tt >> 3);   // the tile's first output row
-            const int zeros = (cg * 2 * WG_HALO * WG_RAW_PITCH + 9) * 4;
+            const int r0 = seg_pos<SEG>(a, item0 + i * gx8, tseg).y0 + 2 * (tt >> 3);   // the tile's first output row
+            const int zeros = (cg * 2 * WG_PLANE + WG_HALO * WG_RAW_PITCH) * 4;
             if (ti == 0 && r0 % a.img_h == 0) oa = zeros;
             if (ti == 3 && (r0 + 2) % a.img_h == 0) ob = zeros;
         }
@@ -300,7 +338,7 @@ __global__ __launch_bounds__(WG_THREADS, 1) void winograd_fwd_kernel(const WinoA
     float4_t t[4];
     float4_t dc[2][2];                         // column s of the patch waits in dc[s & 1] until its section
     auto read_col_at = [&](const float* ra, const float* rb, int s) {   // the same through per-lane pointers
-        const int o = (((s & 1) * WG_HALO) * WG_RAW_PITCH + (s >> 1)) * 4;
+        const int o = ((s & 1) * WG_PLANE + (s >> 1)) * 4;
         dc[s & 1][0] = *(const float4_t*)(ra + o);
         dc[s & 1][1] = *(const float4_t*)(rb + o);
     };
@@ -364,9 +402,9 @@ __global__ __launch_bounds__(WG_THREADS, 1) void winograd_fwd_kernel(const WinoA
     store_raw(1, 1);
     load_raw(l_cc);
     advance_l();
-    if (STACKED && tid < 64) {                 // the zeros: units 9 and 10 of row 0 of the 4 planes, both stages
+    if (STACKED && tid < 64) {                 // the zeros: the two units behind the rows of the 4 planes, both stages
         const int stage = tid >> 5, plane = (tid >> 3) & 3, e = tid & 7;
-        lds[WG_RAW_OFF + stage * WG_RAW_STAGE + (plane * WG_HALO * WG_RAW_PITCH + 9) * 4 + e] = 0.f;
+        lds[WG_RAW_OFF + stage * WG_RAW_STAGE + (plane * WG_PLANE + WG_HALO * WG_RAW_PITCH) * 4 + e] = 0.f;
     }
     // patch rows of the step that stage 2 reads next: item p_i of this block, chunk p_cc
     int p_i = 0, p_cc = 0;
@@ -485,7 +523,7 @@ __global__ __launch_bounds__(WG_THREADS, 1) void winograd_fwd_kernel(const WinoA
             const WinoItem w = wino_decode(a, item0 + m_i * gx8);
             const int k0 = w.kb * WG_BN;
             float* stg = lds + WG_OUT_OFF;
-            const size_t oimg = (size_t)w.n * a.H * a.W * a.K;
+            const size_t oimg = SEG == 1 ? (size_t)w.n * a.H * a.W * a.K : 0;
             const int kl = wn * 32 + (lane & 31);
             // accumulator element e of this lane is tile wm*32 + 8*(e/4) + 4*(lane>>5) + e%4, channel kl;
             // its 2 x 2 output pixels sit at a per-lane base plus an offset that depends on (e, i) only
@@ -539,8 +577,11 @@ __global__ __launch_bounds__(WG_THREADS, 1) void winograd_fwd_kernel(const WinoA
             constexpr int NV = 256 * (WG_BN / 4) / WG_THREADS;
             const int k4 = (tid & 15) * 4, pcol = (tid >> 4) & 15, prow = tid >> 8;
             const uint32_t out_bytes = (uint32_t)a.H * a.W * a.K * 4;
-            const bool col_ok = w.x0 + pcol < a.W && k0 + k4 < a.K;
-            const uint32_t obase = (uint32_t)(((w.y0 + prow) * a.W + w.x0 + pcol) * a.K + k0 + k4) * 4;
+            // the thread's pixel column pcol lies in piece pcol / SEGW: rows sy0 + ..., column sx0 + pcol
+            const SegPos sp = seg_pos<SEG>(a, item0 + m_i * gx8, SEG == 1 ? 0 : pcol / SEGW);
+            const int sy0 = sp.y0, sx0 = sp.x0 - (SEG == 1 ? 0 : (pcol / SEGW) * SEGW);
+            const bool col_ok = sp.ok && sx0 + pcol < a.W && k0 + k4 < a.K;
+            const uint32_t obase = (uint32_t)(((sy0 + prow) * a.W + sx0 + pcol) * a.K + k0 + k4) * 4;
             const int row_stride = 2 * a.W * a.K * 4;
             uint32_t mbits = 0;
             auto fetch_mask = [&]() {
@@ -549,7 +590,7 @@ __global__ __launch_bounds__(WG_THREADS, 1) void winograd_fwd_kernel(const WinoA
                 float4_t mk[NV];
 #pragma unroll
                 for (int it = 0; it < NV; ++it) {
-                    const uint32_t voff = (col_ok && w.y0 + prow + 2 * it < a.H) ? obase : 0x80000000u;
+                    const uint32_t voff = (col_ok && sy0 + prow + 2 * it < a.H) ? obase : 0x80000000u;
                     mk[it] = __builtin_bit_cast(
                         float4_t, __builtin_amdgcn_raw_buffer_load_b128(omr, voff, it * row_stride, 2));
                 }
@@ -566,7 +607,7 @@ __global__ __launch_bounds__(WG_THREADS, 1) void winograd_fwd_kernel(const WinoA
                     (void*)(a.unpool_idx + oimg), 0, out_bytes / 4, 0x00020000);
 #pragma unroll
                 for (int it = 0; it < NV; ++it) {
-                    const uint32_t voff = (col_ok && w.y0 + prow + 2 * it < a.H) ? obase / 4 : 0x80000000u;
+                    const uint32_t voff = (col_ok && sy0 + prow + 2 * it < a.H) ? obase / 4 : 0x80000000u;
                     iw[UNPOOL ? it : 0] = __builtin_amdgcn_raw_buffer_load_b32(ir, voff, it * (row_stride / 4), 2);
                 }
             };
@@ -605,14 +646,16 @@ __global__ __launch_bounds__(WG_THREADS, 1) void winograd_fwd_kernel(const WinoA
                 // straddles two tiles.
                 const int Hp = a.H >> 1, Wp = a.W >> 1;
                 const int pc = (tid >> 4) & 7, pr0 = tid >> 7;
-                const size_t pimg = (size_t)w.n * Hp * Wp * a.K;
+                const size_t pimg = SEG == 1 ? (size_t)w.n * Hp * Wp * a.K : 0;
                 const uint32_t pool_elems = (uint32_t)Hp * Wp * a.K;
                 const __amdgpu_buffer_rsrc_t pyr =
                     __builtin_amdgcn_make_buffer_rsrc((void*)(a.pool_y + pimg), 0, pool_elems * 4, 0x00020000);
                 const __amdgpu_buffer_rsrc_t pir =
                     __builtin_amdgcn_make_buffer_rsrc((void*)(a.pool_idx + pimg), 0, pool_elems, 0x00020000);
-                const int py0 = w.y0 >> 1, px0 = w.x0 >> 1;
-                const bool col_ok = px0 + pc < Wp && k0 + k4 < a.K;
+                // (pooled column pc lies in piece pc / (SEGW / 2))
+                const SegPos pp = seg_pos<SEG>(a, item0 + m_i * gx8, SEG == 1 ? 0 : pc / (SEGW / 2));
+                const int py0 = pp.y0 >> 1, px0 = (pp.x0 >> 1) - (SEG == 1 ? 0 : (pc / (SEGW / 2)) * (SEGW / 2));
+                const bool col_ok = pp.ok && px0 + pc < Wp && k0 + k4 < a.K;
                 // (once per ReLU setting: no test of a run-time flag per element, and selects instead of
                 // branches for the running maximum)
                 auto pool_rows = [&](auto with_relu) {
@@ -673,7 +716,7 @@ __global__ __launch_bounds__(WG_THREADS, 1) void winograd_fwd_kernel(const WinoA
                         // writes to the store's data registers with no wait state, and on this part the first
                         // dword of the stored rows then came out overwritten (lanes 12-15 of every 16).  With an
                         // immediate scalar offset it inserts the wait state itself.
-                        const uint32_t voff = ((col_ok && w.y0 + prow + 2 * it < a.H) ? obase : 0x80000000u) +
+                        const uint32_t voff = ((col_ok && sy0 + prow + 2 * it < a.H) ? obase : 0x80000000u) +
                                               (uint32_t)(it * row_stride);
                         float4_t v = *(const float4_t*)(src + it * 2 * WG_PIX * WG_OP) + b4;
                         if (RELU) {
@@ -695,12 +738,12 @@ __global__ __launch_bounds__(WG_THREADS, 1) void winograd_fwd_kernel(const WinoA
                     // of the pooling: (2 row + i, 2 column + j) gets the value where the byte says 4 | 2 i + j
                     const __amdgpu_buffer_rsrc_t fr = __builtin_amdgcn_make_buffer_rsrc(
                         (void*)(a.unpool_y + 4 * oimg), 0, out_bytes * 4, 0x00020000);
-                    const uint32_t fbase = (uint32_t)((2 * (w.y0 + prow) * 2 * a.W + 2 * (w.x0 + pcol)) * a.K + k0 + k4) * 4;
+                    const uint32_t fbase = (uint32_t)((2 * (sy0 + prow) * 2 * a.W + 2 * (sx0 + pcol)) * a.K + k0 + k4) * 4;
                     const uint32_t frow = (uint32_t)(2 * a.W * a.K) * 4;        // one full-resolution row
                     typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
     #pragma unroll
                     for (int it = 0; it < NV; ++it) {
-                        const bool ok = col_ok && w.y0 + prow + 2 * it < a.H;
+                        const bool ok = col_ok && sy0 + prow + 2 * it < a.H;
                         const uint32_t voff = (ok ? obase : 0x80000000u) + (uint32_t)(it * row_stride);
                         const uint32_t foff = (ok ? fbase : 0x80000000u) + (uint32_t)it * (4 * frow);
                         const float4_t v = *(const float4_t*)(src + it * 2 * WG_PIX * WG_OP) + b4;
@@ -764,6 +807,8 @@ extern "C" int pd_conv3x3_winograd_filter_f32(const float* w, float* u, int C, i
 
 namespace {
 
+int g_pieces_mode = 0;   // pd_conv3x3_winograd_set_pieces: 0 = by item count, 1 = wherever the shape allows, -1 = never
+
 int wino_fwd_launch(const char* who, const float* x, const float* u, const float* bias, const float* in_mask,
                     const float* out_mask, float* y, float* pool_y, uint8_t* pool_idx, int N, int H, int W, int C,
                     int K, int relu, void* stream, const uint8_t* unpool_idx = nullptr, float* unpool_y = nullptr) {
@@ -792,20 +837,44 @@ int wino_fwd_launch(const char* who, const float* x, const float* u, const float
     a.tiles_y = (a.H + WG_PIX - 1) / WG_PIX;
     a.k_blocks = (K + WG_BN - 1) / WG_BN;
     a.n_chunks = C / WG_CC;
-    const long items = (long)a.N * a.tiles_x * a.tiles_y * a.k_blocks;
-    PD_REQUIRE(items <= 0x7ffffff0L, PD_ESHAPE, "%s: too many tiles", who);
-    a.n_items = (int)items;
-    a.items_per_xcd = (int)((items + WG_XCD - 1) / WG_XCD);
     // one persistent block per CU (the kernel needs a CU's whole register file), in multiples of 8
     int dev = 0, cus = 0;
     PD_HIP(hipGetDevice(&dev));
     PD_HIP(hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev));
-    long blocks = (long)(cus / WG_XCD) * WG_XCD;
-    if (blocks < WG_XCD) blocks = WG_XCD;
+    const long cu_blocks = (long)(cus / WG_XCD) * WG_XCD > 0 ? (long)(cus / WG_XCD) * WG_XCD : WG_XCD;
+    // A stacked batch whose width is a multiple of 8 (4) but not of 16 pixels can use work items of two (four)
+    // pieces: no padding columns, 7/8 of the items at widths 56 and 28.  What counts is the number of items the
+    // busiest block gets (the blocks of a die share its items evenly): pieces are used when that number falls
+    // (64 images of 56 x 56 with 256 output channels: 13 instead of 14 items per block), not when both divide
+    // into the same number of rounds (28 x 28 with 512 channels: 7 and 6.1 -> 7; the squares then win by their
+    // smaller halo).
+    const long square_items = (long)a.N * a.tiles_x * a.tiles_y * a.k_blocks;
+    int seg = !stacked || W % WG_PIX == 0 ? 1 : W % 8 == 0 ? 2 : W % 4 == 0 ? 4 : 1;
+    a.segs_per_row = W / (WG_PIX / seg);
+    a.n_segs = a.segs_per_row * a.tiles_y;
+    const long piece_items = (long)((a.n_segs + seg - 1) / seg) * a.k_blocks;
+    auto busiest = [&](long n) {
+        const long per_xcd = (n + WG_XCD - 1) / WG_XCD, per_die_blocks = cu_blocks / WG_XCD;
+        return (per_xcd + per_die_blocks - 1) / per_die_blocks;
+    };
+    if (seg > 1 && (g_pieces_mode < 0 || (g_pieces_mode == 0 && busiest(piece_items) >= busiest(square_items)))) seg = 1;
+    const long items = seg == 1 ? square_items : piece_items;
+    PD_REQUIRE(items <= 0x7ffffff0L, PD_ESHAPE, "%s: too many tiles", who);
+    a.n_items = (int)items;
+    a.items_per_xcd = (int)((items + WG_XCD - 1) / WG_XCD);
+    long blocks = cu_blocks;
     if (blocks > (long)a.items_per_xcd * WG_XCD) blocks = (long)a.items_per_xcd * WG_XCD;
     dim3 grid((unsigned)blocks);
     hipStream_t s = (hipStream_t)stream;
-    if (unpool_y) {
+    if (seg == 2) {
+        if (unpool_y) winograd_fwd_kernel<false, false, true, true, 2><<<grid, WG_THREADS, 0, s>>>(a);
+        else if (a.pool_y) winograd_fwd_kernel<false, true, true, false, 2><<<grid, WG_THREADS, 0, s>>>(a);
+        else winograd_fwd_kernel<false, false, true, false, 2><<<grid, WG_THREADS, 0, s>>>(a);
+    } else if (seg == 4) {
+        if (unpool_y) winograd_fwd_kernel<false, false, true, true, 4><<<grid, WG_THREADS, 0, s>>>(a);
+        else if (a.pool_y) winograd_fwd_kernel<false, true, true, false, 4><<<grid, WG_THREADS, 0, s>>>(a);
+        else winograd_fwd_kernel<false, false, true, false, 4><<<grid, WG_THREADS, 0, s>>>(a);
+    } else if (unpool_y) {
         if (stacked) winograd_fwd_kernel<false, false, true, true><<<grid, WG_THREADS, 0, s>>>(a);
         else winograd_fwd_kernel<false, false, false, true><<<grid, WG_THREADS, 0, s>>>(a);
     } else if (stacked) {
@@ -821,6 +890,12 @@ int wino_fwd_launch(const char* who, const float* x, const float* u, const float
 }
 
 }  // namespace
+
+extern "C" int pd_conv3x3_winograd_set_pieces(int mode) {
+    PD_REQUIRE(mode >= -1 && mode <= 1, PD_EINVAL, "pd_conv3x3_winograd_set_pieces: mode is -1, 0 or 1");
+    g_pieces_mode = mode;
+    return PD_OK;
+}
 
 extern "C" int pd_conv3x3_winograd_fwd_nhwc_f32(const float* x, const float* u, const float* bias,
                                                 const float* in_mask, const float* out_mask, float* y, int N, int H,

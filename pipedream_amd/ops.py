@@ -435,6 +435,13 @@ def set_conv_algorithm(name):
     _CONV_ALGO = name
 
 
+def set_conv_pieces(mode):
+    """Work items of the Winograd forward / input-gradient kernel for stacked batches whose width is a multiple of
+    8 or 4 but not of 16 pixels: "auto" (pieces of 16 x 8 or 16 x 4 pixels when they lower the busiest compute
+    unit's item count), "always", "never".  Same results bit for bit."""
+    _cabi.lib().pd_conv3x3_winograd_set_pieces({"auto": 0, "always": 1, "never": -1}[mode])
+
+
 def _use_winograd(c, k, h, w):
     """Whether a convolution with c input and k output channels on h x w images takes the Winograd kernel:
     channel counts it supports, an image it can address with 32-bit offsets (the limits its entry point

@@ -33,6 +33,18 @@ def _nhwc(t):
     return t.cuda().contiguous(memory_format=torch.channels_last)
 
 
+@pytest.fixture(autouse=True)
+def _pieces_back_to_auto():
+    yield
+    ops.set_conv_pieces("auto")
+
+
+def request_pieces(mode):
+    """Work items made of pieces (stacked batches of width 8 k or 4 k) are chosen by item count, which tiny test
+    shapes never reach: force them, or rule them out (the fixture above restores the built-in choice)."""
+    ops.set_conv_pieces(mode)
+
+
 def _direct_conv(x, w, b):
     """Brute-force NCHW 3x3 / pad 1 convolution in numpy float64."""
     N, C, H, W = x.shape
@@ -419,8 +431,15 @@ def test_transformed_filter_layout_and_values(C, K, rot180, offset, conv_algorit
                                         (5, 24, 40, 22, 18),    # ragged in both directions, K % 64 != 0
                                         (3, 32, 64, 28, 28),
                                         (7, 8, 8, 2, 34),       # images of one tile row
-                                        (2, 16, 16, 56, 24)])
-def test_batch_of_images_whose_height_is_no_multiple_of_the_tile(N, C, K, H, W, conv_algorithm):
+                                        (2, 16, 16, 56, 24),
+                                        # widths of 8 k (4 k) pixels: work items of two (four) pieces
+                                        (2, 16, 64, 56, 56),
+                                        (3, 8, 128, 28, 12),    # two blocks of output channels
+                                        (2, 8, 16, 8, 40),      # five pieces per 16 rows: items straddle them
+                                        (5, 8, 8, 6, 4),        # one piece per 16 rows
+                                        (3, 16, 32, 10, 72)])
+@pytest.mark.parametrize("pieces", ["never", "always"])
+def test_batch_of_images_whose_height_is_no_multiple_of_the_tile(N, C, K, H, W, pieces, conv_algorithm):
     """Images of even height that is no multiple of 16 rows are processed as one tall image (work items
     straddle images).  Nothing may leak across an image boundary: every image of the batch must come out
     bit for bit as when it is convolved alone (a batch of one never takes that path), in the forward
@@ -428,6 +447,9 @@ def test_batch_of_images_whose_height_is_no_multiple_of_the_tile(N, C, K, H, W, 
     batch is also checked against torch in fp64."""
     if conv_algorithm != "winograd":
         pytest.skip("a property of the Winograd kernels' work items")
+    if pieces == "always" and not (W % 16 != 0 and W % 4 == 0 and H % 16 != 0):
+        pytest.skip("this width has no work items made of pieces")
+    request_pieces(pieces)
     torch.manual_seed(N * 100 + H)
     x = _nhwc(torch.randn(N, C, H, W))
     w = _nhwc(torch.randn(K, C, 3, 3) / math.sqrt(9 * C))
@@ -458,15 +480,22 @@ def test_batch_of_images_whose_height_is_no_multiple_of_the_tile(N, C, K, H, W, 
 @pytest.mark.parametrize("N,C,K,H,W", [(2, 16, 32, 16, 16),     # pooled 8 x 8: one tile
                                         (3, 64, 64, 28, 28),     # pooled 14 x 14: stacked batch
                                         (1, 32, 64, 40, 72),     # several tiles, ragged
-                                        (2, 8, 24, 12, 20)])
+                                        (2, 8, 24, 12, 20),
+                                        (2, 16, 32, 56, 56),     # pooled 28 x 28: work items of four pieces
+                                        (2, 8, 32, 112, 112),    # pooled 56 x 56: work items of two pieces
+                                        (3, 8, 8, 12, 48)])
 @pytest.mark.parametrize("producer", ["conv_pool", "maxpool"])
-def test_pooling_backward_in_the_consuming_convolution_kernel(N, C, K, H, W, producer, conv_algorithm):
+@pytest.mark.parametrize("pieces", ["never", "always"])
+def test_pooling_backward_in_the_consuming_convolution_kernel(N, C, K, H, W, producer, pieces, conv_algorithm):
     """ReLU + MaxPool2d followed by a convolution, with and without a PoolGradLink between them: the linked pair
     lets the convolution's input-gradient kernel write the gradient in front of the pooling; every output
     and every gradient must equal the unlinked pair's bit for bit (the same values reach the same kernels),
     and the pooling backward kernel must not run in the linked pair."""
     if conv_algorithm != "winograd":
         pytest.skip("the fused epilogue belongs to the Winograd kernel")
+    if pieces == "always" and not ((W // 2) % 16 != 0 and (W // 2) % 4 == 0 and N > 1 and (H // 2) % 16 != 0):
+        pytest.skip("the pooled width has no work items made of pieces")
+    request_pieces(pieces)
     torch.manual_seed(N + C + H)
 
     def build(linked):
@@ -538,3 +567,28 @@ def test_fused_input_gradient_and_unpooling_on_random_shapes(N, C, K, H, W, conv
     want_dx = ops.conv3x3_input_grad(dy, w, x_rectified=pooled)
     assert torch.equal(dx, want_dx)
     assert torch.equal(dfull, ops.maxpool2x2_idx_backward(want_dx, idx, 2 * H, 2 * W, relu_mask=True))
+
+
+def test_pieces_equal_squares_at_vgg_size(conv_algorithm):
+    """64 images of 56 x 56 pixels, 128 -> 256 channels (conv3_1 of VGG16), and 28 x 28, 256 -> 512 (conv4_1): the
+    forward pass, the pooled forward pass and the input gradient (plain, and with the pooling backward in its
+    epilogue) with work items of two / four pieces are bit-identical to the 16 x 16 squares, and the built-in
+    choice gives those bits too."""
+    if conv_algorithm != "winograd":
+        pytest.skip("a property of the Winograd kernels' work items")
+    for (C, K, HW) in ((128, 256, 56), (256, 512, 28)):
+        gen = torch.Generator(device="cuda").manual_seed(HW)
+        x = torch.randn(64, C, HW, HW, device="cuda", generator=gen).contiguous(memory_format=torch.channels_last)
+        w = (torch.randn(K, C, 3, 3, device="cuda", generator=gen) / math.sqrt(9 * C)).contiguous(
+            memory_format=torch.channels_last)
+        b = torch.randn(K, device="cuda", generator=gen)
+        dy = torch.randn(64, K, HW, HW, device="cuda", generator=gen).contiguous(memory_format=torch.channels_last)
+        idx = torch.randint(0, 8, (64, C, HW, HW), device="cuda", generator=gen, dtype=torch.uint8).contiguous(
+            memory_format=torch.channels_last)
+        out = {}
+        for mode in ("never", "always", "auto"):
+            ops.set_conv_pieces(mode)
+            out[mode] = (ops.conv3x3_forward(x, w, b, relu=True),) + ops.conv3x3_forward_pool(x, w, b, relu=True) + \
+                (ops.conv3x3_input_grad(dy, w),) + ops.conv3x3_input_grad_unpool(dy, w, idx)
+        for mode in ("always", "auto"):
+            assert all(torch.equal(p, q) for p, q in zip(out["never"], out[mode])), (C, K, HW, mode)
