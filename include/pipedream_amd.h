@@ -347,7 +347,7 @@ int pd_gemm_bf16(int trans_a, int trans_b, int M, int N, int K,
                  int batch_outer, int batch_inner, const int64_t* strides, void* stream);
 /* Tuning and test hook: force the tile of the direct-to-LDS kernel behind pd_gemm_bf16 / pd_gemm_bf16_gelu
  * for products it can take (K a multiple of 128): (128, 128) or (256, 256); (0, 0) restores the built-in
- * choice (256 x 256 when there are at least 256 such tiles and K >= 2048, else 128 x 128).  Process-wide,
+ * choice (256 x 256 when there are at least 192 such tiles, else 128 x 128).  Process-wide,
  * not thread-safe against concurrent GEMM calls.  No counterpart in the reference (its GEMMs are library calls). */
 int pd_gemm_bf16_set_tile(int bm, int bn);
 

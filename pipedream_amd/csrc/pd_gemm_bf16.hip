@@ -31,6 +31,8 @@
 // that die's L2.
 // Epilogue: (+ bias[N] fp32) (+ residual[M][N] bf16) -> bf16, or fp32 with optional
 // accumulation into C (weight gradients summed over micro-batches).
+#include <type_traits>
+
 #include "pd_internal.h"
 
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
@@ -100,6 +102,93 @@ __device__ __forceinline__ float bf2f(uint16_t h) { return __uint_as_float((uint
 // rounding) and beta*C accumulated on the vectorised side.  `vec` = N, ldc, ldr and the
 // batch offsets are multiples of 8 and C / residual are 16-byte aligned; otherwise the
 // element-wise path is used.
+// One staged 32-row block of a wave's tile -> C, for a block that lies inside the matrix: all LDS reads first,
+// then the operand loads, then the arithmetic and the 16-byte stores.  F32: fp32 output (BETA: accumulated into
+// C); RES: bf16 residual added; ACT: 1 = also store gelu(C) to aux_out, 2 = multiply by gelu'(aux_in).
+template <int TN, bool F32, bool BETA, bool RES, int ACT>
+__device__ __forceinline__ void store_rows_full(const GemmBf16Args& a, const float* stage, int row0, int col0,
+                                                long long c_off, int lane) {
+    constexpr int COLS = 32 * TN, P = COLS + 8;
+    if constexpr (F32) {
+        constexpr int LPR = COLS / 4, ITER = 32 * LPR / 64;
+        const int c4 = (lane % LPR) * 4, r_in = lane / LPR;
+        float4_t v[ITER], old[ITER];
+#pragma unroll
+        for (int it = 0; it < ITER; ++it) v[it] = *(const float4_t*)(stage + (it * (64 / LPR) + r_in) * P + c4);
+        float* const base = (float*)a.C + c_off + (long long)(row0 + r_in) * a.ldc + col0 + c4;
+        if (BETA) {
+#pragma unroll
+            for (int it = 0; it < ITER; ++it) old[it] = *(const float4_t*)(base + (long long)it * (64 / LPR) * a.ldc);
+        }
+#pragma unroll
+        for (int it = 0; it < ITER; ++it) {
+            if (BETA) v[it] += a.beta * old[it];
+            *(float4_t*)(base + (long long)it * (64 / LPR) * a.ldc) = v[it];
+        }
+    } else {
+        constexpr int LPR = COLS / 8, ITER = 32 * LPR / 64;
+        const int c8 = (lane % LPR) * 8, r_in = lane / LPR;
+        float4_t v0[ITER], v1[ITER];
+#pragma unroll
+        for (int it = 0; it < ITER; ++it) {
+            const float* src = stage + (it * (64 / LPR) + r_in) * P + c8;
+            v0[it] = *(const float4_t*)src;
+            v1[it] = *(const float4_t*)(src + 4);
+        }
+        u16x8 extra[(RES || ACT == 2) ? ITER : 1];
+        if (RES) {
+            const uint16_t* rb = a.residual + c_off + (long long)(row0 + r_in) * a.ldr + col0 + c8;
+#pragma unroll
+            for (int it = 0; it < ITER; ++it) extra[it] = *(const u16x8*)(rb + (long long)it * (64 / LPR) * a.ldr);
+        }
+        if (ACT == 2) {
+            const uint16_t* xb = a.aux_in + (long long)(row0 + r_in) * a.ld_aux + col0 + c8;
+#pragma unroll
+            for (int it = 0; it < ITER; ++it) extra[it] = *(const u16x8*)(xb + (long long)it * (64 / LPR) * a.ld_aux);
+        }
+        uint16_t* const cb = (uint16_t*)a.C + c_off + (long long)(row0 + r_in) * a.ldc + col0 + c8;
+#pragma unroll
+        for (int it = 0; it < ITER; ++it) {
+            float v[8] = {v0[it][0], v0[it][1], v0[it][2], v0[it][3], v1[it][0], v1[it][1], v1[it][2], v1[it][3]};
+            if (RES) {
+#pragma unroll
+                for (int q = 0; q < 8; ++q) v[q] += bf2f(extra[it][q]);
+            }
+            if (ACT == 2) {
+#pragma unroll
+                for (int q = 0; q < 8; ++q) v[q] *= gelu_grad_f(bf2f(extra[it][q]));
+            }
+            u16x8 o;
+#pragma unroll
+            for (int q = 0; q < 8; ++q) o[q] = f2bf(v[q]);
+            *(u16x8*)(cb + (long long)it * (64 / LPR) * a.ldc) = o;
+            if (ACT == 1) {
+                u16x8 gg;
+#pragma unroll
+                for (int q = 0; q < 8; ++q) gg[q] = f2bf(gelu_f(bf2f(o[q])));
+                *(u16x8*)(a.aux_out + (long long)(row0 + r_in + it * (64 / LPR)) * a.ld_aux + col0 + c8) = gg;
+            }
+        }
+    }
+}
+
+// A wave's whole tile, inside the matrix, in one output form: stage each 32-row block, then store it.
+template <int TM, int TN, bool F32, bool BETA, bool RES, int ACT>
+__device__ __forceinline__ void store_tile_full(const GemmBf16Args& a, float16_t (&acc)[TM][TN], const float (&bv)[TN],
+                                                int m0w, int n0w, long long c_off, float* stage, int lane) {
+    constexpr int P = 32 * TN + 8;
+    const int idx = lane % 32, h = lane / 32;
+#pragma unroll
+    for (int i = 0; i < TM; ++i) {
+#pragma unroll
+        for (int j = 0; j < TN; ++j)
+#pragma unroll
+            for (int e = 0; e < 16; ++e)
+                stage[(8 * (e / 4) + 4 * h + (e % 4)) * P + j * 32 + idx] = a.alpha * acc[i][j][e] + bv[j];
+        store_rows_full<TN, F32, BETA, RES, ACT>(a, stage, m0w + i * 32, n0w, c_off, lane);
+    }
+}
+
 template <int TM, int TN>
 __device__ __forceinline__ void store_tile(const GemmBf16Args& a, float16_t (&acc)[TM][TN], int m0w, int n0w,
                                            long long c_off, float* stage, int lane) {
@@ -139,6 +228,20 @@ __device__ __forceinline__ void store_tile(const GemmBf16Args& a, float16_t (&ac
     for (int j = 0; j < TN; ++j) {
         const int col = n0w + j * 32 + idx;
         bv[j] = (a.bias && col < a.N) ? a.bias[col] : 0.f;
+    }
+    // The wave's tile lies inside the matrix (every transformer product): one loop per output form, without a
+    // test inside, so that the LDS reads, the operand loads and the stores of a 32-row block are issued in
+    // batches.  (With the form and the bounds tested per 16-byte vector every read waited for its own round
+    // trip: 47 000 cycles for a 128 x 128 wave tile, more than the 256 x 256 kernel's whole k loop at K = 1024.)
+    if (m0w + 32 * TM <= a.M && n0w + 32 * TN <= a.N) {
+        if (a.out_f32) {
+            if (a.beta != 0.f) store_tile_full<TM, TN, true, true, false, 0>(a, acc, bv, m0w, n0w, c_off, stage, lane);
+            else store_tile_full<TM, TN, true, false, false, 0>(a, acc, bv, m0w, n0w, c_off, stage, lane);
+        } else if (a.act == 1) store_tile_full<TM, TN, false, false, false, 1>(a, acc, bv, m0w, n0w, c_off, stage, lane);
+        else if (a.act == 2) store_tile_full<TM, TN, false, false, false, 2>(a, acc, bv, m0w, n0w, c_off, stage, lane);
+        else if (a.residual) store_tile_full<TM, TN, false, false, true, 0>(a, acc, bv, m0w, n0w, c_off, stage, lane);
+        else store_tile_full<TM, TN, false, false, false, 0>(a, acc, bv, m0w, n0w, c_off, stage, lane);
+        return;
     }
 #pragma unroll
     for (int i = 0; i < TM; ++i) {
@@ -742,10 +845,10 @@ static int gemm_bf16_run(int trans_a, int trans_b, int M, int N, int K, const ui
         if (g_force_bm == 256 && g_force_bn == 256) return launch_gemm_bf16_dma<256, 256>(trans_a, trans_b, g, batch, s);
         if (g_force_bm == 128 && g_force_bn == 128) return launch_gemm_bf16_dma<128, 128>(trans_a, trans_b, g, batch, s);
     }
-    // A 256 x 256 tile pays about 25 us of ring fill and epilogue that nothing overlaps (one block per CU); below
-    // a reduction depth of 2048 two co-resident 128 x 128 blocks per CU, which overlap each other's, are faster
-    // (4096 x 4096 x 1024: 43 against 50 us; x 2048: 80 against 74 us).
-    if (dma_ok && wide && tiles256 >= 256 && K >= 2048) return launch_gemm_bf16_dma<256, 256>(trans_a, trans_b, g, batch, s);
+    // 256 x 256 tiles (one block per CU, half the LDS reads per MFMA) from 192 tiles on, i.e. three quarters of
+    // the CUs busy: 4096 x 4096 x 1024 takes 41 us against 49 with 128 x 128 tiles, 4096 x 3072 x 1024 (192
+    // tiles) 34 against 39; products with fewer large tiles (4096 x 1024: 64) run two 128 x 128 blocks per CU.
+    if (dma_ok && wide && tiles256 >= 192) return launch_gemm_bf16_dma<256, 256>(trans_a, trans_b, g, batch, s);
     if (dma_ok && M >= 128 && N >= 128) return launch_gemm_bf16_dma<128, 128>(trans_a, trans_b, g, batch, s);
     if (wide && tiles256 >= 192) return launch_gemm_bf16<256, 256, 2, 4>(trans_a, trans_b, g, batch, s);
     // narrow outputs (attention: N = head dimension): tall tiles, all waves stacked along M

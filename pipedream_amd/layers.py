@@ -629,8 +629,7 @@ class _TransformerLayerFn(torch.autograd.Function):
         def linear_backward(d_out, inp, w, b, through_gelu_of=None):
             # parameters are read (and their bf16 image taken) at backward time: the version
             # load_old_params made current
-            _accumulate(w, lambda: ops.gemm_bf16(d_out, inp, trans_a=True, out_f32=True),
-                        lambda acc: ops.gemm_bf16(d_out, inp, trans_a=True, out=acc, beta=1.0))
+            _accumulate(w, lambda: ops.gemm_bf16_wgrad(d_out, inp), lambda acc: ops.gemm_bf16_wgrad(d_out, inp, acc))
             # (the bias gradient, a column sum of d_out, waits for the end of the layer: all column sums of
             # the layer's backward then take two launches)
             if b.grad is None:

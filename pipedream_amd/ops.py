@@ -823,6 +823,34 @@ def gemm_bf16_gelu_backward(dy, w, f):
     return df
 
 
+def gemm_bf16_wgrad(dy, x, acc=None):
+    """Weight gradient of a bf16 Linear layer in fp32: ``dy[T, N]^T x[T, K]``, returned as a new [N, K] tensor or
+    added to ``acc``.  A product with few output tiles (the 1024 x 1024 attention projection: 64 tiles of
+    128 x 128 for 256 CUs) is split over the tokens into partial products, one batch entry each, which a second
+    kernel adds in index order (deterministic)."""
+    _mat_bf16(dy, "dy")
+    _mat_bf16(x, "x")
+    T, N = dy.shape
+    K = x.shape[1]
+    tiles = -(-N // 128) * -(-K // 128)
+    splits = min(256 // tiles, T // 1024, 8) if tiles <= 64 else 1
+    if splits < 2 or T % (splits * 128) != 0 or N % 4 != 0 or K % 4 != 0:
+        if acc is None:
+            return gemm_bf16(dy, x, trans_a=True, out_f32=True)
+        return gemm_bf16(dy, x, trans_a=True, out=acc, beta=1.0)
+    part = torch.empty((splits, N, K), dtype=torch.float32, device=dy.device)
+    rows = T // splits
+    strides = (ctypes.c_int64 * 6)(rows * dy.stride(0), 0, rows * x.stride(0), 0, N * K, 0)
+    lib = _cabi.lib()
+    with _timed("gemm_bf16", 2.0 * N * K * T):
+        lib.pd_gemm_bf16(1, 0, N, K, rows, _ptr(dy), dy.stride(0), _ptr(x), x.stride(0), _ptr(part), K, 1, 1.0, 0.0,
+                         None, None, 0, splits, 1, strides, _cabi.stream_ptr())
+    out = acc if acc is not None else torch.empty((N, K), dtype=torch.float32, device=dy.device)
+    lib.pd_splitk_reduce_f32(_ptr(part), splits, N, K, None, 0, 1.0 if acc is not None else 0.0, _ptr(out),
+                             out.stride(0), _cabi.stream_ptr())
+    return out
+
+
 def _batched(ta, tb, M, N, K, A, a_off, lda, B, b_off, ldb, C, c_off, ldc, alpha, bo, bi, strides):
     arr = (ctypes.c_int64 * 6)(*strides)
     es = 2

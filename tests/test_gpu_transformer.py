@@ -61,7 +61,7 @@ def test_gemm_bf16_epilogues():
 @pytest.mark.parametrize("tile", [128, 256])
 def test_gemm_bf16_large_tiles(M, N, K, ta, tb, tile):
     """K a multiple of 128 runs the direct-to-LDS ring kernel (one to three ring rounds), here with each of
-    its two tile sizes forced in turn (the built-in choice takes 256 x 256 tiles only for K >= 2048); other K
+    its two tile sizes forced in turn (the built-in choice takes 256 x 256 tiles from 192 of them on); other K
     the register-staged kernels; M and N that are not tile multiples exercise the clamped loads and the masked
     vector stores.  The fp32 reference product is computed on the device by torch from the same bf16 inputs."""
     from pipedream_amd import _cabi, ops
@@ -81,16 +81,16 @@ def test_gemm_bf16_large_tiles(M, N, K, ta, tb, tile):
 
 
 def test_gemm_bf16_built_in_tile_choice_and_hook_errors():
-    """Deep reductions take the 256 x 256 kernel by themselves, shallow ones the 128 x 128 kernel; both agree with
-    the forced runs bit for bit (the tile size does not change the order of a dot product's additions)."""
+    """Whatever tile the built-in choice takes (256 x 256 from 192 such tiles on, else 128 x 128), it agrees with
+    both forced runs bit for bit (the tile size does not change the order of a dot product's additions)."""
     from pipedream_amd import _cabi, ops
     lib = _cabi.lib()
     with pytest.raises(_cabi.PipedreamAmdError):
         lib.pd_gemm_bf16_set_tile(64, 64)
     g = torch.Generator().manual_seed(11)
-    for K in (1024, 2048):
+    for N, K in ((4096, 1024), (1024, 2048)):
         a = (torch.randn(4096, K, generator=g) / 8).to(BF).cuda()
-        b = (torch.randn(4096, K, generator=g) / 8).to(BF).cuda()
+        b = (torch.randn(N, K, generator=g) / 8).to(BF).cuda()
         auto = ops.gemm_bf16(a, b, trans_b=True, out_f32=True)
         for tile in (128, 256):
             lib.pd_gemm_bf16_set_tile(tile, tile)
@@ -363,6 +363,23 @@ def test_full_size_stage_six_layers_vs_oracle():
     print("output %.2e, input gradient %.2e" % (errs["output"], errs["input gradient"]))
     bad = {k: v for k, v in errs.items() if not v < 2e-2}
     assert not bad, bad
+
+
+def test_weight_gradient_split_over_tokens():
+    """``ops.gemm_bf16_wgrad``: the 1024 x 1024 product (64 tiles) is split over the 4096 tokens into four partial
+    products added in index order; a wider one is not.  Fresh and accumulated, against fp64."""
+    from pipedream_amd import ops
+    g = torch.Generator().manual_seed(9)
+    for (T, N, K) in ((4096, 1024, 1024), (4096, 1024, 512), (2048, 1024, 4096), (1000, 256, 128)):
+        dy = (torch.randn(T, N, generator=g) / 8).to(BF).cuda()
+        x = torch.randn(T, K, generator=g).to(BF).cuda()
+        want = dy.double().t() @ x.double()
+        got = ops.gemm_bf16_wgrad(dy, x)
+        assert got.dtype == torch.float32 and _rel(got, want.cpu()) < 1e-5
+        acc = torch.randn(N, K, generator=g).cuda()
+        want2 = acc.double() + want
+        ops.gemm_bf16_wgrad(dy, x, acc)
+        assert _rel(acc, want2.cpu()) < 1e-5
 
 
 def test_batched_column_sums_match_the_single_ones():
