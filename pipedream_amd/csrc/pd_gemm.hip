@@ -448,6 +448,18 @@ __global__ __launch_bounds__(GEMM_THREADS) void pd_gemm_skinny_kernel(const Gemm
         sk_wait_vmcnt<0>();     // the trailing re-fetches must not outlive the block's LDS allocation
     }
 
+    if (a.M == S::BM && n0 + SK_COLS <= a.N) {
+        // the whole tile lies inside the matrix (the LSTM products): 64 stores per lane without a test each
+#pragma unroll
+        for (int i = 0; i < 2; ++i)
+#pragma unroll
+            for (int j = 0; j < TN; ++j) {
+                float* const base = C + (size_t)((wm * 2 + i) * 32 + 4 * h) * a.ldc + n0 + (wn * TN + j) * 32 + idx;
+#pragma unroll
+                for (int e = 0; e < 16; ++e) base[(size_t)(8 * (e / 4) + (e % 4)) * a.ldc] = acc[i][j][e];
+            }
+        return;
+    }
 #pragma unroll
     for (int i = 0; i < 2; ++i)
 #pragma unroll
