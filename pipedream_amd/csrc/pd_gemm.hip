@@ -264,10 +264,10 @@ int launch_gemm(int trans_a, int trans_b, const GemmArgs& g, hipStream_t s, int 
 
 // ---------------------------------------------------------------------------------------
 // Skinny split-k kernel: M <= 128 (the LSTM recurrent products with M = batch, the
-// classifier layers with M = 64), A k-contiguous.  A block owns all M rows x 128 columns
-// of one k range and is bound by fetching its operands, so they are streamed with 128-bit
-// direct-to-LDS loads (lane l's 16 bytes land at <base> + 16*l) through a ring of 8
-// stages of 16 k, 6 to 7 stages in flight, and multiplied as they arrive.
+// classifier layers with M = 64), A k-contiguous.  A block owns up to 64 rows (blockIdx.y) x
+// 128 columns of one k range and is bound by fetching its operands, so they are streamed with
+// 128-bit direct-to-LDS loads (lane l's 16 bytes land at <base> + 16*l) through a ring of 8
+// or 4 stages of 16 k, all but one or two in flight, and multiplied as they arrive.
 // Because the LDS placement of such a load is fixed, the lanes fetch a permutation that
 // makes the fragment reads conflict-free: the 16-byte slot q of row r of a k-contiguous
 // stage holds k-group q ^ ((r >> 2) & 3); a row-contiguous stage ([k][128 columns]) has its
@@ -283,7 +283,7 @@ typedef __attribute__((address_space(1))) const void* global_void_ptr;
 constexpr int SK_COLS = 128;             // tile columns
 // (ring stages of BK = 16, SK_STAGES below: 8 or 4)
 
-// WM = 2: up to 128 rows, waves 2 x 2, 64 x 64 each.  WM = 1: up to 64 rows, waves 1 x 4, 64 x 32 each.
+// Rows per block: WM = 1: 64, waves 1 x 4, 64 x 32 each (the one launched).  WM = 2: 128, waves 2 x 2, 64 x 64 each.
 template <int WM, bool B_KC, int SK_STAGES>
 struct Skinny {
     static constexpr int BM = 64 * WM;
@@ -299,14 +299,14 @@ struct Skinny {
     size_t src_a[A_PER_WAVE], src_b[B_PER_WAVE];
     uint32_t fa_addr[2][2], fb_addr[TN][2];       // [fragment][k-group g] LDS byte addresses, stage 0
 
-    __device__ __forceinline__ void init(const GemmArgs& a, int n0, int wave, int lane, uint32_t lds_base) {
+    __device__ __forceinline__ void init(const GemmArgs& a, int m0, int n0, int wave, int lane, uint32_t lds_base) {
         const int wm = wave / WN, wn = wave % WN;
         const int idx = lane % 32, h = lane / 32;
 #pragma unroll
         for (int t = 0; t < A_PER_WAVE; ++t) {
             const int row = (wave + 4 * t) * 16 + lane / 4;
             const int kq = (lane % 4) ^ ((row >> 2) & 3);
-            src_a[t] = (size_t)min(row, a.M - 1) * a.lda + kq * 4;
+            src_a[t] = (size_t)min(m0 + row, a.M - 1) * a.lda + kq * 4;
         }
 #pragma unroll
         for (int t = 0; t < B_PER_WAVE; ++t) {
@@ -399,7 +399,7 @@ __global__ __launch_bounds__(GEMM_THREADS) void pd_gemm_skinny_kernel(const Gemm
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / 64);
     const int wm = wave / S::WN, wn = wave % S::WN;
     const int idx = lane % 32, h = lane / 32;
-    const int n0 = blockIdx.x * SK_COLS;
+    const int m0 = blockIdx.y * S::BM, n0 = blockIdx.x * SK_COLS;
     const int k_begin = blockIdx.z * a.k_per_split;
     const int k_end = min(a.K, k_begin + a.k_per_split);
     const int total = k_end > k_begin ? (k_end - k_begin) / BK : 0;      // stages to multiply
@@ -415,7 +415,7 @@ __global__ __launch_bounds__(GEMM_THREADS) void pd_gemm_skinny_kernel(const Gemm
 
     if (total > 0) {
         S sk;
-        sk.init(a, n0, wave, lane, (uint32_t)(size_t)(lds_void_ptr)lds);
+        sk.init(a, m0, n0, wave, lane, (uint32_t)(size_t)(lds_void_ptr)lds);
         // k of stage number i, clamped to the last stage of the range
 #define SK_K(i) (k_begin + min((i), total - 1) * BK)
 #define SK_FILL(ST) if constexpr (ST < SK_STAGES - 1) sk.template issue<ST>(a, lds, SK_K(ST), wave);
@@ -448,13 +448,13 @@ __global__ __launch_bounds__(GEMM_THREADS) void pd_gemm_skinny_kernel(const Gemm
         sk_wait_vmcnt<0>();     // the trailing re-fetches must not outlive the block's LDS allocation
     }
 
-    if (a.M == S::BM && n0 + SK_COLS <= a.N) {
+    if (m0 + S::BM <= a.M && n0 + SK_COLS <= a.N) {
         // the whole tile lies inside the matrix (the LSTM products): 64 stores per lane without a test each
 #pragma unroll
         for (int i = 0; i < 2; ++i)
 #pragma unroll
             for (int j = 0; j < TN; ++j) {
-                float* const base = C + (size_t)((wm * 2 + i) * 32 + 4 * h) * a.ldc + n0 + (wn * TN + j) * 32 + idx;
+                float* const base = C + (size_t)(m0 + (wm * 2 + i) * 32 + 4 * h) * a.ldc + n0 + (wn * TN + j) * 32 + idx;
 #pragma unroll
                 for (int e = 0; e < 16; ++e) base[(size_t)(8 * (e / 4) + (e % 4)) * a.ldc] = acc[i][j][e];
             }
@@ -468,7 +468,7 @@ __global__ __launch_bounds__(GEMM_THREADS) void pd_gemm_skinny_kernel(const Gemm
             if (col >= a.N) continue;
 #pragma unroll
             for (int e = 0; e < 16; ++e) {
-                const int row = (wm * 2 + i) * 32 + 8 * (e / 4) + 4 * h + (e % 4);
+                const int row = m0 + (wm * 2 + i) * 32 + 8 * (e / 4) + 4 * h + (e % 4);
                 if (row < a.M) C[(size_t)row * a.ldc + col] = acc[i][j][e];
             }
         }
@@ -564,16 +564,18 @@ extern "C" int pd_gemm_splitk_f32(int trans_a, int trans_b, int M, int N, int K,
     if (!trans_a && M <= 128 && N % 4 == 0 && g.a_vec && g.b_vec && g.k_per_split % BK == 0 && K % BK == 0 &&
         (size_t)128 * (lda > ldb ? lda : ldb) * 4 < (1ull << 31)) {
         const dim3 grid((N + SK_COLS - 1) / SK_COLS, 1, splits);
-        // up to 64 rows: 8 ring stages (96 KB; these products stream large weight matrices from HBM once).
-        // 65 to 128 rows (the LSTM recurrences): 4 stages, 64 KB, so that two blocks share a CU -- of one launch,
-        // or of the forward recurrence of one minibatch and the backward recurrence of another running on
-        // different streams; with 8 stages (128 KB) a second block only found room between launches.
+        // up to 64 rows: one block row, 8 ring stages (96 KB; these products stream large weight matrices from HBM
+        // once).  65 to 128 rows (the LSTM recurrences): two block rows of 64 and 4 stages (48 KB).  For the same
+        // number of blocks that halves the k split, and with it the partial results written here and read back by
+        // the consumer (16 -> 8 MB per LSTM time step); three such blocks fit a CU, of one launch or of the
+        // recurrences of two minibatches running on different streams.
         if (M <= 64) {
             if (trans_b) pd_gemm_skinny_kernel<1, true, 8><<<grid, GEMM_THREADS, 0, s>>>(g);
             else pd_gemm_skinny_kernel<1, false, 8><<<grid, GEMM_THREADS, 0, s>>>(g);
         } else {
-            if (trans_b) pd_gemm_skinny_kernel<2, true, 4><<<grid, GEMM_THREADS, 0, s>>>(g);
-            else pd_gemm_skinny_kernel<2, false, 4><<<grid, GEMM_THREADS, 0, s>>>(g);
+            const dim3 grid2((N + SK_COLS - 1) / SK_COLS, 2, splits);
+            if (trans_b) pd_gemm_skinny_kernel<1, true, 4><<<grid2, GEMM_THREADS, 0, s>>>(g);
+            else pd_gemm_skinny_kernel<1, false, 4><<<grid2, GEMM_THREADS, 0, s>>>(g);
         }
         PD_CHECK_LAUNCH("pd_gemm_splitk_f32");
         return PD_OK;

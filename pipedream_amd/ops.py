@@ -82,6 +82,21 @@ def gemm(a, b, trans_a=False, trans_b=False, bias=None, relu=False, out=None, be
     ldb = b.stride(0) if b.size(0) > 1 else b.size(1)
     ldc = out.stride(0) if out.size(0) > 1 else out.size(1)
     splits = splitk_factor(M, N, K, trans_a)
+    tail = _tail_rows(M, N, K) if splits == 1 and _TAIL_SPLIT else None
+    if tail is not None and N % 4 == 0 and ldc % 4 == 0 and out.data_ptr() % 16 == 0:
+        # whole rounds of 768 blocks on the upper rows, then the few tile rows left over as a k-split of their own
+        rows, tail_splits = tail
+        lib = _cabi.lib()
+        a_top, a_tail = (a[:, :rows], a[:, rows:]) if trans_a else (a[:rows], a[rows:])
+        with _timed("gemm_f32", 2.0 * M * N * K):
+            lib.pd_gemm_f32(int(trans_a), int(trans_b), rows, N, K, _ptr(a_top), lda, _ptr(b), ldb, float(beta),
+                            _ptr(out), ldc, _ptr(bias), int(relu), _cabi.stream_ptr())
+            part = torch.empty((tail_splits, M - rows, N), dtype=torch.float32, device=a.device)
+            lib.pd_gemm_splitk_f32(int(trans_a), int(trans_b), M - rows, N, K, _ptr(a_tail), lda, _ptr(b), ldb,
+                                   _ptr(part), tail_splits, _cabi.stream_ptr())
+            lib.pd_splitk_reduce_f32(_ptr(part), tail_splits, M - rows, N, _ptr(bias), int(relu), float(beta),
+                                     _ptr(out[rows:]), ldc, _cabi.stream_ptr())
+        return out
     # M <= 128: the streaming kernel behind pd_gemm_splitk_f32 also wins without a split (one partial)
     skinny = not trans_a and M <= 128 and K % 16 == 0 and K >= 256 and N >= 128
     if (splits > 1 or skinny) and N % 4 == 0 and ldc % 4 == 0 and out.data_ptr() % 16 == 0:
@@ -108,11 +123,11 @@ SPLITK_DEEP_K = 1024           # ... worth filling by a split only if every part
 def splitk_factor(M, N, K, trans_a=False):
     """Number of k ranges a product is split into so that about one block per CU runs (1 = no split).
     Mirrors the tile choice of pd_gemm_splitk_f32: its streaming kernel for M <= 128 (A not transposed,
-    K a multiple of 16) owns all rows x 128 columns per block; otherwise tiles are 128 x 128 when M > 64
+    K a multiple of 16) owns up to 64 rows x 128 columns per block; otherwise tiles are 128 x 128 when M > 64
     and N >= 128, else 64 x 64."""
     t_general = 0
     if not trans_a and M <= 128 and K % 16 == 0:
-        tiles = -(-N // 128)
+        tiles = -(-N // 128) * -(-M // 64)
     else:
         t = t_general = 128 if (M > 64 and N >= 128) else 64
         tiles = -(-M // t) * -(-N // t)
@@ -126,6 +141,30 @@ def splitk_factor(M, N, K, trans_a=False):
                 return splits
         return 1
     return max(1, min(SPLITK_TARGET_BLOCKS // tiles, K // SPLITK_MIN_K, 64))
+
+
+_TAIL_SPLIT = True
+
+
+def _tail_rows(M, N, K):
+    """Products of more than one full house of 128 x 128 tiles: (rows, splits) such that the tiles of the first
+    ``rows`` rows fill whole rounds of SPLITK_FULL_HOUSE blocks and the tile rows below them, split ``splits``
+    ways over k, fill most of one more round -- or None where that does not apply.  Without it the blocks left
+    over after the last whole round (64 of 1600 for 6400 x 4096) run as a round of their own that lasts as long
+    as a full one: blocks start and finish in step, and a block with a CU to itself is no faster."""
+    tm, tn = -(-M // 128), -(-N // 128)
+    tiles = tm * tn
+    whole = tiles // SPLITK_FULL_HOUSE
+    if whole < 1 or tiles == whole * SPLITK_FULL_HOUSE:
+        return None
+    top = min(tm - 1, (whole * SPLITK_FULL_HOUSE) // tn)
+    tail_tiles = (tm - top) * tn
+    if top < 1 or tail_tiles > SPLITK_FULL_HOUSE // 2:
+        return None
+    splits = min(SPLITK_FULL_HOUSE // tail_tiles, K // SPLITK_MIN_K)
+    if splits < 2:
+        return None
+    return top * 128, splits
 
 
 def gemm_splitk(a, b, trans_a, trans_b, partials):

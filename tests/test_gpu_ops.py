@@ -270,3 +270,35 @@ def test_gemm_many_tiles_and_deep_split(ta, tb):
         torch.testing.assert_close(got.double(), want, rtol=1e-5, atol=1e-5 * (K ** 0.5))
     assert ops.splitk_factor(2048, 2048, 4096) == 3 and ops.splitk_factor(4096, 1024, 6400, True) == 3
     assert ops.splitk_factor(6400, 4096, 1024) == 1 and ops.splitk_factor(6400, 1024, 4096) == 1
+
+
+@pytest.mark.parametrize("ta,tb", [(False, True), (False, False), (True, False), (True, True)])
+def test_gemm_tile_rows_left_over_after_whole_rounds_are_split_over_k(ta, tb):
+    """6400 x 4096: 1600 tiles = two rounds of 768 blocks + 64; the two tile rows left over run as a k-split of their
+    own.  Bias, ReLU and beta reach both parts; the result equals the one-launch product up to the summation
+    order, and torch's fp64 product to 1e-6."""
+    from pipedream_amd import ops
+    assert ops._tail_rows(6400, 4096, 1024) == (6144, 8) and ops._tail_rows(6400, 4096, 256) == (6144, 2)
+    assert ops._tail_rows(4096, 6400, 1024) == (3840, 7)
+    assert ops._tail_rows(6144, 4096, 1024) is None and ops._tail_rows(2048, 2048, 4096) is None
+    assert ops._tail_rows(8192, 4096, 1024) is None        # 512 tiles left over: most of a round anyway
+    g = torch.Generator().manual_seed(11)
+    M, N, K = 6400, 4096, 512
+    a = torch.randn((K, M) if ta else (M, K), generator=g).cuda()
+    b = torch.randn((N, K) if tb else (K, N), generator=g).cuda()
+    bias = torch.randn(N, generator=g).cuda()
+    prior = torch.randn(M, N, generator=g).cuda()
+    want = torch.relu((a.double().t() if ta else a.double()) @ (b.double().t() if tb else b.double()) + bias.double()
+                      + 0.5 * prior.double())
+    outs = []
+    for split in (True, False):
+        ops._TAIL_SPLIT = split
+        try:
+            outs.append(ops.gemm(a, b, trans_a=ta, trans_b=tb, bias=bias, relu=True, out=prior.clone(), beta=0.5))
+        finally:
+            ops._TAIL_SPLIT = True
+    for got in outs:
+        assert float((got.double() - want).norm() / want.norm()) < 1e-6
+    assert torch.equal(outs[0][:6144], outs[1][:6144])
+    torch.testing.assert_close(outs[0][6144:], outs[1][6144:], rtol=1e-5, atol=1e-4)
+    assert not torch.equal(outs[0][6144:], outs[1][6144:])    # the tail did take the other path
