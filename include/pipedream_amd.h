@@ -315,6 +315,18 @@ int pd_lstm_cell_fwd_f32(float* gates, const float* rec, int n_rec, const float*
 int pd_lstm_cell_bwd_f32(const float* gates, const float* c_prev, const float* c, const float* dy,
                          const float* dh_rec, int n_rec, float* dc_io, float* dgates, int B, int H,
                          int first_step, void* stream);
+/* The time loop of one torch.nn.LSTM layer (stage0.py:14-19; batch_first=False, zero initial state) over the
+ * two calls above, issued from native code: a layer of T = 50 steps is 99 launches and one call.
+ * Forward: gates[T][B][4H] holds x_t W_ih^T on entry and the activated gates on exit; c[T][B][H] and
+ * y[T][B][H] (= h_t) are written; rec[splits][B][4H] is scratch for the k-split products h_{t-1} W_hh^T
+ * (w_hh[4H][H]; may be NULL when T == 1).  Backward: dy[T][B][H] is dL/dy; dgates[T][B][4H] is written;
+ * dh_rec[splits][B][H] and dc[B][H] are scratch.  The weight and input gradients are plain products of dgates
+ * (pd_gemm_f32).  All pointers 16-byte aligned. */
+int pd_lstm_recurrence_fwd_f32(float* gates, const float* w_hh, const float* b_ih, const float* b_hh, float* rec,
+                               int splits, float* c, float* y, int T, int B, int H, void* stream);
+int pd_lstm_recurrence_bwd_f32(const float* gates, const float* c, const float* dy, const float* w_hh,
+                               float* dh_rec, int splits, float* dc, float* dgates, int T, int B, int H,
+                               void* stream);
 /* y = a + b: the residual connections `out13 = out13 + out10` (stage0.py:32, 36). */
 int pd_add_f32(const float* a, const float* b, float* y, uint64_t n, void* stream);
 /* torch.nn.Embedding (stage0.py:10): out[p][:] = weight[ids[p]][:].  Backward writes the

@@ -97,6 +97,8 @@ SIGNATURES = {
     "pd_conv3x3_wgrad_noalloc_nhwc_f32": (_i, [_vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _vp], True),
     "pd_lstm_cell_fwd_f32": (_i, [_vp, _vp, _i, _vp, _vp, _vp, _vp, _vp, _i, _i, _vp], True),
     "pd_lstm_cell_bwd_f32": (_i, [_vp, _vp, _vp, _vp, _vp, _i, _vp, _vp, _i, _i, _i, _vp], True),
+    "pd_lstm_recurrence_fwd_f32": (_i, [_vp, _vp, _vp, _vp, _vp, _i, _vp, _vp, _i, _i, _i, _vp], True),
+    "pd_lstm_recurrence_bwd_f32": (_i, [_vp, _vp, _vp, _vp, _vp, _i, _vp, _vp, _i, _i, _i, _vp], True),
     "pd_add_f32": (_i, [_vp, _vp, _vp, _u64, _vp], True),
     "pd_embedding_fwd_f32": (_i, [_vp, _vp, _vp, _i, _i, _i64, _vp], True),
     "pd_embedding_bwd_f32": (_i, [_vp, _vp, _vp, _i, _i, _i64, _i64, _vp], True),

@@ -273,6 +273,48 @@ extern "C" int pd_lstm_cell_bwd_f32(const float* gates, const float* c_prev, con
     return PD_OK;
 }
 
+// The time loop of one layer, issued from native code: per step one k-split product (none at the first step)
+// and one cell launch, all on `stream`.  Shapes and pointers are checked once, by the first step's calls.
+extern "C" int pd_lstm_recurrence_fwd_f32(float* gates, const float* w_hh, const float* b_ih, const float* b_hh,
+                                          float* rec, int splits, float* c, float* y, int T, int B, int H,
+                                          void* stream) {
+    PD_REQUIRE(T > 0 && B > 0 && H > 0 && H % 4 == 0 && splits >= 1, PD_ESHAPE,
+               "pd_lstm_recurrence_fwd_f32: need T, B > 0, H a positive multiple of 4 and splits >= 1");
+    PD_REQUIRE(gates && w_hh && c && y && (T == 1 || rec), PD_EINVAL, "pd_lstm_recurrence_fwd_f32: NULL pointer");
+    const size_t bh = (size_t)B * H;
+    for (int t = 0; t < T; ++t) {
+        if (t > 0) {
+            const int rc = pd_gemm_splitk_f32(0, 1, B, 4 * H, H, y + (t - 1) * bh, H, w_hh, H, rec, splits, stream);
+            if (rc != PD_OK) return rc;
+        }
+        const int rc = pd_lstm_cell_fwd_f32(gates + t * 4 * bh, rec, t > 0 ? splits : 0, b_ih, b_hh,
+                                            t > 0 ? c + (t - 1) * bh : nullptr, c + t * bh, y + t * bh, B, H, stream);
+        if (rc != PD_OK) return rc;
+    }
+    return PD_OK;
+}
+
+extern "C" int pd_lstm_recurrence_bwd_f32(const float* gates, const float* c, const float* dy, const float* w_hh,
+                                          float* dh_rec, int splits, float* dc, float* dgates, int T, int B, int H,
+                                          void* stream) {
+    PD_REQUIRE(T > 0 && B > 0 && H > 0 && H % 4 == 0 && splits >= 1, PD_ESHAPE,
+               "pd_lstm_recurrence_bwd_f32: need T, B > 0, H a positive multiple of 4 and splits >= 1");
+    PD_REQUIRE(gates && c && dy && w_hh && dc && dgates && (T == 1 || dh_rec), PD_EINVAL,
+               "pd_lstm_recurrence_bwd_f32: NULL pointer");
+    const size_t bh = (size_t)B * H;
+    for (int t = T - 1; t >= 0; --t) {
+        int rc = pd_lstm_cell_bwd_f32(gates + t * 4 * bh, t > 0 ? c + (t - 1) * bh : nullptr, c + t * bh, dy + t * bh,
+                                      t < T - 1 ? dh_rec : nullptr, splits, dc, dgates + t * 4 * bh, B, H,
+                                      t == T - 1, stream);
+        if (rc != PD_OK) return rc;
+        if (t > 0) {      // dh_{t-1} += dgates_t W_hh: [B][4H] x [4H][H], split over 4H
+            rc = pd_gemm_splitk_f32(0, 0, B, H, 4 * H, dgates + t * 4 * bh, 4 * H, w_hh, H, dh_rec, splits, stream);
+            if (rc != PD_OK) return rc;
+        }
+    }
+    return PD_OK;
+}
+
 extern "C" int pd_add_f32(const float* a, const float* b, float* y, uint64_t n, void* stream) {
     if (n == 0) return PD_OK;
     PD_REQUIRE(a && b && y, PD_EINVAL, "pd_add_f32: NULL pointer");

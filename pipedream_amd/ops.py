@@ -698,7 +698,12 @@ def lstm_forward(x, w_ih, w_hh, b_ih, b_hh):
     c = torch.empty((T, B, H), dtype=torch.float32, device=x.device)
     # the recurrent product h_{t-1} W_hh^T has only B rows: split over k, summed inside the cell kernel
     rec = torch.empty((splitk_factor(B, 4 * H, H), B, 4 * H), dtype=torch.float32, device=x.device)
-    for t in range(T):
+    if kernel_timer is None and w_hh.is_contiguous():
+        # the time loop in native code: one call instead of 2 T - 1
+        lib.pd_lstm_recurrence_fwd_f32(_ptr(gates), _ptr(w_hh), _ptr(b_ih), _ptr(b_hh), _ptr(rec), rec.size(0),
+                                       _ptr(c), _ptr(y), T, B, H, s())
+        return y, (gates, c)
+    for t in range(T):      # the same loop with an event pair around every product (per-kernel timing)
         if t > 0:
             gemm_splitk(y[t - 1], w_hh, False, True, rec)
         lib.pd_lstm_cell_fwd_f32(_ptr(gates[t]), _ptr(rec), rec.size(0) if t > 0 else 0, _ptr(b_ih), _ptr(b_hh),
@@ -715,7 +720,11 @@ def lstm_backward(dy, x, y, gates, c, w_ih, w_hh, need_dx=True):
     dgates = torch.empty((T, B, 4 * H), dtype=torch.float32, device=x.device)
     dc = torch.empty((B, H), dtype=torch.float32, device=x.device)
     dh_rec = torch.empty((splitk_factor(B, H, 4 * H), B, H), dtype=torch.float32, device=x.device)
-    for t in range(T - 1, -1, -1):
+    native = kernel_timer is None and w_hh.is_contiguous() and gates.is_contiguous() and c.is_contiguous()
+    if native:
+        lib.pd_lstm_recurrence_bwd_f32(_ptr(gates), _ptr(c), _ptr(dy), _ptr(w_hh), _ptr(dh_rec), dh_rec.size(0),
+                                       _ptr(dc), _ptr(dgates), T, B, H, s())
+    for t in (() if native else range(T - 1, -1, -1)):
         lib.pd_lstm_cell_bwd_f32(_ptr(gates[t]), _ptr(c[t - 1]) if t > 0 else None, _ptr(c[t]), _ptr(dy[t]),
                                  _ptr(dh_rec) if t < T - 1 else None, dh_rec.size(0), _ptr(dc), _ptr(dgates[t]), B, H,
                                  int(t == T - 1), s())

@@ -40,6 +40,42 @@ def test_lstm_layer_matches_torch():
         torch.testing.assert_close(p.grad.cpu(), q.grad, rtol=1e-5, atol=2e-6, msg=k)
 
 
+@pytest.mark.parametrize("T,B,I,H", [(7, 5, 24, 32), (1, 3, 16, 16), (12, 128, 256, 256), (6, 100, 128, 1024)])
+def test_lstm_time_loop_in_native_code_equals_the_step_by_step_calls(T, B, I, H):
+    """ops.lstm_forward / lstm_backward issue a layer's time loop through pd_lstm_recurrence_fwd/bwd_f32; with the
+    per-launch timer on they call the product and the cell once per step instead.  Same kernels on the same
+    operands: every result bit for bit.  (100 and 128 rows: the recurrence product's two block rows of 64.)"""
+    from pipedream_amd import ops
+    g = torch.Generator().manual_seed(5)
+    x = torch.randn(T, B, I, generator=g).cuda()
+    w_ih = (torch.randn(4 * H, I, generator=g) * 0.1).cuda()
+    w_hh = (torch.randn(4 * H, H, generator=g) * 0.1).cuda()
+    b_ih, b_hh = torch.randn(4 * H, generator=g).cuda(), torch.randn(4 * H, generator=g).cuda()
+    dy = torch.randn(T, B, H, generator=g).cuda()
+
+    def run():
+        y, (gates, c) = ops.lstm_forward(x, w_ih, w_hh, b_ih, b_hh)
+        return (y, gates, c) + tuple(ops.lstm_backward(dy, x, y, gates, c, w_ih, w_hh))
+    native = run()
+    ops.kernel_timer = {}
+    try:
+        stepwise = run()
+        assert (T == 1) == ("gemm_f32_splitk" not in ops.kernel_timer)     # the other path did run
+    finally:
+        ops.kernel_timer = None
+    for a, b in zip(native, stepwise):
+        assert torch.equal(a, b)
+    ref = torch.nn.LSTM(I, H).cuda()
+    with torch.no_grad():
+        for p, v in zip(ref.parameters(), (w_ih, w_hh, b_ih, b_hh)):
+            p.copy_(v)
+    xr = x.clone().requires_grad_(True)
+    yr = ref(xr)[0]
+    yr.backward(dy)
+    torch.testing.assert_close(native[0], yr.detach(), rtol=1e-4, atol=1e-5)
+    torch.testing.assert_close(native[3], xr.grad, rtol=1e-4, atol=1e-4)
+
+
 def test_embedding_matches_torch_including_duplicates_and_padding():
     from pipedream_amd import layers
     torch.manual_seed(1)
