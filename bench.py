@@ -269,6 +269,8 @@ def _run_steps(step, steps, warmup, before_instrumented=None):
     elapsed = time.perf_counter() - t0
     if before_instrumented is not None:
         before_instrumented()
+        step()                      # one step to settle on the new stream arrangement, outside the event pairs
+        torch.cuda.synchronize()
     ops.kernel_timer = {}
     for _ in range(min(steps, 4)):
         step()
