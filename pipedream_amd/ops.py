@@ -82,20 +82,23 @@ def gemm(a, b, trans_a=False, trans_b=False, bias=None, relu=False, out=None, be
     ldb = b.stride(0) if b.size(0) > 1 else b.size(1)
     ldc = out.stride(0) if out.size(0) > 1 else out.size(1)
     splits = splitk_factor(M, N, K, trans_a)
-    tail = _tail_rows(M, N, K) if splits == 1 and _TAIL_SPLIT else None
-    if tail is not None and N % 4 == 0 and ldc % 4 == 0 and out.data_ptr() % 16 == 0:
+    plan = _row_plan(M, N, K) if splits == 1 and _ROW_PLAN else None
+    if plan is not None and N % 4 == 0 and ldc % 4 == 0 and out.data_ptr() % 16 == 0:
         # whole rounds of 768 blocks on the upper rows, then the few tile rows left over as a k-split of their own
-        rows, tail_splits = tail
+        rows, top_splits, tail_splits = plan
         lib = _cabi.lib()
-        a_top, a_tail = (a[:, :rows], a[:, rows:]) if trans_a else (a[:rows], a[rows:])
         with _timed("gemm_f32", 2.0 * M * N * K):
-            lib.pd_gemm_f32(int(trans_a), int(trans_b), rows, N, K, _ptr(a_top), lda, _ptr(b), ldb, float(beta),
-                            _ptr(out), ldc, _ptr(bias), int(relu), _cabi.stream_ptr())
-            part = torch.empty((tail_splits, M - rows, N), dtype=torch.float32, device=a.device)
-            lib.pd_gemm_splitk_f32(int(trans_a), int(trans_b), M - rows, N, K, _ptr(a_tail), lda, _ptr(b), ldb,
-                                   _ptr(part), tail_splits, _cabi.stream_ptr())
-            lib.pd_splitk_reduce_f32(_ptr(part), tail_splits, M - rows, N, _ptr(bias), int(relu), float(beta),
-                                     _ptr(out[rows:]), ldc, _cabi.stream_ptr())
+            for r0, r1, sp in ((0, rows, top_splits), (rows, M, tail_splits)):
+                a_part = a[:, r0:r1] if trans_a else a[r0:r1]
+                if sp == 1:
+                    lib.pd_gemm_f32(int(trans_a), int(trans_b), r1 - r0, N, K, _ptr(a_part), lda, _ptr(b), ldb,
+                                    float(beta), _ptr(out[r0:]), ldc, _ptr(bias), int(relu), _cabi.stream_ptr())
+                    continue
+                part = torch.empty((sp, r1 - r0, N), dtype=torch.float32, device=a.device)
+                lib.pd_gemm_splitk_f32(int(trans_a), int(trans_b), r1 - r0, N, K, _ptr(a_part), lda, _ptr(b), ldb,
+                                       _ptr(part), sp, _cabi.stream_ptr())
+                lib.pd_splitk_reduce_f32(_ptr(part), sp, r1 - r0, N, _ptr(bias), int(relu), float(beta),
+                                         _ptr(out[r0:]), ldc, _cabi.stream_ptr())
         return out
     # M <= 128: the streaming kernel behind pd_gemm_splitk_f32 also wins without a split (one partial)
     skinny = not trans_a and M <= 128 and K % 16 == 0 and K >= 256 and N >= 128
@@ -143,28 +146,54 @@ def splitk_factor(M, N, K, trans_a=False):
     return max(1, min(SPLITK_TARGET_BLOCKS // tiles, K // SPLITK_MIN_K, 64))
 
 
-_TAIL_SPLIT = True
+_ROW_PLAN = True
 
 
-def _tail_rows(M, N, K):
-    """Products of more than one full house of 128 x 128 tiles: (rows, splits) such that the tiles of the first
-    ``rows`` rows fill whole rounds of SPLITK_FULL_HOUSE blocks and the tile rows below them, split ``splits``
-    ways over k, fill most of one more round -- or None where that does not apply.  Without it the blocks left
-    over after the last whole round (64 of 1600 for 6400 x 4096) run as a round of their own that lasts as long
-    as a full one: blocks start and finish in step, and a block with a CU to itself is no faster."""
+def _house_time(blocks, k):
+    """Time, in steps of k of a full round, that ``blocks`` blocks of the 128 x 128 kernel take to reduce over ``k``
+    each: whole rounds of SPLITK_FULL_HOUSE blocks, plus a last round that costs 0.45 + 0.55 x its fill (blocks
+    with fewer neighbours on their CU run faster, but not in proportion: measured 0.75 for 400 of 768)."""
+    whole, rem = divmod(blocks, SPLITK_FULL_HOUSE)
+    return k * (whole + (0.45 + 0.55 * rem / SPLITK_FULL_HOUSE if rem else 0.0))
+
+
+def _reduce_time(rows, n, splits):
+    """pd_splitk_reduce_f32 in the same unit (one step of k of a full round is about 0.18 us): a launch and
+    (splits + 1) x rows x n x 4 bytes at about 4 TB/s."""
+    return 30 + rows * n * 4 * (splits + 1) / 4e6 / 0.18
+
+
+def _row_plan(M, N, K):
+    """(rows, top_splits, tail_splits) or None.  A product of more than half a full house of 128 x 128 tiles can
+    leave a last round nearly empty (64 of 1600 tiles for 6400 x 4096, 400 tiles on 768 places for 6400 x 1024):
+    that round lasts almost as long as a full one.  The plan gives the first ``rows`` rows whole rounds -- as they
+    are, or split two or three ways over a reduction that is deep enough -- and runs the tile rows left over as a
+    k-split of their own that fills one more round.  Chosen by the cost model above; None where the plain launch
+    is within 7 % of the best plan."""
     tm, tn = -(-M // 128), -(-N // 128)
     tiles = tm * tn
-    whole = tiles // SPLITK_FULL_HOUSE
-    if whole < 1 or tiles == whole * SPLITK_FULL_HOUSE:
+    if tiles <= SPLITK_FULL_HOUSE // 2:
         return None
-    top = min(tm - 1, (whole * SPLITK_FULL_HOUSE) // tn)
-    tail_tiles = (tm - top) * tn
-    if top < 1 or tail_tiles > SPLITK_FULL_HOUSE // 2:
-        return None
-    splits = min(SPLITK_FULL_HOUSE // tail_tiles, K // SPLITK_MIN_K)
-    if splits < 2:
-        return None
-    return top * 128, splits
+    best, best_cost = None, 0.93 * _house_time(tiles, K)
+    for top_splits in (1, 2, 3):
+        if top_splits > 1 and K // top_splits < SPLITK_DEEP_K:
+            break
+        per_row = tn * top_splits
+        rounds = (tm * per_row) // SPLITK_FULL_HOUSE
+        top = min(tm - 1, (rounds * SPLITK_FULL_HOUSE) // per_row)
+        if rounds < 1 or top < 1:
+            continue
+        tail_tiles = (tm - top) * tn
+        tail_splits = max(1, min(SPLITK_FULL_HOUSE // tail_tiles, K // SPLITK_MIN_K))
+        k_top = -(-K // top_splits)
+        cost = _house_time(top * per_row, k_top) + _house_time(tail_tiles * tail_splits, -(-K // tail_splits)) + 30
+        if top_splits > 1:
+            cost += _reduce_time(top * 128, N, top_splits)
+        if tail_splits > 1:
+            cost += _reduce_time(M - top * 128, N, tail_splits)
+        if cost < best_cost:
+            best, best_cost = (top * 128, top_splits, tail_splits), cost
+    return best
 
 
 def gemm_splitk(a, b, trans_a, trans_b, partials):

@@ -273,17 +273,18 @@ def test_gemm_many_tiles_and_deep_split(ta, tb):
 
 
 @pytest.mark.parametrize("ta,tb", [(False, True), (False, False), (True, False), (True, True)])
-def test_gemm_tile_rows_left_over_after_whole_rounds_are_split_over_k(ta, tb):
+@pytest.mark.parametrize("M,N,K,plan", [(6400, 4096, 1024, (6144, 1, 8)), (6400, 1024, 2560, (6144, 2, 20))])
+def test_gemm_tile_rows_left_over_after_whole_rounds_are_split_over_k(ta, tb, M, N, K, plan):
     """6400 x 4096: 1600 tiles = two rounds of 768 blocks + 64; the two tile rows left over run as a k-split of their
-    own.  Bias, ReLU and beta reach both parts; the result equals the one-launch product up to the summation
-    order, and torch's fp64 product to 1e-6."""
+    own.  6400 x 1024 with a deep reduction: 400 tiles; the first 48 tile rows, split two ways, are one round of
+    768 blocks and the two left over a second, small one.  Bias, ReLU and beta reach both parts; the result equals
+    the one-launch product up to the summation order, and torch's fp64 product to 1e-6."""
     from pipedream_amd import ops
-    assert ops._tail_rows(6400, 4096, 1024) == (6144, 8) and ops._tail_rows(6400, 4096, 256) == (6144, 2)
-    assert ops._tail_rows(4096, 6400, 1024) == (3840, 7)
-    assert ops._tail_rows(6144, 4096, 1024) is None and ops._tail_rows(2048, 2048, 4096) is None
-    assert ops._tail_rows(8192, 4096, 1024) is None        # 512 tiles left over: most of a round anyway
+    assert ops._row_plan(M, N, K) == plan
+    assert ops._row_plan(6144, 4096, 1024) is None and ops._row_plan(2048, 2048, 4096) is None
+    assert ops._row_plan(8192, 4096, 1024) is None        # 512 tiles left over: most of a round anyway
+    assert ops._row_plan(6400, 1024, 1024) is None        # too shallow to split the upper rows
     g = torch.Generator().manual_seed(11)
-    M, N, K = 6400, 4096, 512
     a = torch.randn((K, M) if ta else (M, K), generator=g).cuda()
     b = torch.randn((N, K) if tb else (K, N), generator=g).cuda()
     bias = torch.randn(N, generator=g).cuda()
@@ -291,14 +292,16 @@ def test_gemm_tile_rows_left_over_after_whole_rounds_are_split_over_k(ta, tb):
     want = torch.relu((a.double().t() if ta else a.double()) @ (b.double().t() if tb else b.double()) + bias.double()
                       + 0.5 * prior.double())
     outs = []
-    for split in (True, False):
-        ops._TAIL_SPLIT = split
+    for planned in (True, False):
+        ops._ROW_PLAN = planned
         try:
             outs.append(ops.gemm(a, b, trans_a=ta, trans_b=tb, bias=bias, relu=True, out=prior.clone(), beta=0.5))
         finally:
-            ops._TAIL_SPLIT = True
+            ops._ROW_PLAN = True
     for got in outs:
         assert float((got.double() - want).norm() / want.norm()) < 1e-6
-    assert torch.equal(outs[0][:6144], outs[1][:6144])
-    torch.testing.assert_close(outs[0][6144:], outs[1][6144:], rtol=1e-5, atol=1e-4)
-    assert not torch.equal(outs[0][6144:], outs[1][6144:])    # the tail did take the other path
+    rows = plan[0]
+    if plan[1] == 1:
+        assert torch.equal(outs[0][:rows], outs[1][:rows])
+    torch.testing.assert_close(outs[0], outs[1], rtol=1e-5, atol=1e-5 * K ** 0.5)    # sums of K terms of size ~1
+    assert not torch.equal(outs[0][rows:], outs[1][rows:])    # the tail did take the other path
