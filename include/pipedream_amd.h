@@ -231,6 +231,12 @@ int pd_conv3x3_dgrad_nhwc_f32(const float* dy, const float* w_rot, const float* 
  * compute unit; 1: pieces wherever the shape allows; -1: never.  Results are bit-identical either way.
  * Process-wide, not thread-safe against concurrent convolution calls.  No counterpart in the reference. */
 int pd_conv3x3_winograd_set_pieces(int mode);
+/* Tuning and test hook for pd_conv3x3_winograd_wgrad_nhwc_f32.  Its blocks sum over strips of eight 2 x 2 tiles:
+ * 2 x 16 pixels of one image, or, upright, 16 rows x 2 columns of the batch taken as one image of N * H rows
+ * (H, W even, H >= 14), which leaves no padding columns at widths that are no multiple of 16.  mode 0 (default):
+ * upright strips exactly where the width is no multiple of 16; 1: never; 2: wherever the shape allows.  Results
+ * differ by the summation order only.  Process-wide.  No counterpart in the reference. */
+int pd_conv3x3_winograd_set_wgrad_strips(int mode);
 
 /* The same convolution (and, with rot180, its input gradient) by the Winograd algorithm
  * F(2x2, 3x3) in fp32: 2.25x fewer multiplications; results agree with the direct kernels to

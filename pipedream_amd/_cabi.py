@@ -85,6 +85,7 @@ SIGNATURES = {
     "pd_conv3x3_winograd_filter_bytes": (_i, [_i, _i, ctypes.POINTER(_u64)], True),
     "pd_conv3x3_winograd_filter_f32": (_i, [_vp, _vp, _i, _i, _i, _vp], True),
     "pd_conv3x3_winograd_set_pieces": (_i, [_i], True),
+    "pd_conv3x3_winograd_set_wgrad_strips": (_i, [_i], True),
     "pd_conv3x3_winograd_fwd_nhwc_f32": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _vp], True),
     "pd_conv3x3_winograd_fwd_pool_nhwc_f32": (_i, [_vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _vp], True),
     "pd_conv3x3_winograd_fwd_unpool_nhwc_f32": (_i, [_vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _vp], True),

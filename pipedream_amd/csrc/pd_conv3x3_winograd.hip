@@ -962,7 +962,9 @@ constexpr int WW_ROW_PIECES = 320;                   // 16-byte pieces per patch
 constexpr int WW_V_STAGE = WG_G * WW_TILES * 64;     // floats: [g][tile][c]
 constexpr int WW_RAW_STAGE = 4 * WW_PATCH_W * 64;    // floats: [row][pixel][c]
 constexpr int WW_RAW_OFF = 2 * WW_V_STAGE;
-constexpr int WW_LDS_FLOATS = WW_RAW_OFF + 2 * WW_RAW_STAGE;
+constexpr int WW_ZERO_OFF = WW_RAW_OFF + 2 * WW_RAW_STAGE;   // upright strips: one patch row (4 pixels) of zeros
+constexpr int WW_LDS_FLOATS = WW_ZERO_OFF + 4 * 64;
+constexpr int WW_VROWS = 2 * WW_TILES;               // output rows of an upright strip
 constexpr int WW_BLOCKS = 256;                       // persistent blocks: 8 dies x 32
 constexpr int WW_PART_FLOATS = WG_G * 64 * 64;       // one block's partial dU
 constexpr int WW_PART_STRIDE = WW_PART_FLOATS;       // floats between two blocks' partials
@@ -973,12 +975,14 @@ struct WinoWgradArgs {
     float* part;         // [pair][rank][16][64][64]
     float* part_db;      // [pair][rank][2][64]
     int N, H, W, C, K;
-    int sx, sy;          // strips per row pair, row pairs per image
+    int sx, sy;          // strips per row pair, row pairs per image (upright strips: strips side by side, unused)
     int n_strips, strips_per_rank;
+    int rows_all;        // upright strips: N * H, the rows of the batch taken as one tall image
     int c_blocks, n_pairs, ranks;
 };
 
 struct StripPos { int n, y0, x0, row; };      // row = n * H + y0, the strip's first output row counted over all images
+// (upright strips: row = first output row in the stacked batch, y0 = row % H, n unused)
 
 // Strips are numbered down the image first (row pair fastest), then across, then over images: a block's
 // consecutive strips share two of their four input rows, which the second one finds in cache.
@@ -993,6 +997,32 @@ __device__ __forceinline__ StripPos strip_decode(const WinoWgradArgs& a, int s) 
     p.row = p.n * a.H + p.y0;
     return p;
 }
+// Upright strips (8 tiles on top of each other: 16 output rows x 2 columns of the batch taken as one image of
+// N * H rows) are numbered across the image first: neighbours share two of their four patch columns.
+__device__ __forceinline__ StripPos vstrip_decode(const WinoWgradArgs& a, int s) {
+    StripPos p;
+    const int sr = s / a.sx;
+    p.n = 0;
+    p.x0 = 2 * (s - sr * a.sx);
+    p.row = WW_VROWS * sr;
+    p.y0 = p.row % a.H;
+    return p;
+}
+// (y0 is kept only for the cursor that needs it; H >= 14, so two subtractions at most)
+template <bool WITH_Y0 = false>
+__device__ __forceinline__ void vstrip_next(const WinoWgradArgs& a, StripPos& p) {
+    p.x0 += 2;
+    if (p.x0 >= a.W) {
+        p.x0 = 0;
+        p.row += WW_VROWS;
+        if (WITH_Y0) {
+            p.y0 += WW_VROWS;
+            if (p.y0 >= a.H) p.y0 -= a.H;
+            if (p.y0 >= a.H) p.y0 -= a.H;
+        }
+    }
+}
+
 __device__ __forceinline__ void strip_next(const WinoWgradArgs& a, StripPos& p) {
     p.y0 += 2;
     p.row += 2;
@@ -1004,6 +1034,14 @@ __device__ __forceinline__ void strip_next(const WinoWgradArgs& a, StripPos& p) 
     }
 }
 
+// VERT: upright strips.  A strip of 2 x 16 pixels pads image widths of 56, 28 and 14 pixels to 64, 32 and 16; eight
+// tiles on top of each other fit every even width, and with the batch taken as one image of N * H rows (H even, so
+// no tile straddles two images) only the batch's last strip row can be partly empty.  The patch is then 18 rows x 4
+// pixels (as many pixels as 4 x 18).  A tile in the first (last) tile row of an image must see zeros in the first
+// (last) row of its 4 x 4 window, where the stacked layout holds the neighbouring image's row: only the threads
+// that form row 0 (d0 - d2) resp. row 3 (d1 - d3) of B^T d read those rows, and for such a tile they read a row of
+// zeros in LDS instead.  Needs H >= 14 (one conditional subtraction finds a tile's row inside its image).
+template <bool VERT>
 __global__ __launch_bounds__(WW_THREADS, 1) void winograd_wgrad_kernel(const WinoWgradArgs a) {
     __shared__ __attribute__((aligned(16))) float lds[WW_LDS_FLOATS];
 
@@ -1038,6 +1076,14 @@ __global__ __launch_bounds__(WW_THREADS, 1) void winograd_wgrad_kernel(const Win
 #pragma unroll
     for (int j = 0; j < 3; ++j) {
         const int p = tid + WW_THREADS * j;
+        if (VERT) {      // a wave = one patch row: 4 pixels x 16 channel groups, one contiguous kilobyte
+            prow[j] = wave + 8 * j;
+            const int ppx = lane >> 4, pcg = lane & 15;
+            live[j] = prow[j] < WW_VROWS + 2;
+            xoff[j] = live[j] ? (uint32_t)(((ppx - 1) * a.C + pcg * 4) * 4) : 0x80000000u;
+            raw_dst[j] = ((live[j] ? prow[j] : 0) * 4 + ppx) * 64 + pcg * 4;
+            continue;
+        }
         prow[j] = __builtin_amdgcn_readfirstlane(p / WW_ROW_PIECES);
         const int rem = p % WW_ROW_PIECES, ppx = rem >> 4, pcg = rem & 15;
         live[j] = ppx < WW_PATCH_W && p < 4 * WW_ROW_PIECES;
@@ -1053,16 +1099,17 @@ __global__ __launch_bounds__(WW_THREADS, 1) void winograd_wgrad_kernel(const Win
     const char* xrow0[3];
 #pragma unroll
     for (int j = 0; j < 3; ++j) xrow0[j] = (const char*)(a.x + cb * 64) + (int64_t)(prow[j] - 1) * row_pitch_x;
-    const bool third_row_live = wave < 4;      // the third round of pieces covers the patch's last row only
+    const bool third_row_live = VERT ? wave < 2 : wave < 4;   // the third round of pieces: the patch's last row(s) only
     auto load_raw = [&](const StripPos& p, bool valid) {
         const uint32_t strip_off = (uint32_t)(p.x0 * a.C) * 4;
         const uint32_t live_bytes = valid ? row_bytes_x : 0u;
         const uint64_t strip_row = (uint64_t)(uint32_t)p.row * row_pitch_x;
 #pragma unroll
         for (int j = 0; j < 3; ++j) {
-            const uint32_t gy = (uint32_t)(p.y0 - 1 + prow[j]);
+            // (upright strips: p.row counts rows of the whole batch, and a row of the neighbouring image is data)
+            const uint32_t gy = (uint32_t)((VERT ? p.row : p.y0) - 1 + prow[j]);
             const uint32_t row_bytes = (j < 2 || third_row_live) ? live_bytes : 0u;
-            const uint32_t bytes = gy < (uint32_t)a.H ? row_bytes : 0u;
+            const uint32_t bytes = gy < (uint32_t)(VERT ? a.rows_all : a.H) ? row_bytes : 0u;
             const __amdgpu_buffer_rsrc_t r =
                 __builtin_amdgcn_make_buffer_rsrc((void*)(xrow0[j] + strip_row), 0, bytes, 0x00020000);
             rawr[j] = __builtin_bit_cast(float4_t, __builtin_amdgcn_raw_buffer_load_b128(r, xoff[j] + strip_off, 0, 0));
@@ -1078,12 +1125,34 @@ __global__ __launch_bounds__(WW_THREADS, 1) void winograd_wgrad_kernel(const Win
     const int row_a = ti == 0 ? 0 : ti == 2 ? 2 : 1;
     const int row_b = ti == 2 ? 1 : ti == 3 ? 3 : 2;
     const float sgn = ti == 1 ? 1.f : -1.f;
-    const int src_a = (row_a * WW_PATCH_W + 2 * tt) * 64 + cg * 4, src_b = (row_b * WW_PATCH_W + 2 * tt) * 64 + cg * 4;
+    const int src_a = VERT ? ((2 * tt + row_a) * 4) * 64 + cg * 4 : (row_a * WW_PATCH_W + 2 * tt) * 64 + cg * 4;
+    const int src_b = VERT ? ((2 * tt + row_b) * 4) * 64 + cg * 4 : (row_b * WW_PATCH_W + 2 * tt) * 64 + cg * 4;
+    // upright strips: where this thread reads rows Ra / Rb of the strip being transformed -- src_a / src_b, or the
+    // row of zeros when the tile's window row lies in the neighbouring image (ti = 0: row 0, ti = 3: row 3)
+    // (offsets from the start of LDS, raw stage included)
+    int sa = 0, sb = 0;
+    auto set_window_rows = [&](const StripPos& p, int stage) {
+        if (!VERT) return;
+        const int base = WW_RAW_OFF + stage * WW_RAW_STAGE;
+        sa = base + src_a;
+        sb = base + src_b;
+        if (ti == 0 || ti == 3) {
+            int t = p.y0 + 2 * tt;              // the tile's first output row inside its image (y0 < H, 2 tt <= 14 <= H)
+            t = t >= a.H ? t - a.H : t;
+            if (ti == 0 && t == 0) sa = WW_ZERO_OFF + cg * 4;
+            if (ti == 3 && t + 2 == a.H) sb = WW_ZERO_OFF + cg * 4;
+        }
+    };
     const int v_dst = (ti * 4 * WW_TILES + tt) * 64 + ((cg * 4) ^ (32 * (tt & 1)));
     float4_t t[4], dc[2], vout;
     auto read_col = [&](const float* rs, int s) {
-        dc[0] = *(const float4_t*)(rs + src_a + s * 64);
-        dc[1] = *(const float4_t*)(rs + src_b + s * 64);
+        if (VERT) {
+            dc[0] = *(const float4_t*)(lds + sa + s * 64);
+            dc[1] = *(const float4_t*)(lds + sb + s * 64);
+        } else {
+            dc[0] = *(const float4_t*)(rs + src_a + s * 64);
+            dc[1] = *(const float4_t*)(rs + src_b + s * 64);
+        }
     };
     auto transform_col = [&](int s) { t[s] = dc[0] + sgn * dc[1]; };
     auto transform_out = [&](int m) {
@@ -1105,16 +1174,27 @@ __global__ __launch_bounds__(WW_THREADS, 1) void winograd_wgrad_kernel(const Win
 #pragma unroll
     for (int j = 0; j < 4; ++j)
 #pragma unroll
-        for (int b = 0; b < 2; ++b) dyoff[j][b] = (uint32_t)((4 * j + 2 * h + b) * a.K + kb * 64 + wm * 32 + cl) * 4;
+        for (int b = 0; b < 2; ++b)
+            dyoff[j][b] = VERT ? (uint32_t)(((4 * j + 2 * h) * a.W + b) * a.K + kb * 64 + wm * 32 + cl) * 4
+                               : (uint32_t)((4 * j + 2 * h + b) * a.K + kb * 64 + wm * 32 + cl) * 4;
     float dyr[2][2][4];                        // [row a][column b][j]
     const uint32_t row_pitch_dy = (uint32_t)(a.W * a.K) * 4;
     auto load_dy = [&](const StripPos& p, bool valid) {
-        const uint32_t live_bytes = valid ? (uint32_t)((a.W - p.x0) * a.K) * 4 : 0u;
+        // upright strips: tile 2j + h lies 2 (2j + h) rows further down (in dyoff); one descriptor per row parity,
+        // from the strip's first pixel of that row to the end of the strip's last row inside the batch
+        int vrows = a.rows_all - p.row;
+        vrows = vrows < WW_VROWS ? vrows : WW_VROWS;
+        const uint32_t live_bytes = !valid ? 0u : VERT ? (uint32_t)((vrows * a.W - p.x0) * a.K) * 4
+                                                       : (uint32_t)((a.W - p.x0) * a.K) * 4;
         const char* row0 = (const char*)a.dy + (uint64_t)(uint32_t)(p.row * a.W + p.x0) * (uint32_t)(a.K * 4);
 #pragma unroll
         for (int r = 0; r < 2; ++r) {
             // the strip's first row always lies in the image, its second may not (odd H)
-            const uint32_t bytes = (r == 0 || p.y0 + 1 < a.H) ? live_bytes : 0u;
+            // (readfirstlane: the compiler forms the saturating difference in a vector register, and a descriptor
+            // built from one is taken as different per lane -- a loop around every load)
+            const uint32_t bytes = VERT ? (r == 0 ? live_bytes : (uint32_t)__builtin_amdgcn_readfirstlane((int)(
+                                               live_bytes > row_pitch_dy ? live_bytes - row_pitch_dy : 0u)))
+                                        : (r == 0 || p.y0 + 1 < a.H) ? live_bytes : 0u;
             const __amdgpu_buffer_rsrc_t rs =
                 __builtin_amdgcn_make_buffer_rsrc((void*)(row0 + (r ? row_pitch_dy : 0u)), 0, bytes, 0x00020000);
 #pragma unroll
@@ -1137,10 +1217,12 @@ __global__ __launch_bounds__(WW_THREADS, 1) void winograd_wgrad_kernel(const Win
     if (n_my > 0) {
         // cursors of the stages: strip of the next raw-x request (3 ahead of the multiply), of the next
         // dY request (1 ahead)
-        StripPos lp = strip_decode(a, s_begin), dp = lp;
+        StripPos lp = VERT ? vstrip_decode(a, s_begin) : strip_decode(a, s_begin), dp = lp;
+        StripPos tp = lp;                      // upright strips: the strip whose patch stage 2 reads next
         int l_left = n_my, d_left = n_my;      // strips not yet requested
-        auto next_l = [&]() { --l_left; strip_next(a, lp); };
-        auto next_d = [&]() { --d_left; strip_next(a, dp); };
+        auto next_l = [&]() { --l_left; if (VERT) vstrip_next(a, lp); else strip_next(a, lp); };
+        auto next_d = [&]() { --d_left; if (VERT) vstrip_next(a, dp); else strip_next(a, dp); };
+        if (VERT && tid < 4 * 64) lds[WW_ZERO_OFF + tid] = 0.f;
 
         // ---- prologue: strips 0 and 1 into LDS, strip 2 into registers, strip 0 transformed, dY of strip 0
         load_raw(lp, l_left > 0); next_l();
@@ -1152,10 +1234,12 @@ __global__ __launch_bounds__(WW_THREADS, 1) void winograd_wgrad_kernel(const Win
         for (int j = 0; j < 3; ++j) store_raw(1, j);
         load_raw(lp, l_left > 0); next_l();
         __syncthreads();
+        set_window_rows(tp, 0);
 #pragma unroll
         for (int s = 0; s < 4; ++s) { read_col(lds + WW_RAW_OFF, s); transform_col(s); }
 #pragma unroll
         for (int m = 0; m < 4; ++m) { transform_out(m); store_out(lds, m); }
+        if (VERT) { vstrip_next<true>(a, tp); set_window_rows(tp, 1); }      // strip 1 sits in the second raw stage
         __builtin_amdgcn_s_waitcnt(0);
         __syncthreads();
         float bf[2][2][4];                     // B fragments of GEMM pair p wait in bf[p & 1]: [g of the pair][j]
@@ -1250,6 +1334,8 @@ __global__ __launch_bounds__(WW_THREADS, 1) void winograd_wgrad_kernel(const Win
                     if (gp == 0 && k == 6) read_col(rs, 2);
                     if (gp == 1 && k == 1) transform_col(2);
                     if (gp == 1 && k == 2) read_col(rs, 3);
+                    // (strip q+1's last patch read; the next one, in the last section, is strip q+2's first)
+                    if (VERT && gp == 1 && k == 3) { vstrip_next<true>(a, tp); set_window_rows(tp, q & 1); }
                     if (gp == 1 && k == 4) transform_col(3);
                     if (gp == 2 && (k == 1 || k == 3 || k == 5)) transform_out(k >> 1);
                     if (gp == 2 && (k == 2 || k == 4 || k == 6)) store_out(vn, (k >> 1) - 1);
@@ -1375,6 +1461,13 @@ bool wino_wgrad_shape_ok(int C, int K) {
 
 }  // namespace
 
+static int g_wgrad_strips = 0;
+extern "C" int pd_conv3x3_winograd_set_wgrad_strips(int mode) {
+    PD_REQUIRE(mode >= 0 && mode <= 2, PD_EINVAL, "pd_conv3x3_winograd_set_wgrad_strips: mode is 0, 1 or 2");
+    g_wgrad_strips = mode;
+    return PD_OK;
+}
+
 extern "C" int pd_conv3x3_winograd_wgrad_supported(int C, int K) {
     return (C > 0 && K > 0 && wino_wgrad_shape_ok(C, K)) ? 1 : 0;
 }
@@ -1409,9 +1502,14 @@ extern "C" int pd_conv3x3_winograd_wgrad_nhwc_f32(const float* x, const float* d
     WinoWgradArgs a;
     a.x = x; a.dy = dy;
     a.N = N; a.H = H; a.W = W; a.C = C; a.K = K;
-    a.sx = (W + 2 * WW_TILES - 1) / (2 * WW_TILES);
+    // upright strips where strips of 2 x 16 pixels would pad the width (g_wgrad_strips: 0 = that rule, 1 = never,
+    // 2 = wherever the upright kernel applies)
+    const bool upright_ok = H % 2 == 0 && W % 2 == 0 && H >= 14;
+    const bool upright = upright_ok && (g_wgrad_strips == 2 || (g_wgrad_strips == 0 && W % (2 * WW_TILES) != 0));
+    a.rows_all = N * H;
+    a.sx = upright ? W / 2 : (W + 2 * WW_TILES - 1) / (2 * WW_TILES);
     a.sy = (H + 1) / 2;
-    const long strips = (long)N * a.sx * a.sy;
+    const long strips = upright ? (long)((a.rows_all + WW_VROWS - 1) / WW_VROWS) * a.sx : (long)N * a.sx * a.sy;
     PD_REQUIRE(strips <= 0x7ffffff0L, PD_ESHAPE, "%s: too many strips", who);
     a.n_strips = (int)strips;
     a.c_blocks = C / 64;
@@ -1424,7 +1522,8 @@ extern "C" int pd_conv3x3_winograd_wgrad_nhwc_f32(const float* x, const float* d
     float* du = a.part_db + (size_t)WW_BLOCKS * 128;
     float* dbsum = du + (size_t)WW_SUM_GROUPS * a.n_pairs * WW_PART_FLOATS;
     hipStream_t s = (hipStream_t)stream;
-    winograd_wgrad_kernel<<<WW_BLOCKS, WW_THREADS, 0, s>>>(a);
+    if (upright) winograd_wgrad_kernel<true><<<WW_BLOCKS, WW_THREADS, 0, s>>>(a);
+    else winograd_wgrad_kernel<false><<<WW_BLOCKS, WW_THREADS, 0, s>>>(a);
     PD_CHECK_LAUNCH(who);
     const long sum_threads = (long)a.n_pairs * (WW_PART_FLOATS / 4);
     winograd_wgrad_sum_kernel<<<dim3((unsigned)((sum_threads + 255) / 256), WW_SUM_GROUPS), 256, 0, s>>>(

@@ -510,6 +510,13 @@ def set_conv_pieces(mode):
     _cabi.lib().pd_conv3x3_winograd_set_pieces({"auto": 0, "always": 1, "never": -1}[mode])
 
 
+def set_conv_wgrad_strips(mode):
+    """Strips of the Winograd weight-gradient kernel: "auto" (upright strips of 16 rows x 2 columns of the stacked
+    batch where the width is no multiple of 16 pixels), "flat" (2 x 16 pixels always), "upright" (wherever the shape
+    allows).  The results differ by the summation order only."""
+    _cabi.lib().pd_conv3x3_winograd_set_wgrad_strips({"auto": 0, "flat": 1, "upright": 2}[mode])
+
+
 def _use_winograd(c, k, h, w):
     """Whether a convolution with c input and k output channels on h x w images takes the Winograd kernel:
     channel counts it supports, an image it can address with 32-bit offsets (the limits its entry point

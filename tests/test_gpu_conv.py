@@ -308,6 +308,48 @@ def test_winograd_weight_gradient_on_ragged_images(N, C, K, H, W, conv_algorithm
     torch.testing.assert_close(db.cpu().double(), bd.grad, rtol=1e-5, atol=4e-7 * math.sqrt(R) * 4)
 
 
+@pytest.fixture
+def _wgrad_strips_back_to_auto():
+    yield
+    ops.set_conv_wgrad_strips("auto")
+
+
+@pytest.mark.parametrize("N,C,K,H,W", [(3, 64, 64, 14, 14), (5, 64, 128, 14, 6), (2, 128, 64, 28, 28), (1, 64, 64, 56, 56),
+                                       (3, 64, 64, 18, 22), (2, 64, 64, 16, 32), (7, 64, 64, 14, 2), (1, 64, 256, 30, 46)])
+def test_winograd_weight_gradient_upright_strips(N, C, K, H, W, conv_algorithm, _wgrad_strips_back_to_auto):
+    """Strips of eight tiles on top of each other over the batch taken as one image of N * H rows: strips that
+    straddle two or three images (H = 14: every strip), a last strip row that is partly empty (N * H no multiple of
+    16), widths of one to 28 tile columns.  Weight and bias gradients against torch in fp64, and against the
+    flat strips of 2 x 16 pixels, from which they differ by the summation order only."""
+    if conv_algorithm != "winograd":
+        pytest.skip("covers the Winograd kernel")
+    g = torch.Generator().manual_seed(H * 100 + W)
+    x = torch.randn(N, C, H, W, generator=g)
+    dy = torch.randn(N, K, H, W, generator=g)
+    wd = torch.zeros(K, C, 3, 3, dtype=torch.float64, requires_grad=True)
+    bd = torch.zeros(K, dtype=torch.float64, requires_grad=True)
+    F.conv2d(x.double(), wd, bd, padding=1).backward(dy.double())
+    R = N * H * W
+    got = {}
+    for mode in ("upright", "flat"):
+        ops.set_conv_wgrad_strips(mode)
+        dw, db = ops.conv3x3_weight_grad(_nhwc(x), _nhwc(dy))
+        torch.testing.assert_close(dw.cpu().double(), wd.grad, rtol=1e-5, atol=4e-7 * math.sqrt(R) * 4)
+        torch.testing.assert_close(db.cpu().double(), bd.grad, rtol=1e-5, atol=4e-7 * math.sqrt(R) * 4)
+        got[mode] = dw
+    assert not torch.equal(got["upright"], got["flat"])       # the other kernel did run
+    # an image whose values are confined to its first and last rows: what a neighbour's rows would add shows up here
+    x2 = torch.zeros(N, C, H, W)
+    x2[:, :, 0] = torch.randn(N, C, W, generator=g)
+    x2[:, :, H - 1] = torch.randn(N, C, W, generator=g)
+    wd.grad = None
+    bd.grad = None
+    F.conv2d(x2.double(), wd, bd, padding=1).backward(dy.double())
+    ops.set_conv_wgrad_strips("upright")
+    dw, _ = ops.conv3x3_weight_grad(_nhwc(x2), _nhwc(dy))
+    torch.testing.assert_close(dw.cpu().double(), wd.grad, rtol=1e-5, atol=4e-7 * math.sqrt(R) * 4)
+
+
 def test_winograd_impulse_response_and_brute_force():
     # the Winograd path on shapes it accepts: (a) brute-force direct convolution of a small case with
     # random (asymmetric) filters; (b) a unit impulse must return the flipped filter taps around it
