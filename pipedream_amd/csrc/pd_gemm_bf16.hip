@@ -710,6 +710,20 @@ __global__ __launch_bounds__(256, (BM * BN <= 128 * 128 ? 2 : 1)) void pd_gemm_b
     c.b_step = TB::chunk_bytes(a.ldb);
     c.ring = ring;
     c.wave = wave;
+    const int nk = a.K / DK;       // a multiple of NS
+    // fill the ring: chunks 0 .. NS-1 into stages 0 .. NS-1
+#pragma unroll
+    for (int d = 0; d < IPT; ++d) G::template dma_unit<0>(c, d, 0);
+#pragma unroll
+    for (int d = 0; d < IPT; ++d) G::template dma_unit<1>(c, d, 1);
+#pragma unroll
+    for (int d = 0; d < IPT; ++d) G::template dma_unit<2>(c, d, 2);
+#pragma unroll
+    for (int d = 0; d < IPT; ++d) G::template dma_unit<3>(c, d, 3);
+    static_assert(NS == 4, "the ring fill and the unrolled loop below are written for 4 stages");
+    // The first chunks are on their way: everything the loads do not need is set up behind them (fragment
+    // addresses, cleared accumulators), inside the round trip to memory instead of in front of it.
+    __builtin_amdgcn_sched_barrier(0);
     const uint32_t ring_base = (uint32_t)(size_t)(lds_void_ptr)ring;
 #pragma unroll
     for (int s = 0; s < 2; ++s) {
@@ -727,17 +741,6 @@ __global__ __launch_bounds__(256, (BM * BN <= 128 * 128 ? 2 : 1)) void pd_gemm_b
 #pragma unroll
             for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.f;
 
-    const int nk = a.K / DK;       // a multiple of NS
-    // fill the ring: chunks 0 .. NS-1 into stages 0 .. NS-1
-#pragma unroll
-    for (int d = 0; d < IPT; ++d) G::template dma_unit<0>(c, d, 0);
-#pragma unroll
-    for (int d = 0; d < IPT; ++d) G::template dma_unit<1>(c, d, 1);
-#pragma unroll
-    for (int d = 0; d < IPT; ++d) G::template dma_unit<2>(c, d, 2);
-#pragma unroll
-    for (int d = 0; d < IPT; ++d) G::template dma_unit<3>(c, d, 3);
-    static_assert(NS == 4, "the ring fill and the unrolled loop below are written for 4 stages");
     wait_vmcnt<(NS - 1) * IPT>();      // chunk 0 has landed
     __builtin_amdgcn_s_barrier();
 
