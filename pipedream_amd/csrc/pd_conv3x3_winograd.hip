@@ -1504,7 +1504,8 @@ extern "C" int pd_conv3x3_winograd_wgrad_nhwc_f32(const float* x, const float* d
     a.N = N; a.H = H; a.W = W; a.C = C; a.K = K;
     // upright strips where strips of 2 x 16 pixels would pad the width (g_wgrad_strips: 0 = that rule, 1 = never,
     // 2 = wherever the upright kernel applies)
-    const bool upright_ok = H % 2 == 0 && W % 2 == 0 && H >= 14;
+    // (an upright strip's dY is addressed with 32-bit byte offsets over its 16 rows)
+    const bool upright_ok = H % 2 == 0 && W % 2 == 0 && H >= 14 && (long)WW_VROWS * W * K * 4 < (1L << 31);
     const bool upright = upright_ok && (g_wgrad_strips == 2 || (g_wgrad_strips == 0 && W % (2 * WW_TILES) != 0));
     a.rows_all = N * H;
     a.sx = upright ? W / 2 : (W + 2 * WW_TILES - 1) / (2 * WW_TILES);
