@@ -369,6 +369,17 @@ int pd_gemm_bf16(int trans_a, int trans_b, int M, int N, int K,
  * not thread-safe against concurrent GEMM calls.  No counterpart in the reference (its GEMMs are library calls). */
 int pd_gemm_bf16_set_tile(int bm, int bn);
 
+/* Operand preparation for an fp32 product computed on the bf16 matrix pipes (no counterpart in the reference,
+ * whose fp32 products are library calls).  x[rows][ld] (cols used) is written as six bf16 slots of three terms
+ * x1 = bf16(x), x2 = bf16(x - x1), x3 = bf16(x - x1 - x2) (x = x1 + x2 + x3 exactly): slots 1 3 2 2 1 1 for the
+ * A operand (b_side = 0), 3 1 1 2 2 1 for the B operand (b_side = 1).  stacked = 0: out[rows][6 cols], the slots
+ * side by side (an operand whose columns are the reduction index); stacked = 1: out[6 rows][cols], six row blocks
+ * (rows are the reduction index).  pd_gemm_bf16 over the six-fold reduction with fp32 output then adds
+ * a3 b1 + a1 b3 + a2 b1 + a2 b2 + a1 b2 + a1 b1: the fp32 product up to 2^-24 relative per term, with fp32
+ * accumulation.  cols and ld multiples of 4; x 16-byte, out 8-byte aligned. */
+int pd_split3_bf16_f32(const float* x, int64_t rows, int64_t cols, int64_t ld, uint16_t* out, int b_side,
+                       int stacked, void* stream);
+
 /* The same GEMM (unbatched, bf16 output) with the exact GELU of a feed-forward block in its epilogue.
  * backward = 0:  C = op(A) op(B) + bias  (the pre-activation, kept for the backward) and aux = gelu(C),
  *                with C taken as rounded to bf16, both written by the kernel;

@@ -106,6 +106,7 @@ SIGNATURES = {
     "pd_gemm_bf16": (_i, [_i, _i, _i, _i, _i, _vp, _i, _vp, _i, _vp, _i, _i, _f, _f, _vp, _vp, _i, _i, _i,
                           ctypes.POINTER(ctypes.c_int64), _vp], True),
     "pd_gemm_bf16_set_tile": (_i, [_i, _i], True),
+    "pd_split3_bf16_f32": (_i, [_vp, _i64, _i64, _i64, _vp, _i, _i, _vp], True),
     "pd_gemm_bf16_gelu": (_i, [_i, _i, _i, _i, _i, _i, _vp, _i, _vp, _i, _vp, _i, _vp, _vp, _i, _vp], True),
     "pd_layernorm_fwd_bf16": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _f, _vp], True),
     "pd_layernorm_bwd_partials": (_i, [_i], False),

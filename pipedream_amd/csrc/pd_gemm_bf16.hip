@@ -884,3 +884,72 @@ extern "C" int pd_gemm_bf16_gelu(int backward, int trans_a, int trans_b, int M, 
     return gemm_bf16_run(trans_a, trans_b, M, N, K, A, lda, B, ldb, C, ldc, 0, 1.0f, 0.0f, bias, nullptr, 0, 1, 1,
                          nullptr, stream, backward ? 2 : 1, backward ? nullptr : aux, backward ? aux : nullptr, ld_aux);
 }
+
+// ---------------------------------------------------------------------------------------
+// fp32 products on the bf16 matrix pipes.  An fp32 value is the exact sum of three bf16 values
+// (x1 = bf16(x), x2 = bf16(x - x1), x3 = bf16(x - x1 - x2): 3 x 8 significant bits), and a bf16 x bf16 product is
+// exact in fp32, so  a . b = a1 b1 + (a1 b2 + a2 b1) + (a2 b2 + a1 b3 + a3 b1) + terms below 2^-24 a b  needs six bf16
+// MFMAs where the fp32 MFMA needs one at a sixteenth of the rate -- and, unlike the fp32 MFMA, they run beside
+// vector instructions.  The six products are one bf16 GEMM over a reduction six times as long: this kernel writes
+// an operand's six slots -- A side: terms 1 3 2 2 1 1, B side: 3 1 1 2 2 1, small products first -- next to each
+// other along the reduction index (side by side in a row, or stacked as six row blocks for an operand whose rows
+// are the reduction index).
+namespace {
+
+__device__ __forceinline__ uint32_t split_rne(float f) {           // bf16 bits of f, round to nearest even
+    uint32_t u = __float_as_uint(f);
+    if ((u & 0x7fffffffu) > 0x7f800000u) return (u >> 16) | 0x0040u;
+    const uint32_t r = (u + 0x7fffu + ((u >> 16) & 1u)) >> 16;
+    // a finite value that would round to infinity keeps its leading bits instead (the remainder carries the rest)
+    return ((r & 0x7f80u) == 0x7f80u && (u & 0x7f800000u) != 0x7f800000u) ? (u >> 16) : r;
+}
+
+typedef uint16_t u16x4 __attribute__((ext_vector_type(4)));
+
+__global__ __launch_bounds__(256) void split3_bf16_kernel(const float* __restrict__ x, long long rows, int cols,
+                                                          long long ld, uint16_t* __restrict__ out, int b_side,
+                                                          int stacked) {
+    const int c4 = cols / 4;
+    const long long id = (long long)blockIdx.x * 256 + threadIdx.x;
+    if (id >= rows * c4) return;
+    const long long r = id / c4;
+    const int c = (int)(id % c4) * 4;
+    const float4_t v = *(const float4_t*)(x + r * ld + c);
+    u16x4 t[3];
+#pragma unroll
+    for (int k = 0; k < 4; ++k) {
+        float rem = v[k];
+#pragma unroll
+        for (int i = 0; i < 3; ++i) {
+            const uint32_t h = split_rne(rem);
+            t[i][k] = (uint16_t)h;
+            const float hf = __uint_as_float(h << 16);
+            // (an infinity or a NaN is carried by the first term alone)
+            rem = (h & 0x7f80u) == 0x7f80u ? 0.f : rem - hf;
+        }
+    }
+    const int a_terms[6] = {0, 2, 1, 1, 0, 0}, b_terms[6] = {2, 0, 0, 1, 1, 0};
+#pragma unroll
+    for (int s = 0; s < 6; ++s) {
+        const u16x4 val = t[b_side ? b_terms[s] : a_terms[s]];
+        uint16_t* dst = stacked ? out + ((long long)s * rows + r) * cols + c : out + r * (6ll * cols) + (long long)s * cols + c;
+        *(u16x4*)dst = val;
+    }
+}
+
+}  // namespace
+
+extern "C" int pd_split3_bf16_f32(const float* x, int64_t rows, int64_t cols, int64_t ld, uint16_t* out, int b_side,
+                                  int stacked, void* stream) {
+    PD_REQUIRE(rows >= 0 && cols >= 0 && cols % 4 == 0 && ld >= cols && ld % 4 == 0 && cols < (1ll << 30), PD_ESHAPE,
+               "pd_split3_bf16_f32: cols and ld must be multiples of 4, ld >= cols");
+    if (rows == 0 || cols == 0) return PD_OK;
+    PD_REQUIRE(x && out && pd_aligned(x, 16) && pd_aligned(out, 8), PD_EINVAL,
+               "pd_split3_bf16_f32: NULL or unaligned pointer");
+    const long long threads = rows * (cols / 4);
+    PD_REQUIRE((threads + 255) / 256 <= 0x7fffffffll, PD_ESHAPE, "pd_split3_bf16_f32: too large");
+    split3_bf16_kernel<<<dim3((unsigned)((threads + 255) / 256)), dim3(256), 0, (hipStream_t)stream>>>(
+        x, rows, (int)cols, ld, out, b_side != 0, stacked != 0);
+    PD_CHECK_LAUNCH("pd_split3_bf16_f32");
+    return PD_OK;
+}

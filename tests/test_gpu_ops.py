@@ -305,3 +305,89 @@ def test_gemm_tile_rows_left_over_after_whole_rounds_are_split_over_k(ta, tb, M,
         assert torch.equal(outs[0][:rows], outs[1][:rows])
     torch.testing.assert_close(outs[0], outs[1], rtol=1e-5, atol=1e-5 * K ** 0.5)    # sums of K terms of size ~1
     assert not torch.equal(outs[0][rows:], outs[1][rows:])    # the tail did take the other path
+
+
+@pytest.fixture
+def _gemm_algorithm_back_to_auto():
+    from pipedream_amd import ops
+    yield
+    ops.set_gemm_f32_algorithm("auto")
+
+
+@pytest.mark.parametrize("ta,tb", [(False, True), (False, False), (True, False)])
+def test_gemm_as_six_bf16_products_is_closer_to_fp64_than_the_fp32_kernel(ta, tb, _gemm_algorithm_back_to_auto):
+    """Large fp32 products run on the bf16 matrix pipes: each operand as the exact sum of three bf16 terms, six
+    products per term pair, fp32 accumulation.  Against torch's fp64 product the result must be at least as close
+    as the fp32 MFMA kernel's (it is about three times closer: fewer roundings of the running sum), with bias and
+    beta applied; the default takes that path for this shape and not for a narrow or a small one."""
+    from pipedream_amd import ops
+    M, N, K = 4096, 3072, 1408
+    assert ops._use_split_bf16(M, N, K, ta, tb, False, *(torch.empty(8, 8, device="cuda"),) * 3)
+    assert ops._split_bf16_parts(6400, 1024, 4096) == 2 and ops._split_bf16_parts(4096, 1024, 6400) == 4
+    assert ops._split_bf16_parts(M, N, K) == 1 and ops._split_bf16_parts(512, 512, 4096) == 6
+    assert not ops._use_split_bf16(6400, 1024, 4096, ta, tb, False, *(torch.empty(8, 8, device="cuda"),) * 3)
+    assert not ops._use_split_bf16(1024, 1024, 1024, ta, tb, False, *(torch.empty(8, 8, device="cuda"),) * 3)
+    assert not ops._use_split_bf16(M, N, K, ta, tb, True, *(torch.empty(8, 8, device="cuda"),) * 3)     # ReLU epilogue
+    g = torch.Generator().manual_seed(21)
+    a = torch.randn((K, M) if ta else (M, K), generator=g).cuda()
+    b = (torch.randn((N, K) if tb else (K, N), generator=g) * 0.05).cuda()
+    bias = torch.randn(N, generator=g).cuda()
+    prior = torch.randn(M, N, generator=g).cuda()
+    want = (a.double().t() if ta else a.double()) @ (b.double().t() if tb else b.double()) + bias.double() + 0.5 * prior.double()
+    err = {}
+    for mode in ("mfma_f32", "split_bf16", "auto"):
+        ops.set_gemm_f32_algorithm(mode)
+        out = ops.gemm(a, b, trans_a=ta, trans_b=tb, bias=bias, out=prior.clone(), beta=0.5)
+        err[mode] = (float((out.double() - want).norm() / want.norm()), float((out.double() - want).abs().max()), out)
+    assert err["split_bf16"][0] <= err["mfma_f32"][0] and err["split_bf16"][1] <= 1.5 * err["mfma_f32"][1], err
+    assert err["split_bf16"][0] < 4e-7
+    assert torch.equal(err["auto"][2], err["split_bf16"][2])
+
+
+@pytest.mark.parametrize("ta,tb", [(False, True), (False, False), (True, False)])
+def test_gemm_as_six_bf16_products_with_few_output_tiles(ta, tb, _gemm_algorithm_back_to_auto):
+    """A narrow output (1024 columns: 28 tiles of 256 x 256): the six-fold reduction is cut into ranges that run as
+    batch entries, and their partial products are added in index order with bias and beta."""
+    from pipedream_amd import ops
+    M, N, K = 1792, 1024, 1536
+    assert ops._split_bf16_parts(M, N, K) == 6
+    g = torch.Generator().manual_seed(22)
+    a = torch.randn((K, M) if ta else (M, K), generator=g).cuda()
+    b = (torch.randn((N, K) if tb else (K, N), generator=g) * 0.05).cuda()
+    bias = torch.randn(N, generator=g).cuda()
+    prior = torch.randn(M, N, generator=g).cuda()
+    want = (a.double().t() if ta else a.double()) @ (b.double().t() if tb else b.double()) + bias.double() + 0.5 * prior.double()
+    err = {}
+    for mode in ("mfma_f32", "split_bf16"):
+        ops.set_gemm_f32_algorithm(mode)
+        out = ops.gemm(a, b, trans_a=ta, trans_b=tb, bias=bias, out=prior.clone(), beta=0.5)
+        err[mode] = float((out.double() - want).norm() / want.norm())
+    assert err["split_bf16"] <= err["mfma_f32"] and err["split_bf16"] < 4e-7, err
+
+
+def test_three_way_bf16_split_is_exact_and_keeps_special_values():
+    """pd_split3_bf16_f32: the three terms add up to the fp32 value exactly (normal numbers), slot order per side,
+    both placements; infinities and NaNs stay in the first term, a value that bf16 would round to infinity does not."""
+    from pipedream_amd import _cabi, ops
+    g = torch.Generator().manual_seed(3)
+    x = torch.randn(64, 128, generator=g) * torch.exp2(torch.randint(-60, 60, (64, 128), generator=g).float())
+    x[0, :8] = torch.tensor([float("inf"), float("-inf"), float("nan"), 3.4e38, -3.4e38, 0.0, -0.0, 1.0])
+    x = x.cuda()
+    lib = _cabi.lib()
+    for b_side, slots in ((0, (0, 2, 1, 1, 0, 0)), (1, (2, 0, 0, 1, 1, 0))):
+        flat = torch.empty(64, 6 * 128, dtype=torch.bfloat16, device="cuda")
+        tall = torch.empty(6 * 64, 128, dtype=torch.bfloat16, device="cuda")
+        lib.pd_split3_bf16_f32(ops._ptr(x), 64, 128, 128, ops._ptr(flat), b_side, 0, _cabi.stream_ptr())
+        lib.pd_split3_bf16_f32(ops._ptr(x), 64, 128, 128, ops._ptr(tall), b_side, 1, _cabi.stream_ptr())
+        parts = [flat[:, s * 128:(s + 1) * 128] for s in range(6)]
+        bits = lambda t: t.contiguous().view(torch.int16)      # (NaN is not equal to itself)
+        for s in range(6):
+            assert torch.equal(bits(parts[s]), bits(tall[s * 64:(s + 1) * 64]))
+            assert torch.equal(bits(parts[s]), bits(parts[slots.index(slots[s])]))       # equal terms are equal slots
+        t = [parts[slots.index(i)].float() for i in range(3)]
+        total = (t[0].double() + t[1].double() + t[2].double()).float()
+        ok = torch.isfinite(x)
+        assert torch.equal(total[ok], x[ok])
+        assert torch.isinf(t[0][0, 0]) and torch.isinf(t[0][0, 1]) and torch.isnan(t[0][0, 2])
+        assert float(t[1][0, :3].abs().sum()) == 0.0 and float(t[2][0, :3].abs().sum()) == 0.0
+        assert torch.isfinite(t[0][0, 3]) and torch.isfinite(t[0][0, 4])
